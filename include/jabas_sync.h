@@ -1,0 +1,222 @@
+/*
+ * jabas_sync.h -- C ABI of libjabas_sync.so: the per-GPU gradient synchronisation
+ * step of IIDP/JABAS on one MI355X (gfx950).
+ *
+ * One call covers, in a single pass over HBM:
+ *   (1) the batch-weighted aggregate of the K virtual-stream-worker (VSW) gradient
+ *       buckets,      acc = g_0*w_0; acc = acc + g_k*w_k  (k = 1..K-1),
+ *       every product and sum individually rounded to fp32, bf16 inputs widened first;
+ *   (2) the per-span gradient statistics used by similarity-based adaptive batching;
+ *   (3) the weight update (SGD-momentum, Adam, AdamW) over the flat parameter span,
+ *       optionally followed by the fan-out of the new weights to other VSW replicas.
+ *
+ * Conventions
+ *   - plain C types only; every buffer is caller-owned device memory;
+ *   - no entry point allocates, frees or synchronises the device; all work is queued
+ *     on the stream passed in (jabas_stream_t is a hipStream_t);
+ *   - the library keeps no mutable global state besides cached device attributes, so
+ *     calls from different threads on different streams do not interfere as long as
+ *     they use different workspaces;
+ *   - return value: JABAS_OK (0) or a negative JabasStatus; nothing is launched when a
+ *     negative status is returned (except JABAS_ERR_LAUNCH, reported after the fact).
+ *
+ * What each entry point stands in for in the reference is cited beside it
+ * (paths relative to the JABAS repository).
+ */
+#ifndef JABAS_SYNC_H
+#define JABAS_SYNC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JABAS_MAX_K 8           /* VSWs aggregated by one launch                      */
+#define JABAS_MAX_GROUPS 16     /* optimizer parameter groups per launch              */
+#define JABAS_STATS_STRIDE 12   /* doubles per span in stats_out: 4 + JABAS_MAX_K     */
+#define JABAS_GRAM_STRIDE 64    /* doubles per call in gram_out: JABAS_MAX_K squared  */
+
+typedef void* jabas_stream_t;   /* hipStream_t */
+
+typedef enum JabasStatus {
+    JABAS_OK = 0,
+    JABAS_ERR_NULL = -1,        /* a required pointer is NULL                          */
+    JABAS_ERR_K = -2,           /* K outside 1..JABAS_MAX_K                            */
+    JABAS_ERR_ALIGN = -3,       /* buffers of a span are not mutually 16-byte congruent*/
+    JABAS_ERR_DTYPE = -4,       /* grad_dtype is neither JABAS_F32 nor JABAS_BF16      */
+    JABAS_ERR_OPT = -5,         /* unknown optimizer kind or inconsistent state ptrs   */
+    JABAS_ERR_GROUP = -6,       /* group index / count out of range, unsorted bounds   */
+    JABAS_ERR_WORKSPACE = -7,   /* workspace missing or too small                      */
+    JABAS_ERR_PLAN = -8,        /* plan blob malformed or too small                    */
+    JABAS_ERR_SIZE = -9,        /* numel / span count out of range                     */
+    JABAS_ERR_LAUNCH = -10,     /* the HIP runtime refused the launch                  */
+    JABAS_ERR_ALIAS = -11       /* agg_out aliases a gradient buffer that is not fp32  */
+} JabasStatus;
+
+enum { JABAS_F32 = 0, JABAS_BF16 = 1 };
+enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAMW = 3 };
+
+/* Slots of one stats_out row (JABAS_STATS_STRIDE doubles per span). A = VSWs with
+ * half_id 0, B = VSWs with half_id 1; g_A = sum_{k in A} g_k*half_weight_k formed in
+ * fp32 in increasing k (same rounding rule as the aggregate), g_B likewise. Products
+ * and sums of the statistics themselves are fp64. */
+enum {
+    JABAS_STAT_DOT_AB = 0,      /* sum g_A * g_B                                       */
+    JABAS_STAT_NORM_A = 1,      /* sum g_A^2                                           */
+    JABAS_STAT_NORM_B = 2,      /* sum g_B^2                                           */
+    JABAS_STAT_NORM_AGG = 3,    /* sum gbar^2 of the aggregate                         */
+    JABAS_STAT_NORM_VSW0 = 4    /* + k: sum g_k^2 of VSW k                             */
+};
+
+/* One contiguous stretch of the flat layout. All buffers hold `numel` elements and are
+ * indexed alike. Their addresses must be congruent modulo 16 bytes in element terms
+ * (element e of every buffer falls at the same position of a 16-byte line), which holds
+ * whenever they are views at one element offset into 16-byte aligned arenas.
+ * agg_out may alias grads[0] when the gradients are fp32 (in-place bucket update).
+ * Unused pointers are NULL. */
+typedef struct JabasSpan {
+    const void* grads[JABAS_MAX_K];     /* K gradient buffers (fp32 or bf16)           */
+    float*      agg_out;                /* aggregated fp32 gradient, or NULL           */
+    float*      param;                  /* fp32 weights (optimizer kinds other than NONE) */
+    float*      state1;                 /* SGD momentum buffer / Adam exp_avg          */
+    float*      state2;                 /* Adam exp_avg_sq                             */
+    float*      fanout[JABAS_MAX_K - 1];/* replicas that receive the updated weights   */
+    uint64_t    numel;
+    uint32_t    n_fanout;
+    uint32_t    bound_begin;            /* first entry of this span in the bounds table*/
+    uint32_t    bound_count;            /* 0: the whole span is parameter group 0      */
+    uint32_t    reserved;
+} JabasSpan;
+
+/* Parameter-group change inside a span: elements [start, next start) use `group`.
+ * The first bound of a span has start 0; starts are strictly increasing. */
+typedef struct JabasBound {
+    uint64_t start;
+    uint32_t group;
+    uint32_t reserved;
+} JabasBound;
+
+/* Hyper-parameters of one parameter group, as the Python optimizer holds them
+ * (doubles). `step` is the 1-based Adam step count of this call. */
+typedef struct JabasGroup {
+    double  lr;
+    double  weight_decay;
+    int64_t step;
+} JabasGroup;
+
+typedef struct JabasStepArgs {
+    int32_t K;
+    int32_t grad_dtype;                 /* JABAS_F32 / JABAS_BF16                      */
+    float   weight[JABAS_MAX_K];        /* w_k = fp32(b_k / B)                         */
+    int32_t stats;                      /* 0: none, 1: write a stats_out row per span  */
+    uint8_t half_id[JABAS_MAX_K];       /* 0 = half A, 1 = half B                      */
+    float   half_weight[JABAS_MAX_K];   /* fp32(b_k / sum of b over k's half)          */
+    int32_t opt_kind;                   /* JABAS_OPT_*                                 */
+    int32_t n_groups;
+    int32_t first_step;                 /* SGD: momentum buffer not initialised yet    */
+    int32_t nesterov;
+    double  momentum, dampening;        /* SGD                                         */
+    double  beta1, beta2, eps;          /* Adam / AdamW                                */
+    JabasGroup groups[JABAS_MAX_GROUPS];
+} JabasStepArgs;
+
+/* Library identification. No reference counterpart. */
+const char* jabas_sync_version(void);
+const char* jabas_status_string(int status);
+
+/* Bytes of device workspace a fused or statistics call over n_span spans needs
+ * (per-block partial sums of the two-level reduction). */
+size_t jabas_sync_workspace_bytes(uint32_t n_span);
+
+/* --- multi-span plan --------------------------------------------------------------
+ * A plan is the launch-invariant description of a set of spans (pointer table, tile
+ * prefix sums, group bounds). jabas_plan_encode validates the spans and writes the
+ * blob into host memory; the caller copies the same bytes to the device once and
+ * passes both copies to jabas_sync_fused at every step. Pure host code: runs without
+ * a GPU.
+ * Stands in for the per-tensor Python loops that walk buckets and parameters at every
+ * step in the reference: jabas/train/trainer.py:327-337 (hook registration per local
+ * model), examples/gnmt/seq2seq/train/shard_optimizer.py:40-73 (per-parameter loop
+ * matching gradients to parameters by .index). */
+size_t jabas_plan_bytes(uint32_t n_span, uint32_t n_bounds);
+int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span,
+                      const JabasBound* bounds, uint32_t n_bounds,
+                      int32_t K, int32_t grad_dtype, int32_t opt_kind,
+                      void* host_blob, size_t blob_bytes);
+/* Number of 16-byte-line tiles the plan covers (grid sizing, diagnostics). */
+int64_t jabas_plan_tiles(const void* host_blob);
+
+/* --- the fused sync step ------------------------------------------------------------
+ * Aggregate + statistics + optimizer (+ fan-out) over every span of a plan, one
+ * launch (plus a one-block-per-span finalize launch when args->stats is set).
+ * stats_out: n_span * JABAS_STATS_STRIDE doubles (device), required when stats != 0.
+ * Replaces, for one GPU:
+ *   - the local aggregation of the K VSW buckets inside IIDPTrainer.compute()/step()
+ *     and iidp_allreduce_hook's division by the worker count
+ *     (call sites jabas/ddp_comm_hooks/similarity_allreduce.py:42,
+ *      jabas/train/trainer.py:452-468, 594-599);
+ *   - clone + sub-group sum + div_ of subgroup_allreduce_hook
+ *     (jabas/ddp_comm_hooks/similarity_allreduce.py:20-35) and the cat + reductions of
+ *     _compute_cosine_similarity (jabas/train/trainer.py:470-483);
+ *   - torch.optim.SGD / Adam / AdamW and iidp.optim.ShardSGD / ShardAdam / ShardAdamW
+ *     .step() (examples/resnet50/main.py:351-359, examples/vit/main.py:425-437,
+ *      examples/gnmt/seq2seq/train/shard_optimizer.py:30-90);
+ *   - the weight copy main VSW -> other VSWs (jabas/train/trainer.py:530-534). */
+int jabas_sync_fused(const void* plan_host, const void* plan_dev,
+                     const JabasStepArgs* args, double* stats_out,
+                     void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* The same step over ONE span passed by value (no plan, no device table): what a
+ * comm hook calls for the bucket it was handed. bounds_dev is a device array of
+ * span->bound_count entries starting at span->bound_begin, or NULL when
+ * bound_count == 0. stats_out: JABAS_STATS_STRIDE doubles or NULL.
+ * Replaces hook_with_allreduce for one bucket
+ * (jabas/ddp_comm_hooks/similarity_allreduce.py:38-45) and, with an optimizer kind,
+ * the optimizer hook of the overlap weight-sync mode (jabas/train/trainer.py:327-333). */
+int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev,
+                      const JabasStepArgs* args, double* stats_out,
+                      void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* --- single-purpose entry points (thin fronts over the same kernels) ---------------- */
+
+/* out = sum_k w_k g_k in the canonical order. out may alias grads[0] (fp32).
+ * Local VSW aggregation only (jabas/train/trainer.py:452-468, 594-599). */
+int jabas_aggregate(const void* const* grads, int32_t K, int32_t grad_dtype,
+                    const float* weight, float* out, uint64_t numel,
+                    jabas_stream_t stream);
+
+/* Statistics row of one span without touching any output buffer
+ * (jabas/ddp_comm_hooks/similarity_allreduce.py:20-35, jabas/train/trainer.py:470-483). */
+int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype,
+                const float* weight, const uint8_t* half_id, const float* half_weight,
+                uint64_t numel, double* stats_out,
+                void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* K x K Gram matrix of the worker gradients, gram_out[a*JABAS_MAX_K + b] = sum g_a*g_b
+ * (fp64 products and sums), symmetric, JABAS_GRAM_STRIDE doubles. The "between
+ * workers" statistics; no reference counterpart beyond the pairwise cosine of
+ * jabas/train/trainer.py:478. */
+int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype,
+               uint64_t numel, double* gram_out,
+               void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* SGD step with a ready fp32 gradient (torch 1.8.1 optim/_functional.sgd as used by
+ * examples/resnet50/main.py:351-359, examples/faster_r_cnn/train.py:266-276).
+ * momentum_buf may be NULL when momentum == 0. */
+int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t numel,
+              double lr, double weight_decay, double momentum, double dampening,
+              int32_t nesterov, int32_t first_step, jabas_stream_t stream);
+
+/* Adam (adamw == 0) / AdamW (adamw != 0) step with a ready fp32 gradient
+ * (torch 1.8.1 optim/_functional.adam / adamw as called by
+ * examples/gnmt/seq2seq/train/shard_optimizer.py:78-90, examples/vit/main.py:425-437). */
+int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq,
+               uint64_t numel, double lr, double weight_decay, double beta1, double beta2,
+               double eps, int64_t step, int32_t adamw, jabas_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* JABAS_SYNC_H */

@@ -1,0 +1,535 @@
+// C ABI of libjabas_sync.so: argument validation, plan encoding, derivation of the fp32
+// kernel constants, grid sizing, and the finalize kernel of the two-level statistics
+// reduction. The streaming kernels themselves live in fused_kernel.hip / gram_kernel.hip.
+#include <math.h>
+#include <string.h>
+
+#include "jabas_internal.h"
+
+#define JABAS_API extern "C" __attribute__((visibility("default")))
+
+namespace jabas {
+
+int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream);
+int launch_gram_finalize(int K, const double* partials, unsigned grid, double* gram_out, hipStream_t stream);
+
+namespace {
+
+constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
+constexpr uint32_t kPlanVersion = 1;
+
+struct PlanHeader {
+    uint32_t magic, version;
+    uint32_t n_span, n_bounds, n_tiles;
+    int32_t K, grad_dtype, opt_kind;
+    uint32_t max_group;       // largest group index any bound names
+    uint32_t all_have_s1;     // every span carries a state1 pointer
+    uint64_t off_spans, off_prefix, off_bounds, total_bytes;
+};
+static_assert(sizeof(PlanHeader) == 72, "plan header layout");
+constexpr size_t kHeaderBytes = 80;
+
+inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
+
+inline int opt_class_of(int kind) {
+    switch (kind) {
+        case JABAS_OPT_NONE: return 0;
+        case JABAS_OPT_SGD: return 1;
+        case JABAS_OPT_ADAM:
+        case JABAS_OPT_ADAMW: return 2;
+        default: return -1;
+    }
+}
+
+inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    return a0 < b0 + nb && b0 < a0 + na;
+}
+
+// Validates one span and produces the rebased device view. Host-only logic.
+int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDev* out, uint32_t* tiles) {
+    const int gs = grad_dtype == JABAS_BF16 ? 2 : 4;
+    const int ept = ept_of(grad_dtype);
+    if (in.numel > (static_cast<uint64_t>(1) << 40)) return JABAS_ERR_SIZE;
+    if (in.n_fanout > JABAS_MAX_K - 1) return JABAS_ERR_SIZE;
+    if (in.numel == 0) {                       // empty span: nothing to read, pointers may be NULL
+        memset(out, 0, sizeof(*out));
+        *tiles = 0;
+        return JABAS_OK;
+    }
+    for (int k = 0; k < K; ++k)
+        if (!in.grads[k]) return JABAS_ERR_NULL;
+    const int oc = opt_class_of(opt_kind);
+    if (oc < 0) return JABAS_ERR_OPT;
+    if (oc != 0 && !in.param) return JABAS_ERR_NULL;
+    if (oc == 2 && (!in.state1 || !in.state2)) return JABAS_ERR_NULL;
+    if (oc == 0 && in.n_fanout) return JABAS_ERR_OPT;
+    for (uint32_t r = 0; r < in.n_fanout; ++r)
+        if (!in.fanout[r]) return JABAS_ERR_NULL;
+
+    const uintptr_t g0 = reinterpret_cast<uintptr_t>(in.grads[0]);
+    if (g0 % gs) return JABAS_ERR_ALIGN;
+    const uint32_t skew = static_cast<uint32_t>((g0 / gs) % ept);   // elements before a 16-byte line start
+    auto rebase_g = [&](const void* p, const void** dst) -> bool {
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        if (a % gs || (a / gs) % ept != skew) return false;
+        *dst = reinterpret_cast<const void*>(a - static_cast<uintptr_t>(skew) * gs);
+        return true;
+    };
+    auto rebase_f = [&](float* p, float** dst) -> bool {
+        if (!p) { *dst = nullptr; return true; }
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        if (a % 4 || (a / 4) % 4 != skew % 4) return false;
+        *dst = reinterpret_cast<float*>(a - static_cast<uintptr_t>(skew) * 4);
+        return true;
+    };
+    memset(out, 0, sizeof(*out));
+    for (int k = 0; k < K; ++k)
+        if (!rebase_g(in.grads[k], &out->g[k])) return JABAS_ERR_ALIGN;
+    if (!rebase_f(in.agg_out, &out->out)) return JABAS_ERR_ALIGN;
+    if (oc != 0) {
+        if (!rebase_f(in.param, &out->p) || !rebase_f(in.state1, &out->s1) || !rebase_f(in.state2, &out->s2))
+            return JABAS_ERR_ALIGN;
+        for (uint32_t r = 0; r < in.n_fanout; ++r)
+            if (!rebase_f(in.fanout[r], &out->fan[r])) return JABAS_ERR_ALIGN;
+        out->n_fan = in.n_fanout;
+    }
+    if (in.agg_out) {
+        const size_t ob = in.numel * 4;
+        for (int k = 0; k < K; ++k) {
+            if (!ranges_overlap(in.agg_out, ob, in.grads[k], in.numel * gs)) continue;
+            if (grad_dtype != JABAS_F32 || static_cast<const void*>(in.agg_out) != in.grads[k]) return JABAS_ERR_ALIAS;
+        }
+    }
+    out->lo = skew;
+    out->hi = skew + in.numel;
+    out->bound_begin = in.bound_begin;
+    out->bound_count = in.bound_count;
+    const uint64_t te = tile_elems(grad_dtype);
+    const uint64_t nt = in.numel ? (out->hi + te - 1) / te : 0;
+    if (nt > 0x7fffffffull) return JABAS_ERR_SIZE;
+    *tiles = static_cast<uint32_t>(nt);
+    return JABAS_OK;
+}
+
+int check_bounds_host(const JabasSpan& sp, const JabasBound* bounds, uint32_t n_bounds, uint32_t* max_group) {
+    if (sp.bound_count == 0) return JABAS_OK;
+    if (!bounds) return JABAS_ERR_NULL;
+    if (static_cast<uint64_t>(sp.bound_begin) + sp.bound_count > n_bounds) return JABAS_ERR_GROUP;
+    const JabasBound* b = bounds + sp.bound_begin;
+    if (b[0].start != 0) return JABAS_ERR_GROUP;
+    for (uint32_t i = 0; i < sp.bound_count; ++i) {
+        if (b[i].group >= JABAS_MAX_GROUPS) return JABAS_ERR_GROUP;
+        if (i && b[i].start <= b[i - 1].start) return JABAS_ERR_GROUP;
+        if (sp.numel && b[i].start >= sp.numel && i) return JABAS_ERR_GROUP;
+        if (b[i].group > *max_group) *max_group = b[i].group;
+    }
+    return JABAS_OK;
+}
+
+// StepArgs (doubles, as the Python optimizer holds them) -> fp32 kernel constants.
+int fill_kargs(const JabasStepArgs* s, KArgs* a) {
+    if (!s) return JABAS_ERR_NULL;
+    if (s->K < 1 || s->K > JABAS_MAX_K) return JABAS_ERR_K;
+    if (s->grad_dtype != JABAS_F32 && s->grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
+    const int oc = opt_class_of(s->opt_kind);
+    if (oc < 0) return JABAS_ERR_OPT;
+    memset(a, 0, sizeof(*a));
+    uint32_t mask = 0;
+    for (int k = 0; k < s->K; ++k) {
+        a->w[k] = s->weight[k];
+        a->wh[k] = s->half_weight[k];
+        if (s->half_id[k] > 1) return JABAS_ERR_K;
+        if (s->half_id[k]) mask |= 1u << k;
+    }
+    a->half_mask = mask;
+    if (oc == 0) return JABAS_OK;
+    if (s->n_groups < 1 || s->n_groups > JABAS_MAX_GROUPS) return JABAS_ERR_GROUP;
+    OptDev& o = a->opt;
+    o.momentum = static_cast<float>(s->momentum);
+    o.one_minus_damp = static_cast<float>(1.0 - s->dampening);
+    o.beta1 = static_cast<float>(s->beta1);
+    o.one_minus_beta1 = static_cast<float>(1.0 - s->beta1);
+    o.beta2 = static_cast<float>(s->beta2);
+    o.one_minus_beta2 = static_cast<float>(1.0 - s->beta2);
+    o.eps = static_cast<float>(s->eps);
+    o.has_momentum = (oc == 1 && s->momentum != 0.0) ? 1 : 0;
+    o.first_step = s->first_step ? 1 : 0;
+    o.nesterov = s->nesterov ? 1 : 0;
+    o.adamw = s->opt_kind == JABAS_OPT_ADAMW ? 1 : 0;
+    if (oc == 1 && o.nesterov && (s->momentum <= 0.0 || s->dampening != 0.0)) return JABAS_ERR_OPT;
+    for (int i = 0; i < s->n_groups; ++i) {
+        const JabasGroup& g = s->groups[i];
+        GroupDev& d = a->groups[i];
+        d.wd = static_cast<float>(g.weight_decay);
+        d.neg_lr = static_cast<float>(-g.lr);
+        d.decay = static_cast<float>(1.0 - g.lr * g.weight_decay);
+        d.neg_step_size = 0.0f;
+        d.sqrt_bc2 = 1.0f;
+        if (oc == 2) {
+            if (g.step < 1) return JABAS_ERR_OPT;
+            const double bc1 = 1.0 - pow(s->beta1, static_cast<double>(g.step));
+            const double bc2 = 1.0 - pow(s->beta2, static_cast<double>(g.step));
+            d.neg_step_size = static_cast<float>(-(g.lr / bc1));
+            d.sqrt_bc2 = static_cast<float>(sqrt(bc2));
+        }
+    }
+    return JABAS_OK;
+}
+
+int cu_count() {
+    static int cache[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cache[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        cache[dev] = n;
+    }
+    return cache[dev];
+}
+
+typedef int (*LaunchFn)(int, int, int, const KArgs&, unsigned, hipStream_t);
+typedef int (*OccFn)(int, int, int);
+const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_fused_k3, launch_fused_k4,
+                                       launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
+const OccFn kOcc[JABAS_MAX_K] = {occupancy_k1, occupancy_k2, occupancy_k3, occupancy_k4,
+                                 occupancy_k5, occupancy_k6, occupancy_k7, occupancy_k8};
+
+unsigned pick_grid(int K, int grad_dtype, int oc, int stats, uint32_t n_tiles) {
+    const int occ = kOcc[K - 1](grad_dtype, oc, stats);
+    uint64_t g = static_cast<uint64_t>(cu_count()) * static_cast<uint64_t>(occ);
+    if (g > static_cast<uint64_t>(kMaxGrid)) g = kMaxGrid;
+    if (g > n_tiles) g = n_tiles;
+    if (g < 1) g = 1;
+    return static_cast<unsigned>(g);
+}
+
+// Second level of the statistics reduction: one wave per span sums, in increasing
+// workgroup order, the partial rows the workgroups that touched the span left behind.
+__global__ void __launch_bounds__(64) finalize_stats_kernel(const uint32_t* tile_prefix, uint32_t n_tiles,
+                                                            uint32_t use_inline, uint32_t grid, int ns,
+                                                            const double* partials, double* stats_out) {
+    const uint32_t s = blockIdx.x, lane = threadIdx.x;
+    uint32_t ts0 = 0, ts1 = n_tiles;
+    if (!use_inline) { ts0 = tile_prefix[s]; ts1 = tile_prefix[s + 1]; }
+    double acc[kStatsStride];
+#pragma unroll
+    for (int i = 0; i < kStatsStride; ++i) acc[i] = 0.0;
+    if (ts1 > ts0) {
+        // workgroup b owns tiles [b*T/G, (b+1)*T/G): owner(t) = ((t+1)*G - 1) / T
+        const uint64_t T = n_tiles, G = grid;
+        const uint32_t b_lo = static_cast<uint32_t>(((static_cast<uint64_t>(ts0) + 1) * G - 1) / T);
+        const uint32_t b_hi = static_cast<uint32_t>((static_cast<uint64_t>(ts1) * G - 1) / T);
+        for (uint32_t b = b_lo + lane; b <= b_hi; b += 64) {
+            const double* row = partials + static_cast<uint64_t>(b + s) * kStatsStride;
+#pragma unroll
+            for (int i = 0; i < kStatsStride; ++i)
+                if (i < ns) acc[i] += row[i];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kStatsStride; ++i) {
+        double v = acc[i];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+        acc[i] = v;
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < kStatsStride; ++i) stats_out[static_cast<uint64_t>(s) * kStatsStride + i] = acc[i];
+    }
+}
+
+int run_fused(KArgs& a, const JabasStepArgs* s, double* stats_out, void* workspace, size_t workspace_bytes,
+              hipStream_t stream) {
+    const int oc = opt_class_of(s->opt_kind);
+    const int stats = s->stats ? 1 : 0;
+    if (stats) {
+        if (!stats_out) return JABAS_ERR_NULL;
+        if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
+        if (workspace_bytes < jabas_sync_workspace_bytes(a.n_span)) return JABAS_ERR_WORKSPACE;
+        if (reinterpret_cast<uintptr_t>(stats_out) % 8) return JABAS_ERR_ALIGN;
+    }
+    a.partials = static_cast<double*>(workspace);
+    unsigned grid = 0;
+    if (a.n_tiles) {
+        grid = pick_grid(s->K, s->grad_dtype, oc, stats, a.n_tiles);
+        const int err = kLaunch[s->K - 1](s->grad_dtype, oc, stats, a, grid, stream);
+        if (err != 0) return JABAS_ERR_LAUNCH;
+    }
+    if (stats) {
+        hipLaunchKernelGGL(finalize_stats_kernel, dim3(a.n_span), dim3(64), 0, stream, a.tile_prefix, a.n_tiles,
+                           a.use_inline, grid ? grid : 1u, 4 + s->K, a.partials, stats_out);
+        if (hipGetLastError() != hipSuccess) return JABAS_ERR_LAUNCH;
+    }
+    return JABAS_OK;
+}
+
+}  // namespace
+}  // namespace jabas
+
+using namespace jabas;
+
+JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.1 (gfx950)"; }
+
+JABAS_API const char* jabas_status_string(int status) {
+    switch (status) {
+        case JABAS_OK: return "ok";
+        case JABAS_ERR_NULL: return "a required pointer is NULL";
+        case JABAS_ERR_K: return "K outside 1..8 or half_id not 0/1";
+        case JABAS_ERR_ALIGN: return "buffers of a span are not mutually congruent modulo 16 bytes";
+        case JABAS_ERR_DTYPE: return "unsupported gradient dtype";
+        case JABAS_ERR_OPT: return "unknown optimizer kind or inconsistent optimizer arguments";
+        case JABAS_ERR_GROUP: return "parameter group index/count out of range or bounds not sorted";
+        case JABAS_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case JABAS_ERR_PLAN: return "plan blob malformed, too small or not matching the step arguments";
+        case JABAS_ERR_SIZE: return "element, span or fan-out count out of range";
+        case JABAS_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
+        case JABAS_ERR_ALIAS: return "agg_out overlaps a gradient buffer other than exactly in place (fp32)";
+        default: return "unknown status";
+    }
+}
+
+JABAS_API size_t jabas_sync_workspace_bytes(uint32_t n_span) {
+    return (static_cast<size_t>(kMaxGrid) + n_span) * kStatsStride * sizeof(double);
+}
+
+JABAS_API size_t jabas_plan_bytes(uint32_t n_span, uint32_t n_bounds) {
+    return kHeaderBytes + align16(static_cast<size_t>(n_span) * sizeof(SpanDev)) +
+           align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t)) +
+           align16(static_cast<size_t>(n_bounds) * sizeof(BoundDev));
+}
+
+JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
+                                uint32_t n_bounds, int32_t K, int32_t grad_dtype, int32_t opt_kind,
+                                void* host_blob, size_t blob_bytes) {
+    static_assert(sizeof(BoundDev) == sizeof(JabasBound), "bound layout");
+    if (!spans || !host_blob) return JABAS_ERR_NULL;
+    if (n_bounds && !bounds) return JABAS_ERR_NULL;
+    if (n_span < 1 || n_span > (1u << 24)) return JABAS_ERR_SIZE;
+    if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
+    if (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
+    if (opt_class_of(opt_kind) < 0) return JABAS_ERR_OPT;
+    if (blob_bytes < jabas_plan_bytes(n_span, n_bounds)) return JABAS_ERR_PLAN;
+    if (reinterpret_cast<uintptr_t>(host_blob) % 8) return JABAS_ERR_ALIGN;
+
+    char* base = static_cast<char*>(host_blob);
+    memset(base, 0, jabas_plan_bytes(n_span, n_bounds));
+    PlanHeader h;
+    memset(&h, 0, sizeof(h));
+    h.magic = kPlanMagic;
+    h.version = kPlanVersion;
+    h.n_span = n_span;
+    h.n_bounds = n_bounds;
+    h.K = K;
+    h.grad_dtype = grad_dtype;
+    h.opt_kind = opt_kind;
+    h.off_spans = kHeaderBytes;
+    h.off_prefix = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
+    h.off_bounds = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
+    h.total_bytes = jabas_plan_bytes(n_span, n_bounds);
+    h.all_have_s1 = 1;
+
+    SpanDev* sd = reinterpret_cast<SpanDev*>(base + h.off_spans);
+    uint32_t* prefix = reinterpret_cast<uint32_t*>(base + h.off_prefix);
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < n_span; ++i) {
+        uint32_t tiles = 0;
+        int rc = encode_span(spans[i], K, grad_dtype, opt_kind, &sd[i], &tiles);
+        if (rc != JABAS_OK) return rc;
+        rc = check_bounds_host(spans[i], bounds, n_bounds, &h.max_group);
+        if (rc != JABAS_OK) return rc;
+        if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
+        prefix[i] = static_cast<uint32_t>(total);
+        total += tiles;
+        if (total > 0x7fffffffull) return JABAS_ERR_SIZE;
+    }
+    prefix[n_span] = static_cast<uint32_t>(total);
+    h.n_tiles = static_cast<uint32_t>(total);
+    if (n_bounds) memcpy(base + h.off_bounds, bounds, static_cast<size_t>(n_bounds) * sizeof(JabasBound));
+    memcpy(base, &h, sizeof(h));
+    return JABAS_OK;
+}
+
+JABAS_API int64_t jabas_plan_tiles(const void* host_blob) {
+    if (!host_blob) return JABAS_ERR_NULL;
+    PlanHeader h;
+    memcpy(&h, host_blob, sizeof(h));
+    if (h.magic != kPlanMagic || h.version != kPlanVersion) return JABAS_ERR_PLAN;
+    return h.n_tiles;
+}
+
+JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, const JabasStepArgs* args,
+                               double* stats_out, void* workspace, size_t workspace_bytes,
+                               jabas_stream_t stream) {
+    if (!plan_host || !plan_dev || !args) return JABAS_ERR_NULL;
+    PlanHeader h;
+    memcpy(&h, plan_host, sizeof(h));
+    if (h.magic != kPlanMagic || h.version != kPlanVersion) return JABAS_ERR_PLAN;
+    if (reinterpret_cast<uintptr_t>(plan_dev) % 16) return JABAS_ERR_ALIGN;
+    KArgs a;
+    int rc = fill_kargs(args, &a);
+    if (rc != JABAS_OK) return rc;
+    if (args->K != h.K || args->grad_dtype != h.grad_dtype) return JABAS_ERR_PLAN;
+    const int oc = opt_class_of(args->opt_kind);
+    if (oc != 0) {
+        if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;       // state pointers were not validated
+        if (h.max_group >= static_cast<uint32_t>(args->n_groups)) return JABAS_ERR_GROUP;
+        if (oc == 1 && args->momentum != 0.0 && !h.all_have_s1) return JABAS_ERR_NULL;
+    }
+    const char* dev = static_cast<const char*>(plan_dev);
+    a.spans = reinterpret_cast<const SpanDev*>(dev + h.off_spans);
+    a.tile_prefix = reinterpret_cast<const uint32_t*>(dev + h.off_prefix);
+    a.bounds = h.n_bounds ? reinterpret_cast<const BoundDev*>(dev + h.off_bounds) : nullptr;
+    a.n_span = h.n_span;
+    a.n_tiles = h.n_tiles;
+    a.use_inline = 0;
+    return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev, const JabasStepArgs* args,
+                                double* stats_out, void* workspace, size_t workspace_bytes,
+                                jabas_stream_t stream) {
+    if (!span || !args) return JABAS_ERR_NULL;
+    KArgs a;
+    int rc = fill_kargs(args, &a);
+    if (rc != JABAS_OK) return rc;
+    uint32_t tiles = 0;
+    rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind, &a.span0, &tiles);
+    if (rc != JABAS_OK) return rc;
+    const int oc = opt_class_of(args->opt_kind);
+    if (oc == 1 && args->momentum != 0.0 && !span->state1) return JABAS_ERR_NULL;
+    if (span->bound_count && !bounds_dev) return JABAS_ERR_NULL;
+    // bounds_dev is indexed from its own start: the span's entries begin at element 0 of it
+    a.span0.bound_begin = 0;
+    a.bounds = reinterpret_cast<const BoundDev*>(bounds_dev);
+    a.spans = nullptr;
+    a.tile_prefix = nullptr;
+    a.n_span = 1;
+    a.n_tiles = tiles;
+    a.use_inline = 1;
+    return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+JABAS_API int jabas_aggregate(const void* const* grads, int32_t K, int32_t grad_dtype, const float* weight,
+                              float* out, uint64_t numel, jabas_stream_t stream) {
+    if (!grads || !weight || !out) return JABAS_ERR_NULL;
+    if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
+    JabasSpan sp;
+    memset(&sp, 0, sizeof(sp));
+    JabasStepArgs s;
+    memset(&s, 0, sizeof(s));
+    for (int k = 0; k < K; ++k) { sp.grads[k] = grads[k]; s.weight[k] = weight[k]; }
+    sp.agg_out = out;
+    sp.numel = numel;
+    s.K = K;
+    s.grad_dtype = grad_dtype;
+    s.opt_kind = JABAS_OPT_NONE;
+    return jabas_sync_bucket(&sp, nullptr, &s, nullptr, nullptr, 0, stream);
+}
+
+JABAS_API int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype, const float* weight,
+                          const uint8_t* half_id, const float* half_weight, uint64_t numel, double* stats_out,
+                          void* workspace, size_t workspace_bytes, jabas_stream_t stream) {
+    if (!grads || !weight || !half_id || !half_weight || !stats_out) return JABAS_ERR_NULL;
+    if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
+    JabasSpan sp;
+    memset(&sp, 0, sizeof(sp));
+    JabasStepArgs s;
+    memset(&s, 0, sizeof(s));
+    for (int k = 0; k < K; ++k) {
+        sp.grads[k] = grads[k];
+        s.weight[k] = weight[k];
+        s.half_id[k] = half_id[k];
+        s.half_weight[k] = half_weight[k];
+    }
+    sp.numel = numel;
+    s.K = K;
+    s.grad_dtype = grad_dtype;
+    s.stats = 1;
+    s.opt_kind = JABAS_OPT_NONE;
+    return jabas_sync_bucket(&sp, nullptr, &s, stats_out, workspace, workspace_bytes, stream);
+}
+
+JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype, uint64_t numel,
+                         double* gram_out, void* workspace, size_t workspace_bytes, jabas_stream_t stream) {
+    if (!grads || !gram_out) return JABAS_ERR_NULL;
+    if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
+    if (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(gram_out) % 8) return JABAS_ERR_ALIGN;
+    JabasSpan sp;
+    memset(&sp, 0, sizeof(sp));
+    for (int k = 0; k < K; ++k) sp.grads[k] = grads[k];
+    sp.numel = numel;
+    SpanDev sd;
+    uint32_t tiles = 0;
+    const int rc = encode_span(sp, K, grad_dtype, JABAS_OPT_NONE, &sd, &tiles);
+    if (rc != JABAS_OK) return rc;
+    uint64_t g = static_cast<uint64_t>(cu_count()) * 4;
+    if (g > tiles) g = tiles;
+    if (g < 1) g = 1;
+    if (g > static_cast<uint64_t>(kMaxGrid)) g = kMaxGrid;
+    if (workspace_bytes < g * JABAS_GRAM_STRIDE * sizeof(double)) return JABAS_ERR_WORKSPACE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (launch_gram(K, grad_dtype, sd, static_cast<double*>(workspace), static_cast<unsigned>(g), st) != 0)
+        return JABAS_ERR_LAUNCH;
+    if (launch_gram_finalize(K, static_cast<const double*>(workspace), static_cast<unsigned>(g), gram_out, st) != 0)
+        return JABAS_ERR_LAUNCH;
+    return JABAS_OK;
+}
+
+JABAS_API int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t numel, double lr,
+                        double weight_decay, double momentum, double dampening, int32_t nesterov,
+                        int32_t first_step, jabas_stream_t stream) {
+    if (!grad || !param) return JABAS_ERR_NULL;
+    JabasSpan sp;
+    memset(&sp, 0, sizeof(sp));
+    JabasStepArgs s;
+    memset(&s, 0, sizeof(s));
+    sp.grads[0] = grad;
+    sp.param = param;
+    sp.state1 = momentum_buf;
+    sp.numel = numel;
+    s.K = 1;
+    s.grad_dtype = JABAS_F32;
+    s.weight[0] = 1.0f;              // g * 1.0f is exact: the "aggregate" is the gradient itself
+    s.opt_kind = JABAS_OPT_SGD;
+    s.n_groups = 1;
+    s.first_step = first_step;
+    s.nesterov = nesterov;
+    s.momentum = momentum;
+    s.dampening = dampening;
+    s.groups[0].lr = lr;
+    s.groups[0].weight_decay = weight_decay;
+    s.groups[0].step = 1;
+    return jabas_sync_bucket(&sp, nullptr, &s, nullptr, nullptr, 0, stream);
+}
+
+JABAS_API int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq, uint64_t numel,
+                         double lr, double weight_decay, double beta1, double beta2, double eps, int64_t step,
+                         int32_t adamw, jabas_stream_t stream) {
+    if (!grad || !param || !exp_avg || !exp_avg_sq) return JABAS_ERR_NULL;
+    JabasSpan sp;
+    memset(&sp, 0, sizeof(sp));
+    JabasStepArgs s;
+    memset(&s, 0, sizeof(s));
+    sp.grads[0] = grad;
+    sp.param = param;
+    sp.state1 = exp_avg;
+    sp.state2 = exp_avg_sq;
+    sp.numel = numel;
+    s.K = 1;
+    s.grad_dtype = JABAS_F32;
+    s.weight[0] = 1.0f;
+    s.opt_kind = adamw ? JABAS_OPT_ADAMW : JABAS_OPT_ADAM;
+    s.n_groups = 1;
+    s.beta1 = beta1;
+    s.beta2 = beta2;
+    s.eps = eps;
+    s.groups[0].lr = lr;
+    s.groups[0].weight_decay = weight_decay;
+    s.groups[0].step = step;
+    return jabas_sync_bucket(&sp, nullptr, &s, nullptr, nullptr, 0, stream);
+}

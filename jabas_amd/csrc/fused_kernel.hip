@@ -1,0 +1,397 @@
+// Fused VSW-aggregate + gradient statistics + optimizer kernel for gfx950 (MI355X).
+// Compiled once per JABAS_K (number of virtual stream workers) so that the K gradient
+// streams are fully unrolled into independent 128-bit loads.
+//
+// Execution shape
+//   - persistent grid of 256-thread workgroups (4 wave64); workgroup b owns the
+//     contiguous tile range [b*T/G, (b+1)*T/G) of the launch, T = tiles, G = gridDim.x;
+//   - a tile is 256 threads x one 16-byte gradient vector (4 fp32 or 8 bf16 elements);
+//   - tiles that lie wholly inside the live range of a span and inside one parameter
+//     group take the vector path (all loads of U tiles issued before any arithmetic);
+//     the few tiles that straddle a span end or a group change take a scalar path;
+//   - statistics: per-thread fp64 accumulators -> wave64 shuffle tree -> LDS across
+//     the 4 waves -> one partial row per (workgroup, span) in the workspace, summed in
+//     fixed order by the finalize kernel. Same grid => same bits, run to run.
+//
+// Arithmetic is compiled with -ffp-contract=off: every fp32 product and sum of the
+// aggregate and of the optimizer formulas is rounded on its own, so results can be
+// compared bit for bit with a CPU restatement that applies the same operations in the
+// same order. The formulas follow torch 1.8.1 optim/_functional.py (sgd, adam, adamw),
+// the version the reference pins (README.md:59-64 of the JABAS repository).
+#include "jabas_internal.h"
+
+#ifndef JABAS_K
+#error "compile with -DJABAS_K=<1..8>"
+#endif
+#ifndef JABAS_UNROLL_F32
+#define JABAS_UNROLL_F32 2
+#endif
+#ifndef JABAS_UNROLL_BF16
+#define JABAS_UNROLL_BF16 1
+#endif
+
+namespace jabas {
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+template <int DT> struct Grad;
+
+template <> struct Grad<JABAS_F32> {
+    static constexpr int EPT = 4;
+    using Raw = f32x4;
+    static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + e));
+    }
+    static __device__ __forceinline__ void widen(const Raw& r, float (&x)[4]) {
+        x[0] = r.x; x[1] = r.y; x[2] = r.z; x[3] = r.w;
+    }
+    static __device__ __forceinline__ float load1(const void* base, uint64_t e) {
+        return static_cast<const float*>(base)[e];
+    }
+};
+
+template <> struct Grad<JABAS_BF16> {
+    static constexpr int EPT = 8;
+    using Raw = u32x4;
+    static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + e));
+    }
+    // bf16 -> fp32 is exact: the 16 bits become the high half of the fp32 pattern.
+    static __device__ __forceinline__ void widen(const Raw& r, float (&x)[8]) {
+        x[0] = bits_to_float(r.x << 16); x[1] = bits_to_float(r.x & 0xffff0000u);
+        x[2] = bits_to_float(r.y << 16); x[3] = bits_to_float(r.y & 0xffff0000u);
+        x[4] = bits_to_float(r.z << 16); x[5] = bits_to_float(r.z & 0xffff0000u);
+        x[6] = bits_to_float(r.w << 16); x[7] = bits_to_float(r.w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ float load1(const void* base, uint64_t e) {
+        return bits_to_float(static_cast<uint32_t>(static_cast<const uint16_t*>(base)[e]) << 16);
+    }
+};
+
+constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2;
+
+template <int K, bool STATS> struct NStats { static constexpr int value = STATS ? 4 + K : 1; };
+
+// One element of the optimizer step. g is the aggregated gradient.
+template <int OPT>
+__device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2,
+                                         const GroupDev& G, const OptDev& O) {
+    if constexpr (OPT == OPT_SGD) {
+        float d = g;
+        if (G.wd != 0.0f) d = d + G.wd * p;
+        if (O.has_momentum) {
+            if (O.first_step) s1 = d;
+            else s1 = s1 * O.momentum + d * O.one_minus_damp;
+            d = O.nesterov ? d + O.momentum * s1 : s1;
+        }
+        p = p + G.neg_lr * d;
+    } else if constexpr (OPT == OPT_ADAM) {
+        if (O.adamw) p = p * G.decay;
+        else if (G.wd != 0.0f) g = g + G.wd * p;
+        s1 = s1 * O.beta1 + g * O.one_minus_beta1;
+        s2 = s2 * O.beta2 + (O.one_minus_beta2 * g) * g;
+        const float denom = __builtin_sqrtf(s2) / G.sqrt_bc2 + O.eps;
+        p = p + (G.neg_step_size * s1) / denom;
+    }
+}
+
+// Aggregate, statistics and optimizer for N consecutive elements held in registers.
+template <int K, int N, int OPT, bool STATS>
+__device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
+                                        float (&s2)[N], float (&agg)[N], const KArgs& a,
+                                        const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+        float s = g[0][i] * a.w[0];
+#pragma unroll
+        for (int k = 1; k < K; ++k) s = s + g[k][i] * a.w[k];
+        agg[i] = s;
+        if constexpr (STATS) {
+            float ga = 0.0f, gb = 0.0f;
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const float t = g[k][i] * a.wh[k];
+                const bool in_b = (a.half_mask >> k) & 1u;
+                gb = in_b ? gb + t : gb;
+                ga = in_b ? ga : ga + t;
+                const double gk = static_cast<double>(g[k][i]);
+                acc[JABAS_STAT_NORM_VSW0 + k] = __builtin_fma(gk, gk, acc[JABAS_STAT_NORM_VSW0 + k]);
+            }
+            // fp32 x fp32 products are exact in fp64, so fma == mul followed by add here.
+            const double da = static_cast<double>(ga), db = static_cast<double>(gb);
+            const double ds = static_cast<double>(s);
+            acc[JABAS_STAT_DOT_AB] = __builtin_fma(da, db, acc[JABAS_STAT_DOT_AB]);
+            acc[JABAS_STAT_NORM_A] = __builtin_fma(da, da, acc[JABAS_STAT_NORM_A]);
+            acc[JABAS_STAT_NORM_B] = __builtin_fma(db, db, acc[JABAS_STAT_NORM_B]);
+            acc[JABAS_STAT_NORM_AGG] = __builtin_fma(ds, ds, acc[JABAS_STAT_NORM_AGG]);
+        }
+        if constexpr (OPT != OPT_NONE) opt_elem<OPT>(s, p[i], s1[i], s2[i], G, a.opt);
+    }
+}
+
+template <int NV> __device__ __forceinline__ void load_vec(f32x4 (&r)[NV], const float* base, uint64_t e) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) r[v] = *reinterpret_cast<const f32x4*>(base + e + 4 * v);
+}
+template <int NV> __device__ __forceinline__ void store_vec(const float (&x)[4 * NV], float* base, uint64_t e) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        f32x4 r = {x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
+        *reinterpret_cast<f32x4*>(base + e + 4 * v) = r;
+    }
+}
+template <int NV> __device__ __forceinline__ void unpack_vec(const f32x4 (&r)[NV], float (&x)[4 * NV]) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) { x[4 * v] = r[v].x; x[4 * v + 1] = r[v].y; x[4 * v + 2] = r[v].z; x[4 * v + 3] = r[v].w; }
+}
+
+// Vector path over U consecutive full tiles of one parameter group. e is the (rebased)
+// index of this thread's first element in the first tile.
+template <int K, int DT, int OPT, bool STATS, int U>
+__device__ __forceinline__ void fast_tiles(const SpanDev& sp, uint64_t e, const KArgs& a, const GroupDev& G,
+                                           double (&acc)[NStats<K, STATS>::value]) {
+    using GR = Grad<DT>;
+    constexpr int EPT = GR::EPT, NV = EPT / 4;
+    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
+    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
+    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
+
+    typename GR::Raw rg[U][K];
+    f32x4 rp[U][NV], r1[U][NV], r2[U][NV];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t eu = e + u * TE;
+#pragma unroll
+        for (int k = 0; k < K; ++k) rg[u][k] = GR::load(sp.g[k], eu);
+        if constexpr (OPT != OPT_NONE) {
+            load_vec<NV>(rp[u], sp.p, eu);
+            if (load_s1) load_vec<NV>(r1[u], sp.s1, eu);
+            if constexpr (OPT == OPT_ADAM) load_vec<NV>(r2[u], sp.s2, eu);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const uint64_t eu = e + u * TE;
+        float g[K][EPT], p[EPT], s1[EPT], s2[EPT], agg[EPT];
+#pragma unroll
+        for (int k = 0; k < K; ++k) GR::widen(rg[u][k], g[k]);
+        if constexpr (OPT != OPT_NONE) {
+            unpack_vec<NV>(rp[u], p);
+            if (load_s1) unpack_vec<NV>(r1[u], s1);
+            else {
+#pragma unroll
+                for (int i = 0; i < EPT; ++i) s1[i] = 0.0f;
+            }
+            if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r2[u], s2);
+        }
+        compute<K, EPT, OPT, STATS>(g, p, s1, s2, agg, a, G, acc);
+        if (sp.out) store_vec<NV>(agg, sp.out, eu);
+        if constexpr (OPT != OPT_NONE) {
+            store_vec<NV>(p, sp.p, eu);
+            if (use_s1) store_vec<NV>(s1, sp.s1, eu);
+            if constexpr (OPT == OPT_ADAM) store_vec<NV>(s2, sp.s2, eu);
+            for (uint32_t r = 0; r < sp.n_fan; ++r) store_vec<NV>(p, sp.fan[r], eu);
+        }
+    }
+}
+
+// Scalar path for one tile that touches a span edge or a group change. tile_e0 is the
+// (rebased) index of the first element of the tile, j the bound entry covering the
+// first live element of the tile.
+template <int K, int DT, int OPT, bool STATS>
+__device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const KArgs& a, uint32_t j,
+                                          double (&acc)[NStats<K, STATS>::value]) {
+    using GR = Grad<DT>;
+    constexpr int EPT = GR::EPT;
+    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
+    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
+    const BoundDev* bd = sp.bound_count ? a.bounds + sp.bound_begin : nullptr;
+    const uint64_t e_first = tile_e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
+    for (int i = 0; i < EPT; ++i) {
+        const uint64_t e = e_first + i;
+        if (e < sp.lo || e >= sp.hi) continue;
+        uint32_t gid = 0;
+        if (bd) {
+            const uint64_t rel = e - sp.lo;
+            uint32_t jj = j;
+            while (jj + 1 < sp.bound_count && bd[jj + 1].start <= rel) ++jj;
+            gid = bd[jj].group;
+        }
+        const GroupDev G = a.groups[gid];
+        float g[K][1], p[1] = {0.0f}, s1[1] = {0.0f}, s2[1] = {0.0f}, agg[1];
+#pragma unroll
+        for (int k = 0; k < K; ++k) g[k][0] = GR::load1(sp.g[k], e);
+        if constexpr (OPT != OPT_NONE) {
+            p[0] = sp.p[e];
+            if (load_s1) s1[0] = sp.s1[e];
+            if constexpr (OPT == OPT_ADAM) s2[0] = sp.s2[e];
+        }
+        compute<K, 1, OPT, STATS>(g, p, s1, s2, agg, a, G, acc);
+        if (sp.out) sp.out[e] = agg[0];
+        if constexpr (OPT != OPT_NONE) {
+            sp.p[e] = p[0];
+            if (use_s1) sp.s1[e] = s1[0];
+            if constexpr (OPT == OPT_ADAM) sp.s2[e] = s2[0];
+            for (uint32_t r = 0; r < sp.n_fan; ++r) sp.fan[r][e] = p[0];
+        }
+    }
+}
+
+// Tiles [lt0, lt1) of one span (tile indices local to the span).
+template <int K, int DT, int OPT, bool STATS>
+__device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, const KArgs& a,
+                                           double (&acc)[NStats<K, STATS>::value]) {
+    using GR = Grad<DT>;
+    constexpr int EPT = GR::EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
+    constexpr int U = (DT == JABAS_BF16) ? JABAS_UNROLL_BF16 : JABAS_UNROLL_F32;
+    const uint32_t nb = sp.bound_count;
+    const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
+    uint32_t lt = lt0, j = 0;
+    while (lt < lt1) {
+        const uint64_t e0 = static_cast<uint64_t>(lt) * TE;
+        const uint64_t cur = e0 > sp.lo ? e0 : sp.lo;
+        const uint64_t rel = cur - sp.lo;
+        uint64_t stretch_end = sp.hi;
+        uint32_t gid = 0;
+        if (nb) {
+            while (j + 1 < nb && bd[j + 1].start <= rel) ++j;
+            gid = bd[j].group;
+            if (j + 1 < nb) stretch_end = sp.lo + bd[j + 1].start;
+        }
+        uint32_t nfull = 0;
+        if (e0 >= sp.lo && stretch_end >= e0 + TE) {
+            const uint64_t fit = (stretch_end - e0) / TE;
+            const uint32_t left = lt1 - lt;
+            nfull = fit < left ? static_cast<uint32_t>(fit) : left;
+        }
+        if (nfull) {
+            const GroupDev G = a.groups[gid];
+            uint64_t e = e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
+            uint32_t i = 0;
+            for (; i + U <= nfull; i += U, e += U * TE) fast_tiles<K, DT, OPT, STATS, U>(sp, e, a, G, acc);
+            if constexpr (U > 1) {
+                for (; i < nfull; ++i, e += TE) fast_tiles<K, DT, OPT, STATS, 1>(sp, e, a, G, acc);
+            }
+            lt += nfull;
+        } else {
+            careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, acc);
+            lt += 1;
+        }
+    }
+}
+
+template <int NS>
+__device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
+    __shared__ double red[kWaves][NS];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        double v = acc[i];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+        if (lane == 0) red[wave][i] = v;
+        acc[i] = 0.0;
+    }
+    __syncthreads();
+    if (threadIdx.x < NS) {
+        double s = red[0][threadIdx.x];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) s += red[w][threadIdx.x];
+        row[threadIdx.x] = s;
+    }
+    __syncthreads();
+}
+
+template <int K, int DT, int OPT, bool STATS>
+__global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
+    constexpr int NS = NStats<K, STATS>::value;
+    const uint32_t G = gridDim.x, b = blockIdx.x;
+    uint32_t t = static_cast<uint32_t>(static_cast<uint64_t>(b) * a.n_tiles / G);
+    const uint32_t t1 = static_cast<uint32_t>(static_cast<uint64_t>(b + 1) * a.n_tiles / G);
+    uint32_t s = 0;
+    if (!a.use_inline) {                      // largest s with tile_prefix[s] <= t
+        uint32_t lo = 0, hi = a.n_span;       // invariant: prefix[lo] <= t < prefix[hi]
+        while (hi - lo > 1) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (a.tile_prefix[mid] <= t) lo = mid; else hi = mid;
+        }
+        s = lo;
+    }
+    double acc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) acc[i] = 0.0;
+
+    while (t < t1) {
+        uint32_t ts0 = 0, ts1 = a.n_tiles;
+        if (!a.use_inline) { ts0 = a.tile_prefix[s]; ts1 = a.tile_prefix[s + 1]; }
+        const uint32_t te = t1 < ts1 ? t1 : ts1;
+        if (te > t) {
+            if (a.use_inline) span_range<K, DT, OPT, STATS>(a.span0, t - ts0, te - ts0, a, acc);
+            else span_range<K, DT, OPT, STATS>(a.spans[s], t - ts0, te - ts0, a, acc);
+            if constexpr (STATS)
+                flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b + s) * kStatsStride);
+        }
+        t = te;
+        ++s;
+    }
+}
+
+template <int K, int DT, int OPT, bool STATS>
+int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
+    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(kBlock), 0, stream, a);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <int K, int DT, int OPT, bool STATS>
+int occupancy_one() {
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fused_kernel<K, DT, OPT, STATS>, kBlock, 0) != hipSuccess || n < 1)
+        n = 2;
+    return n;
+}
+
+}  // namespace
+
+#define JABAS_CAT_(a, b) a##b
+#define JABAS_CAT(a, b) JABAS_CAT_(a, b)
+
+#define JABAS_DISPATCH(FN, ...)                                                              \
+    const int key = (grad_dtype == JABAS_BF16 ? 6 : 0) + opt_class * 2 + (stats ? 1 : 0);    \
+    switch (key) {                                                                           \
+        case 0:  return FN<JABAS_K, JABAS_F32, OPT_NONE, false>(__VA_ARGS__);                \
+        case 1:  return FN<JABAS_K, JABAS_F32, OPT_NONE, true>(__VA_ARGS__);                 \
+        case 2:  return FN<JABAS_K, JABAS_F32, OPT_SGD, false>(__VA_ARGS__);                 \
+        case 3:  return FN<JABAS_K, JABAS_F32, OPT_SGD, true>(__VA_ARGS__);                  \
+        case 4:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, false>(__VA_ARGS__);                \
+        case 5:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, true>(__VA_ARGS__);                 \
+        case 6:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, false>(__VA_ARGS__);               \
+        case 7:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, true>(__VA_ARGS__);                \
+        case 8:  return FN<JABAS_K, JABAS_BF16, OPT_SGD, false>(__VA_ARGS__);                \
+        case 9:  return FN<JABAS_K, JABAS_BF16, OPT_SGD, true>(__VA_ARGS__);                 \
+        case 10: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, false>(__VA_ARGS__);               \
+        case 11: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, true>(__VA_ARGS__);                \
+        default: return -1;                                                                  \
+    }
+
+int JABAS_CAT(launch_fused_k, JABAS_K)(int grad_dtype, int opt_class, int stats, const KArgs& a,
+                                       unsigned grid, hipStream_t stream) {
+    JABAS_DISPATCH(launch_one, a, grid, stream)
+}
+
+int JABAS_CAT(occupancy_k, JABAS_K)(int grad_dtype, int opt_class, int stats) {
+    static int cache[12] = {0};
+    const int k = (grad_dtype == JABAS_BF16 ? 6 : 0) + opt_class * 2 + (stats ? 1 : 0);
+    if (k < 0 || k >= 12) return 1;
+    if (cache[k] == 0) {
+        auto query = [&]() -> int { JABAS_DISPATCH(occupancy_one) };
+        cache[k] = query();
+    }
+    return cache[k];
+}
+
+}  // namespace jabas

@@ -1,0 +1,85 @@
+// Shared between the C-ABI front (api.hip) and the per-K kernel translation units
+// (fused_kernel.hip compiled once per JABAS_K). Not part of the public interface.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "jabas_sync.h"
+
+namespace jabas {
+
+constexpr int kBlock = 256;                 // threads per workgroup = 4 wave64
+constexpr int kWaves = kBlock / 64;
+constexpr int kMaxGrid = 4096;              // upper bound of persistent workgroups
+constexpr int kStatsStride = JABAS_STATS_STRIDE;
+
+// Elements one thread handles per tile: one 16-byte gradient vector.
+__host__ __device__ constexpr int ept_of(int grad_dtype) { return grad_dtype == JABAS_BF16 ? 8 : 4; }
+__host__ __device__ constexpr int tile_elems(int grad_dtype) { return kBlock * ept_of(grad_dtype); }
+
+// A span as the kernels see it. Pointers are rebased downwards by `lo` elements so that
+// element index 0 of every buffer is 16-byte aligned; [lo, hi) is the live range.
+struct SpanDev {
+    const void* g[JABAS_MAX_K];
+    float* out;
+    float* p;
+    float* s1;
+    float* s2;
+    float* fan[JABAS_MAX_K - 1];
+    uint64_t lo, hi;
+    uint32_t n_fan;
+    uint32_t bound_begin;
+    uint32_t bound_count;
+    uint32_t pad;
+};
+
+struct BoundDev {                            // same layout as JabasBound
+    uint64_t start;                          // in un-rebased span coordinates
+    uint32_t group;
+    uint32_t pad;
+};
+
+// fp32 constants of one parameter group, derived on the host in double and rounded once,
+// the way a Python float becomes an fp32 kernel scalar.
+struct GroupDev {
+    float wd;            // weight_decay
+    float neg_lr;        // SGD: -lr
+    float decay;         // AdamW: 1 - lr*wd
+    float neg_step_size; // Adam: -(lr / (1 - beta1^t))
+    float sqrt_bc2;      // Adam: sqrt(1 - beta2^t)
+    float pad[3];
+};
+
+struct OptDev {
+    float momentum, one_minus_damp;
+    float beta1, one_minus_beta1, beta2, one_minus_beta2, eps;
+    int32_t has_momentum, first_step, nesterov, adamw;
+};
+
+struct KArgs {
+    const SpanDev* spans;                    // device table (n_span > 1 or planned launch)
+    const uint32_t* tile_prefix;             // n_span + 1 entries, device
+    const BoundDev* bounds;                  // device, may be NULL
+    double* partials;                        // (grid + n_span) * kStatsStride doubles
+    uint32_t n_span;
+    uint32_t n_tiles;
+    uint32_t use_inline;                     // 1: the only span is `span0`
+    uint32_t half_mask;                      // bit k set: VSW k belongs to half B
+    SpanDev span0;
+    float w[JABAS_MAX_K];
+    float wh[JABAS_MAX_K];
+    OptDev opt;
+    GroupDev groups[JABAS_MAX_GROUPS];
+};
+
+// Per-K launchers, one translation unit each (fused_kernel.hip with -DJABAS_K=k).
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW. Returns hipError_t as int.
+#define JABAS_DECLARE_K(k)                                                                   \
+    int launch_fused_k##k(int grad_dtype, int opt_class, int stats, const KArgs& a,          \
+                          unsigned grid, hipStream_t stream);                                \
+    int occupancy_k##k(int grad_dtype, int opt_class, int stats);
+JABAS_DECLARE_K(1) JABAS_DECLARE_K(2) JABAS_DECLARE_K(3) JABAS_DECLARE_K(4)
+JABAS_DECLARE_K(5) JABAS_DECLARE_K(6) JABAS_DECLARE_K(7) JABAS_DECLARE_K(8)
+#undef JABAS_DECLARE_K
+
+}  // namespace jabas

@@ -1,0 +1,106 @@
+"""Flat-arena owner of one GPU's gradient-sync state.
+
+``VSWFlatSync`` lays the whole gradient set out MI355X-first: one arena per VSW for the
+gradient buckets, one each for the aggregated gradient, the fp32 weights and the
+optimizer state, all with the same bucket layout (FlatLayout), so that a whole sync
+step is one kernel launch over a device-resident span table instead of the reference's
+per-bucket hook plus per-tensor optimizer loop (jabas/train/trainer.py:327-337,
+examples/gnmt/seq2seq/train/shard_optimizer.py:40-90). Model code reaches its tensors
+through views (``param_view``, ``grad_view``).
+"""
+import torch
+
+from . import _lib as L
+from .layout import FlatLayout
+from .sync import SpanSpec, SyncPlan, make_step_args, opt_kind, cosine_from_stats
+
+
+class VSWFlatSync:
+    def __init__(self, specs, batches, grad_dtype=torch.float32, opt=None, device="cuda", in_place=None,
+                 n_fanout=0, per_tensor_spans=False, caps=None):
+        self.K = len(batches)
+        self.batches = tuple(batches)
+        self.grad_dtype = grad_dtype
+        self.opt = opt
+        self.device = torch.device(device)
+        kw = {} if caps is None else {"caps": caps}
+        self.layout = FlatLayout(specs, per_tensor_spans=per_tensor_spans, **kw)
+        n = self.layout.total
+        # in place: the aggregate overwrites VSW 0's buckets, as the reference's main VSW
+        # bucket ends up holding the synchronised gradient
+        if in_place is None:
+            in_place = grad_dtype == torch.float32
+        if in_place and grad_dtype != torch.float32:
+            raise ValueError("in-place aggregation needs fp32 gradient buckets")
+        self.grads = [torch.zeros(n, dtype=grad_dtype, device=self.device) for _ in range(self.K)]
+        self.agg = self.grads[0] if in_place else torch.zeros(n, dtype=torch.float32, device=self.device)
+        kind = opt_kind(opt)
+        self.param = self.state1 = self.state2 = None
+        self.fanout = []
+        if kind != L.OPT_NONE:
+            if len(opt["groups"]) < self.layout.n_groups:
+                raise ValueError(f"layout names {self.layout.n_groups} parameter groups, optimizer has "
+                                 f"{len(opt['groups'])}")
+            self.param = torch.zeros(n, dtype=torch.float32, device=self.device)
+            if kind != L.OPT_SGD or opt.get("momentum", 0.0) != 0.0:
+                self.state1 = torch.zeros(n, dtype=torch.float32, device=self.device)
+            if kind in (L.OPT_ADAM, L.OPT_ADAMW):
+                self.state2 = torch.zeros(n, dtype=torch.float32, device=self.device)
+            self.fanout = [torch.zeros(n, dtype=torch.float32, device=self.device) for _ in range(n_fanout)]
+        spans = []
+        for (off, numel, bounds, _bucket) in self.layout.spans:
+            sl = slice(off, off + numel)
+            spans.append(SpanSpec(
+                [g[sl] for g in self.grads], agg_out=self.agg[sl],
+                param=None if self.param is None else self.param[sl],
+                state1=None if self.state1 is None else self.state1[sl],
+                state2=None if self.state2 is None else self.state2[sl],
+                fanout=[f[sl] for f in self.fanout],
+                bounds=bounds if kind != L.OPT_NONE else ()))
+        self.span_bucket = [s[3] for s in self.layout.spans]
+        self.plan = SyncPlan(spans, kind)
+        self.step_count = 0
+
+    # ---- views -------------------------------------------------------------------
+    def _view(self, arena, i):
+        off = self.layout.param_offset[i]
+        return arena[off:off + self.layout.specs[i].numel]
+
+    def param_view(self, i):
+        return self._view(self.param, i)
+
+    def grad_view(self, k, i):
+        return self._view(self.grads[k], i)
+
+    def agg_view(self, i):
+        return self._view(self.agg, i)
+
+    def bucket_slice(self, b):
+        bk = self.layout.buckets[b]
+        return slice(bk.offset, bk.offset + bk.numel)
+
+    # ---- the step ----------------------------------------------------------------
+    def step_args(self, stats=False, lr_scale=1.0, with_opt=True):
+        opt = self.opt if with_opt else None
+        first = self.step_count == 0
+        return make_step_args(self.batches, self.grad_dtype, stats=stats, opt=opt, step=self.step_count + 1,
+                              first_step=first, lr_scale=lr_scale)
+
+    def step(self, stats=False, lr_scale=1.0, stream=None):
+        """One fused sync step over the whole gradient set. Returns the per-span stats
+        tensor when ``stats`` is set."""
+        args = self.step_args(stats=stats, lr_scale=lr_scale)
+        out = self.plan.run(args, stream=stream)
+        self.step_count += 1
+        return out
+
+    def bucket_stats(self, stats):
+        """Per-bucket rows from per-span rows (spans of one bucket summed in span order)."""
+        nb = len(self.layout.buckets)
+        idx = torch.tensor(self.span_bucket, device=stats.device)
+        out = torch.zeros(nb, L.STATS_STRIDE, dtype=torch.float64, device=stats.device)
+        return out.index_add_(0, idx, stats)
+
+    @staticmethod
+    def cosine(stats):
+        return cosine_from_stats(stats)

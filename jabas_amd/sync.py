@@ -1,0 +1,340 @@
+"""Host side of the fused gradient-sync step: argument marshalling over the C ABI.
+
+Nothing here computes on tensors; every function ends in a libjabas_sync.so call queued
+on the current HIP stream. torch is used for device memory and streams only.
+
+Vocabulary: a *span* is one contiguous stretch of the flat layout (normally one DDP
+bucket) for which K gradient buffers, the aggregated-gradient output and the parameter /
+optimizer-state buffers are indexed alike; a *plan* is a launch-invariant table of spans.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib as L
+
+
+# ----------------------------------------------------------------------------- weights
+def batch_weights(batches, half_id=None):
+    """Per-VSW fp32 weights of the batch-weighted aggregate and of the two halves.
+
+    w_k = fp32(b_k / B): the quotient is formed in double and rounded once, which is what
+    a Python float becomes when ATen applies it to an fp32 tensor. Halves follow the
+    reference's rank-parity split (jabas/train/trainer.py:427-432) mapped onto the VSW
+    index: even k -> half A (0), odd k -> half B (1).
+    """
+    b = [float(x) for x in batches]
+    K = len(b)
+    if not 1 <= K <= L.MAX_K:
+        raise ValueError(f"number of VSWs must be in 1..{L.MAX_K}, got {K}")
+    if any(x <= 0 for x in b):
+        raise ValueError(f"local batch sizes must be positive: {batches}")
+    total = sum(b)
+    w = np.array([x / total for x in b], dtype=np.float64).astype(np.float32)
+    if half_id is None:
+        half_id = [k % 2 for k in range(K)]
+    half_id = np.array(half_id, dtype=np.uint8)
+    if half_id.shape != (K,) or np.any(half_id > 1):
+        raise ValueError("half_id must hold K entries of 0 or 1")
+    hw = np.zeros(K, dtype=np.float32)
+    for h in (0, 1):
+        tot = sum(x for x, hid in zip(b, half_id) if hid == h)
+        for k in range(K):
+            if half_id[k] == h:
+                hw[k] = np.float32(b[k] / tot)
+    return w, half_id, hw
+
+
+_KIND = {None: L.OPT_NONE, "none": L.OPT_NONE, "sgd": L.OPT_SGD, "adam": L.OPT_ADAM, "adamw": L.OPT_ADAMW}
+
+
+def opt_kind(opt):
+    kind = None if opt is None else opt["kind"]
+    if kind not in _KIND:
+        raise ValueError(f"unknown optimizer kind {kind!r}")
+    return _KIND[kind]
+
+
+def grad_dtype_code(dtype):
+    if dtype == torch.float32:
+        return L.F32
+    if dtype == torch.bfloat16:
+        return L.BF16
+    raise TypeError(f"gradient dtype must be float32 or bfloat16, got {dtype}")
+
+
+def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_step=False, half_id=None,
+                   lr_scale=1.0):
+    """Builds the JabasStepArgs of one call.
+
+    ``opt``: None or dict(kind='sgd'|'adam'|'adamw', groups=[dict(lr=, weight_decay=)], plus
+    momentum/dampening/nesterov or betas/eps). ``step`` is the 1-based Adam step count,
+    ``lr_scale`` the adaptive-batching LR modifier (jabas/train/trainer.py:693-700).
+    """
+    w, hid, hw = batch_weights(batches, half_id)
+    a = L.JabasStepArgs()
+    a.K = len(w)
+    a.grad_dtype = grad_dtype_code(grad_dtype)
+    for k in range(a.K):
+        a.weight[k] = float(w[k])
+        a.half_id[k] = int(hid[k])
+        a.half_weight[k] = float(hw[k])
+    a.stats = 1 if stats else 0
+    a.opt_kind = opt_kind(opt)
+    if opt is not None and a.opt_kind != L.OPT_NONE:
+        groups = opt["groups"]
+        if not 1 <= len(groups) <= L.MAX_GROUPS:
+            raise ValueError(f"1..{L.MAX_GROUPS} parameter groups supported, got {len(groups)}")
+        a.n_groups = len(groups)
+        for i, g in enumerate(groups):
+            a.groups[i].lr = float(g["lr"]) * float(lr_scale)
+            a.groups[i].weight_decay = float(g.get("weight_decay", 0.0))
+            a.groups[i].step = int(g.get("step", step))
+        a.first_step = 1 if first_step else 0
+        a.nesterov = 1 if opt.get("nesterov", False) else 0
+        a.momentum = float(opt.get("momentum", 0.0))
+        a.dampening = float(opt.get("dampening", 0.0))
+        b1, b2 = opt.get("betas", (0.9, 0.999))
+        a.beta1, a.beta2 = float(b1), float(b2)
+        a.eps = float(opt.get("eps", 1e-8))
+    return a
+
+
+# ------------------------------------------------------------------------------- spans
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _check_tensor(t, n, dtype, what, device):
+    if t is None:
+        return
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{what}: expected a tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{what}: expected {dtype}, got {t.dtype}")
+    if t.device != device:
+        raise ValueError(f"{what}: on {t.device}, expected {device}")
+    if not t.is_contiguous() or t.numel() != n:
+        raise ValueError(f"{what}: must be contiguous with {n} elements (has {t.numel()})")
+
+
+class SpanSpec:
+    """Tensors of one span. All 1-D (or contiguous) with the same number of elements."""
+
+    def __init__(self, grads, agg_out=None, param=None, state1=None, state2=None, fanout=(), bounds=()):
+        self.grads = list(grads)
+        self.agg_out, self.param, self.state1, self.state2 = agg_out, param, state1, state2
+        self.fanout = list(fanout)
+        self.bounds = list(bounds)          # [(start_element, group), ...], first start 0
+
+    def validate(self):
+        if not self.grads:
+            raise ValueError("a span needs at least one gradient buffer")
+        g0 = self.grads[0]
+        n, dev, gdt = g0.numel(), g0.device, g0.dtype
+        if dev.type != "cuda":
+            raise ValueError(f"gradient buffers must live on the GPU, got {dev}")
+        for k, g in enumerate(self.grads):
+            _check_tensor(g, n, gdt, f"grads[{k}]", dev)
+        _check_tensor(self.agg_out, n, torch.float32, "agg_out", dev)
+        _check_tensor(self.param, n, torch.float32, "param", dev)
+        _check_tensor(self.state1, n, torch.float32, "state1", dev)
+        _check_tensor(self.state2, n, torch.float32, "state2", dev)
+        for r, f in enumerate(self.fanout):
+            _check_tensor(f, n, torch.float32, f"fanout[{r}]", dev)
+        return n, dev, gdt
+
+    def to_c(self, bound_begin=0):
+        n, _, _ = self.validate()
+        s = L.JabasSpan()
+        for k, g in enumerate(self.grads):
+            s.grads[k] = g.data_ptr()
+        s.agg_out = _ptr(self.agg_out)
+        s.param = _ptr(self.param)
+        s.state1 = _ptr(self.state1)
+        s.state2 = _ptr(self.state2)
+        for r, f in enumerate(self.fanout):
+            s.fanout[r] = f.data_ptr()
+        s.numel = n
+        s.n_fanout = len(self.fanout)
+        s.bound_begin = bound_begin
+        s.bound_count = len(self.bounds)
+        return s
+
+
+def _bounds_array(bounds):
+    arr = (L.JabasBound * max(1, len(bounds)))()
+    for i, (start, group) in enumerate(bounds):
+        arr[i].start = int(start)
+        arr[i].group = int(group)
+    return arr
+
+
+def _stream_ptr(stream=None):
+    s = torch.cuda.current_stream() if stream is None else stream
+    return C.c_void_p(s.cuda_stream)
+
+
+class Workspace:
+    """Device scratch of the two-level statistics reduction plus the stats rows."""
+
+    def __init__(self, n_span, device):
+        nbytes = L.lib().jabas_sync_workspace_bytes(n_span)
+        self.buf = torch.empty(nbytes // 8, dtype=torch.float64, device=device)
+        self.nbytes = nbytes
+        self.stats = torch.zeros(n_span, L.STATS_STRIDE, dtype=torch.float64, device=device)
+
+
+class SyncPlan:
+    """A validated, device-resident table of spans; ``run`` queues the fused step."""
+
+    def __init__(self, spans, opt_kind_code=L.OPT_NONE):
+        lib = L.lib()
+        self.spans = list(spans)
+        if not self.spans:
+            raise ValueError("a plan needs at least one span")
+        n0, dev, gdt = self.spans[0].validate()
+        self.device, self.grad_dtype = dev, gdt
+        self.K = len(self.spans[0].grads)
+        self.opt_kind = opt_kind_code
+        n_span = len(self.spans)
+        c_spans = (L.JabasSpan * n_span)()
+        all_bounds = []
+        for i, sp in enumerate(self.spans):
+            _, d, t = sp.validate()
+            if d != dev or t != gdt or len(sp.grads) != self.K:
+                raise ValueError(f"span {i}: device, gradient dtype or K differs from span 0")
+            c_spans[i] = sp.to_c(bound_begin=len(all_bounds))
+            all_bounds += sp.bounds
+        c_bounds = _bounds_array(all_bounds)
+        nbytes = lib.jabas_plan_bytes(n_span, len(all_bounds))
+        self._host = np.zeros((nbytes + 7) // 8, dtype=np.uint64)        # 8-byte aligned blob
+        L.check(lib.jabas_plan_encode(c_spans, n_span, c_bounds if all_bounds else None, len(all_bounds),
+                                      self.K, grad_dtype_code(gdt), opt_kind_code,
+                                      self._host.ctypes.data, nbytes), "jabas_plan_encode")
+        self.n_tiles = int(lib.jabas_plan_tiles(self._host.ctypes.data))
+        self._dev = torch.from_numpy(self._host.view(np.int64)).to(dev)
+        self.ws = Workspace(n_span, dev)
+        self.n_span = n_span
+
+    def run(self, args, stream=None):
+        """Queues aggregate (+stats, +optimizer) over every span. Returns the stats tensor
+        (n_span x 12 doubles, device) when args.stats is set, else None."""
+        L.check(L.lib().jabas_sync_fused(self._host.ctypes.data, self._dev.data_ptr(), C.byref(args),
+                                         self.ws.stats.data_ptr() if args.stats else None,
+                                         self.ws.buf.data_ptr(), self.ws.nbytes, _stream_ptr(stream)),
+                "jabas_sync_fused")
+        return self.ws.stats if args.stats else None
+
+
+# ------------------------------------------------------------- single-bucket entry points
+def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
+    """One span by value (what a comm hook calls for the bucket it was handed)."""
+    c_span = span.to_c()
+    if span.bounds and bounds_dev is None:
+        host = np.zeros((len(span.bounds), 2), dtype=np.uint64)
+        for i, (start, group) in enumerate(span.bounds):
+            host[i, 0] = start
+            host[i, 1] = group                      # low 32 bits = group, high 32 = reserved
+        bounds_dev = torch.from_numpy(host.view(np.int64)).to(span.grads[0].device)
+    stats_ptr = ws_ptr = None
+    ws_bytes = 0
+    if args.stats:
+        if workspace is None:
+            workspace = Workspace(1, span.grads[0].device)
+        stats_ptr, ws_ptr, ws_bytes = workspace.stats.data_ptr(), workspace.buf.data_ptr(), workspace.nbytes
+    L.check(L.lib().jabas_sync_bucket(C.byref(c_span), None if bounds_dev is None else bounds_dev.data_ptr(),
+                                      C.byref(args), stats_ptr, ws_ptr, ws_bytes, _stream_ptr(stream)),
+            "jabas_sync_bucket")
+    if bounds_dev is not None:
+        bounds_dev.record_stream(torch.cuda.current_stream() if stream is None else stream)
+    return workspace.stats[0] if args.stats else None
+
+
+def _ptr_array(tensors):
+    arr = (C.c_void_p * len(tensors))()
+    for i, t in enumerate(tensors):
+        arr[i] = t.data_ptr()
+    return arr
+
+
+def aggregate(grads, batches, out=None, stream=None):
+    """out = sum_k w_k g_k (canonical order); ``out`` may be grads[0] for fp32 gradients."""
+    span = SpanSpec(grads)
+    n, dev, gdt = span.validate()
+    if out is None:
+        out = torch.empty(n, dtype=torch.float32, device=dev)
+    _check_tensor(out, n, torch.float32, "out", dev)
+    w, _, _ = batch_weights(batches)
+    if len(w) != len(grads):
+        raise ValueError("one batch size per gradient buffer")
+    cw = (C.c_float * len(w))(*[float(x) for x in w])
+    L.check(L.lib().jabas_aggregate(_ptr_array(grads), len(grads), grad_dtype_code(gdt), cw, out.data_ptr(), n,
+                                    _stream_ptr(stream)), "jabas_aggregate")
+    return out
+
+
+def gradient_stats(grads, batches, half_id=None, workspace=None, stream=None):
+    """Statistics row (12 doubles, device) of one span; writes nothing else."""
+    span = SpanSpec(grads)
+    n, dev, gdt = span.validate()
+    w, hid, hw = batch_weights(batches, half_id)
+    if len(w) != len(grads):
+        raise ValueError("one batch size per gradient buffer")
+    if workspace is None:
+        workspace = Workspace(1, dev)
+    K = len(w)
+    L.check(L.lib().jabas_stats(_ptr_array(grads), K, grad_dtype_code(gdt),
+                                (C.c_float * K)(*[float(x) for x in w]),
+                                (C.c_uint8 * K)(*[int(x) for x in hid]),
+                                (C.c_float * K)(*[float(x) for x in hw]), n,
+                                workspace.stats.data_ptr(), workspace.buf.data_ptr(), workspace.nbytes,
+                                _stream_ptr(stream)), "jabas_stats")
+    return workspace.stats[0]
+
+
+def gram(grads, stream=None):
+    """K x K Gram matrix (float64, device) of the worker gradients."""
+    span = SpanSpec(grads)
+    n, dev, gdt = span.validate()
+    K = len(grads)
+    ws = torch.empty(4096 * L.GRAM_STRIDE, dtype=torch.float64, device=dev)
+    out = torch.empty(L.GRAM_STRIDE, dtype=torch.float64, device=dev)
+    L.check(L.lib().jabas_gram(_ptr_array(grads), K, grad_dtype_code(gdt), n, out.data_ptr(), ws.data_ptr(),
+                               ws.numel() * 8, _stream_ptr(stream)), "jabas_gram")
+    ws.record_stream(torch.cuda.current_stream() if stream is None else stream)
+    return out.view(L.MAX_K, L.MAX_K)[:K, :K]
+
+
+def sgd_step(grad, param, momentum_buf, lr, weight_decay=0.0, momentum=0.0, dampening=0.0, nesterov=False,
+             first_step=False, stream=None):
+    n = param.numel()
+    _check_tensor(grad, n, torch.float32, "grad", param.device)
+    _check_tensor(momentum_buf, n, torch.float32, "momentum_buf", param.device)
+    L.check(L.lib().jabas_sgd(grad.data_ptr(), param.data_ptr(), _ptr(momentum_buf), n, lr, weight_decay, momentum,
+                              dampening, int(bool(nesterov)), int(bool(first_step)), _stream_ptr(stream)), "jabas_sgd")
+
+
+def adam_step(grad, param, exp_avg, exp_avg_sq, lr, weight_decay, betas, eps, step, adamw, stream=None):
+    n = param.numel()
+    for t, what in ((grad, "grad"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+        _check_tensor(t, n, torch.float32, what, param.device)
+    L.check(L.lib().jabas_adam(grad.data_ptr(), param.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
+                               lr, weight_decay, betas[0], betas[1], eps, int(step), int(bool(adamw)),
+                               _stream_ptr(stream)), "jabas_adam")
+
+
+# ---------------------------------------------------------------------- cosine similarity
+def cosine_from_stats(stats_rows, eps=1e-8):
+    """cos(g_A, g_B) over all spans from their statistics rows (host scalars).
+
+    Sums the per-span triples (the reference concatenates the per-bucket tensors instead,
+    jabas/train/trainer.py:475) and applies torch 1.8.1's cosine_similarity formula
+    dot / sqrt(max(|a|^2 |b|^2, eps^2)).
+    """
+    rows = stats_rows.detach().to("cpu", torch.float64).reshape(-1, L.STATS_STRIDE)
+    dot = float(rows[:, L.STAT_DOT_AB].sum())
+    na = float(rows[:, L.STAT_NORM_A].sum())
+    nb = float(rows[:, L.STAT_NORM_B].sum())
+    return dot / max(na * nb, eps * eps) ** 0.5

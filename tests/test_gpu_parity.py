@@ -1,0 +1,337 @@
+"""GPU parity: the HIP path, called through the C ABI (ctypes), against the CPU oracle on
+the same seeded inputs. Bars (from the path's specification):
+  aggregate            bit-exact (fp32 and bf16 inputs)
+  statistics           1e-6 relative (fp32 inputs), 1e-2 relative (bf16 inputs)
+  updated weights/state 1e-6 relative (plus an absolute floor of a few ulp of the operands,
+                       because m and buf are sums that may cancel)
+The optimizer checks additionally report how many elements are bit-identical.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BATCHES = {1: (32,), 2: (32, 32), 3: (4, 2, 2), 4: (48, 32, 32, 16), 5: (5, 4, 3, 2, 1),
+           6: (7, 7, 5, 3, 2, 1), 7: (64, 56, 48, 40, 32, 24, 16), 8: tuple(range(64, 0, -8))}
+
+SGD = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+           groups=[dict(lr=0.1, weight_decay=0.0), dict(lr=0.1, weight_decay=1e-4)])
+ADAMW = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+             groups=[dict(lr=5e-4, weight_decay=0.0), dict(lr=5e-4, weight_decay=0.05)])
+ADAM = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, groups=[dict(lr=2e-3, weight_decay=0.0),
+                                                                dict(lr=2e-3, weight_decay=1e-2)])
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int32)
+
+
+def _host_grads(K, n, seed, std=1e-3, dtype=torch.float32):
+    out = []
+    for k in range(K):
+        g = torch.Generator().manual_seed(1234 + 17 * seed + k)
+        out.append((torch.randn(n, generator=g) * std).to(dtype))
+    return out
+
+
+def _host_state(n, seed, scale=0.05):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(n, generator=g) * scale
+
+
+def _dev(t, gpu, skew=0):
+    """Device copy of t placed `skew` elements into a 256-byte aligned allocation."""
+    buf = torch.zeros(t.numel() + 16, dtype=t.dtype, device=gpu)
+    view = buf[skew:skew + t.numel()]
+    view.copy_(t)
+    return view
+
+
+def _close(got, want, rtol, atol):
+    got, want = got.detach().cpu().double(), want.detach().cpu().double()
+    err = (got - want).abs()
+    ok = err <= rtol * want.abs() + atol
+    return bool(ok.all()), float(err.max()) if err.numel() else 0.0
+
+
+def _same_bits(a, b):
+    a, b = _bits(a), _bits(b)
+    return int((a == b).sum()), a.numel()
+
+
+# ---------------------------------------------------------------------------- aggregate
+@pytest.mark.parametrize("K", range(1, 9))
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_aggregate_bit_exact(gpu, K, dtype):
+    from jabas_amd import sync
+    for n, skew in ((1, 0), (3, 1), (1023, 0), (1024, 2), (1025, 3), (4099, 0), (262144 + 77, 0), (1 << 20, 3)):
+        if dtype == torch.bfloat16:
+            skew *= 2            # fp32 outputs and bf16 inputs must agree on the position in a 16-byte line
+        print(f"aggregate K={K} {dtype} n={n} skew={skew}", flush=True)
+        hg = _host_grads(K, n, K + n % 7, dtype=dtype)
+        dg = [_dev(t, gpu, skew) for t in hg]
+        out = _dev(torch.zeros(n), gpu, skew)
+        sync.aggregate(dg, BATCHES[K], out=out)
+        torch.cuda.synchronize()
+        want = O.aggregate(hg, BATCHES[K])
+        assert torch.equal(_bits(out), _bits(want)), f"K={K} n={n} skew={skew}"
+
+
+def test_aggregate_in_place_into_vsw0_bucket(gpu):
+    from jabas_amd import sync
+    K, n = 4, 50001
+    hg = _host_grads(K, n, 3)
+    dg = [_dev(t, gpu) for t in hg]
+    sync.aggregate(dg, BATCHES[K], out=dg[0])
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(dg[0]), _bits(O.aggregate(hg, BATCHES[K])))
+    for k in range(1, K):
+        assert torch.equal(_bits(dg[k]), _bits(hg[k]))        # other workers' buckets untouched
+
+
+def test_aggregate_keeps_zero_rows_exactly_zero(gpu):
+    from jabas_amd import sync
+    K, rows, cols = 4, 512, 1024
+    mask = torch.rand(rows, generator=torch.Generator().manual_seed(0)) < 0.1
+    hg = [torch.where(mask[:, None], t.view(rows, cols), torch.zeros(())).reshape(-1)
+          for t in _host_grads(K, rows * cols, 5)]
+    out = sync.aggregate([_dev(t, gpu) for t in hg], BATCHES[K])
+    torch.cuda.synchronize()
+    got = out.cpu().view(rows, cols)
+    assert torch.all(got[~mask].view(torch.int32) == 0)
+    assert torch.equal(_bits(out), _bits(O.aggregate(hg, BATCHES[K])))
+
+
+# --------------------------------------------------------------------------- statistics
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-6), (torch.bfloat16, 1e-2)])
+def test_stats_row(gpu, K, dtype, rtol):
+    from jabas_amd import sync
+    for n, skew in ((5, 0), (4099, 1), (300007, 0), (1 << 21, 2)):
+        if dtype == torch.bfloat16:
+            skew *= 2
+        print(f"stats K={K} {dtype} n={n} skew={skew}", flush=True)
+        hg = _host_grads(K, n, 20 + K, std=5e-4, dtype=dtype)
+        row = sync.gradient_stats([_dev(t, gpu, skew) for t in hg], BATCHES[K])
+        torch.cuda.synchronize()
+        want = O.stats(hg, BATCHES[K])
+        got = row.cpu()
+        ok, err = _close(got[:4 + K], want[:4 + K], rtol, 1e-30)
+        assert ok, f"K={K} n={n}: {got} vs {want}"
+        assert torch.count_nonzero(got[4 + K:]) == 0
+        # fp64 accumulation: in fact far inside the bar
+        assert _close(got[:4 + K], want[:4 + K], 1e-11, 1e-30)[0]
+
+
+def test_stats_run_to_run_deterministic(gpu):
+    from jabas_amd import sync
+    hg = _host_grads(4, 3_000_001, 41)
+    dg = [_dev(t, gpu) for t in hg]
+    a = sync.gradient_stats(dg, BATCHES[4]).cpu().clone()
+    for _ in range(3):
+        b = sync.gradient_stats(dg, BATCHES[4]).cpu()
+        assert torch.equal(a.view(torch.int64), b.view(torch.int64))
+
+
+def test_stats_cosine_identities(gpu):
+    from jabas_amd import sync
+    g0 = _dev(_host_grads(1, 100003, 43)[0], gpu)
+    assert sync.cosine_from_stats(sync.gradient_stats([g0, g0.clone()], (8, 8))) == pytest.approx(1.0, abs=1e-12)
+    assert sync.cosine_from_stats(sync.gradient_stats([g0, -g0], (8, 8))) == pytest.approx(-1.0, abs=1e-12)
+    z = torch.zeros(1000, device=gpu)
+    assert sync.cosine_from_stats(sync.gradient_stats([z, z], (1, 1))) == 0.0
+
+
+@pytest.mark.parametrize("K", [1, 2, 5, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gram(gpu, K, dtype):
+    from jabas_amd import sync
+    for n, skew in ((7, 0), (100003, 2), (1 << 20, 0)):
+        if dtype == torch.bfloat16:
+            skew *= 2
+        hg = _host_grads(K, n, 30 + K, dtype=dtype)
+        G = sync.gram([_dev(t, gpu, skew) for t in hg]).cpu()
+        want = O.gram(hg)
+        assert _close(G, want, 1e-11, 1e-30)[0], f"K={K} n={n}"
+        assert torch.equal(G, G.t())
+
+
+# ---------------------------------------------------------------------------- optimizer
+@pytest.mark.parametrize("hp", [
+    dict(lr=0.1, weight_decay=1e-4, momentum=0.9, dampening=0.0, nesterov=False),
+    dict(lr=0.05, weight_decay=5e-4, momentum=0.8, dampening=0.0, nesterov=True),
+    dict(lr=0.05, weight_decay=1e-3, momentum=0.7, dampening=0.3, nesterov=False),
+    dict(lr=0.3, weight_decay=1e-2, momentum=0.0, dampening=0.0, nesterov=False),
+])
+def test_sgd_steps(gpu, hp):
+    from jabas_amd import sync
+    n, steps = 70001, 4
+    p_h, buf_h = _host_state(n, 1), torch.zeros(n)
+    p_d, buf_d = _dev(p_h, gpu), _dev(buf_h, gpu)
+    for s in range(steps):
+        g = _host_grads(1, n, 50 + s)[0]
+        O.sgd_step(p_h, g, buf_h, first_step=(s == 0), **hp)
+        sync.sgd_step(_dev(g, gpu), p_d, buf_d if hp["momentum"] else None, first_step=(s == 0), **hp)
+        torch.cuda.synchronize()
+        ok, err = _close(p_d, p_h, 1e-6, 1e-9)
+        assert ok, f"step {s}: max err {err}"
+        if hp["momentum"]:
+            assert _close(buf_d, buf_h, 1e-6, 2e-9)[0]
+    same, tot = _same_bits(p_d, p_h)
+    print(f"sgd {hp}: {same}/{tot} weights bit-identical after {steps} steps")
+    assert same == tot
+
+
+@pytest.mark.parametrize("hp", [
+    dict(lr=5e-4, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8, adamw=True),
+    dict(lr=2e-3, weight_decay=0.0, betas=(0.9, 0.999), eps=1e-8, adamw=False),
+    dict(lr=1e-3, weight_decay=1e-2, betas=(0.8, 0.99), eps=1e-6, adamw=False),
+])
+def test_adam_steps(gpu, hp):
+    from jabas_amd import sync
+    n, steps = 70001, 5
+    p_h, m_h, v_h = _host_state(n, 3), torch.zeros(n), torch.zeros(n)
+    p_d, m_d, v_d = _dev(p_h, gpu), _dev(m_h, gpu), _dev(v_h, gpu)
+    for s in range(1, steps + 1):
+        g = _host_grads(1, n, 70 + s, std=5e-4)[0]
+        O.adam_step(p_h, g, m_h, v_h, step=s, **hp)
+        sync.adam_step(_dev(g, gpu), p_d, m_d, v_d, step=s, **hp)
+        torch.cuda.synchronize()
+        assert _close(p_d, p_h, 1e-6, 1e-9)[0], f"step {s}"
+        assert _close(m_d, m_h, 1e-6, 2e-10)[0], f"step {s}"
+        assert _close(v_d, v_h, 1e-6, 1e-16)[0], f"step {s}"
+    for name, a, b in (("p", p_d, p_h), ("m", m_d, m_h), ("v", v_d, v_h)):
+        same, tot = _same_bits(a, b)
+        print(f"adam {hp} {name}: {same}/{tot} bit-identical after {steps} steps")
+        assert same == tot
+
+
+# ------------------------------------------------------------------ fused, single bucket
+@pytest.mark.parametrize("K,dtype,opt", [(2, torch.float32, SGD), (4, torch.float32, ADAMW),
+                                         (3, torch.float32, ADAM), (8, torch.bfloat16, ADAMW),
+                                         (5, torch.bfloat16, SGD), (1, torch.float32, ADAM)])
+def test_sync_bucket_fused(gpu, K, dtype, opt):
+    from jabas_amd import sync
+    n = 200003
+    skew = 2 if dtype == torch.bfloat16 else 1
+    bounds = ((0, 1), (5, 0), (1029, 1), (70000, 0), (70001, 1), (150000, 0))
+    hg = _host_grads(K, n, 60 + K, std=5e-4, dtype=dtype)
+    p_h, s1_h, s2_h = _host_state(n, 5), torch.zeros(n), torch.zeros(n)
+    dg = [_dev(t, gpu, skew) for t in hg]
+    agg_d = _dev(torch.zeros(n), gpu, skew)
+    p_d, s1_d, s2_d = _dev(p_h, gpu, skew), _dev(s1_h, gpu, skew), _dev(s2_h, gpu, skew)
+    fan = [_dev(torch.zeros(n), gpu, skew) for _ in range(2)]
+    adam = opt["kind"] != "sgd"
+    span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d, state1=s1_d, state2=s2_d if adam else None, fanout=fan,
+                         bounds=bounds)
+    ws = sync.Workspace(1, gpu)
+    for step in (1, 2, 3):
+        args = sync.make_step_args(BATCHES[K], dtype, stats=True, opt=opt, step=step, first_step=(step == 1))
+        row = sync.sync_bucket(span, args, workspace=ws)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg, BATCHES[K], [(0, n, bounds)], opt, p_h, s1_h, s2_h if adam else None,
+                                    step=step, first_step=(step == 1), want_stats=True)
+        assert torch.equal(_bits(agg_d), _bits(agg_h)), f"step {step}"
+        rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        assert _close(row.cpu()[:4 + K], rows_h[0][:4 + K], rtol, 1e-30)[0]
+        assert _close(p_d, p_h, 1e-6, 1e-9)[0], f"step {step}"
+        assert _close(s1_d, s1_h, 1e-6, 2e-9)[0], f"step {step}"
+        if adam:
+            assert _close(s2_d, s2_h, 1e-6, 1e-16)[0], f"step {step}"
+        for f in fan:
+            assert torch.equal(_bits(f), _bits(p_d))
+    same, tot = _same_bits(p_d, p_h)
+    print(f"fused bucket K={K} {dtype} {opt['kind']}: {same}/{tot} weights bit-identical")
+    assert same == tot
+
+
+# ---------------------------------------------------------------- fused, multi-span plan
+@pytest.mark.parametrize("K,dtype,opt,in_place", [
+    (2, torch.float32, SGD, True), (4, torch.float32, ADAMW, True), (3, torch.float32, SGD, False),
+    (4, torch.float32, ADAM, False), (8, torch.bfloat16, ADAMW, False), (6, torch.float32, None, True),
+    (7, torch.bfloat16, None, False)])
+def test_sync_fused_plan_ragged_spans(gpu, K, dtype, opt, in_place):
+    from jabas_amd import sync, _lib as L
+    # span sizes: tiny, exactly one tile, ragged, empty, large; offsets chosen so that some
+    # spans start off a 16-byte line (all buffers share the offset, as views of one layout do)
+    sizes = [1, 1024, 2048, 0, 4097, 333, 8192 * 3 + 5, 7, 500000, 64, 2048 * 40]
+    gaps = [0, 3, 0, 1, 0, 2, 0, 0, 5, 0, 0]
+    if dtype == torch.bfloat16:
+        gaps = [2 * g for g in gaps]
+    offs, off = [], 0
+    for s, gp in zip(sizes, gaps):
+        off += gp
+        offs.append(off)
+        off += s
+    total = off
+    hg = _host_grads(K, total, 80 + K, std=5e-4, dtype=dtype)
+    p_h, s1_h, s2_h = _host_state(total, 7), torch.zeros(total), torch.zeros(total)
+    dg = [_dev(t, gpu) for t in hg]
+    agg_d = dg[0] if in_place else _dev(torch.zeros(total), gpu)
+    p_d, s1_d, s2_d = _dev(p_h, gpu), _dev(s1_h, gpu), _dev(s2_h, gpu)
+    kind = sync.opt_kind(opt)
+    adam = kind in (L.OPT_ADAM, L.OPT_ADAMW)
+    spans_h, spans_d = [], []
+    for i, (o, s) in enumerate(zip(offs, sizes)):
+        if s > 3000:
+            bounds = ((0, i % 2), (s // 3, 1 - i % 2), (s // 3 + 1, i % 2), (s - 1, 1))
+        elif s > 0:
+            bounds = ((0, i % 2),)
+        else:
+            bounds = ()
+        sl = slice(o, o + s)
+        spans_h.append((o, s, bounds))
+        spans_d.append(sync.SpanSpec([g[sl] for g in dg], agg_out=agg_d[sl],
+                                     param=p_d[sl] if opt else None, state1=s1_d[sl] if opt else None,
+                                     state2=s2_d[sl] if adam else None, bounds=bounds if opt else ()))
+    plan = sync.SyncPlan(spans_d, kind)
+    hg_work = [t.clone() for t in hg]
+    for step in (1, 2):
+        args = sync.make_step_args(BATCHES[K], dtype, stats=True, opt=opt, step=step, first_step=(step == 1))
+        rows = plan.run(args)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg_work, BATCHES[K], spans_h, opt, p_h, s1_h, s2_h if adam else None,
+                                    step=step, first_step=(step == 1), want_stats=True)
+        for (o, s, _), i in zip(spans_h, range(len(spans_h))):
+            assert torch.equal(_bits(agg_d[o:o + s]), _bits(agg_h[o:o + s])), f"span {i} step {step}"
+        rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        ok, err = _close(rows.cpu()[:, :4 + K], rows_h[:, :4 + K], rtol, 1e-30)
+        assert ok, f"stats step {step}: {rows.cpu()} vs {rows_h}"
+        if opt:
+            assert _close(p_d, p_h, 1e-6, 1e-9)[0], f"step {step}"
+            assert _close(s1_d, s1_h, 1e-6, 2e-9)[0]
+            if adam:
+                assert _close(s2_d, s2_h, 1e-6, 1e-16)[0]
+        if in_place:
+            # the next step aggregates what is now in VSW 0's buckets, on both sides
+            for (o, s, _) in spans_h:
+                hg_work[0][o:o + s] = agg_h[o:o + s]
+    # elements in the gaps between spans are never written
+    covered = torch.zeros(total, dtype=torch.bool)
+    for o, s, _ in spans_h:
+        covered[o:o + s] = True
+    if opt:
+        assert torch.equal(_bits(p_d)[~covered], _bits(_host_state(total, 7))[~covered])
+
+
+def test_fused_rejects_bad_arguments(gpu):
+    from jabas_amd import sync, _lib as L
+    n = 4096
+    g = [torch.zeros(n + 8, device=gpu) for _ in range(2)]
+    out = torch.zeros(n + 8, device=gpu)
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.aggregate([g[0][1:n + 1], g[1][:n]], (1, 1), out=out[:n])       # mutually misaligned
+    assert e.value.status == L.ERR_ALIGN
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.aggregate([g[0][:n], g[1][:n]], (1, 1), out=g[0][4:n + 4])      # partial overlap
+    assert e.value.status == L.ERR_ALIAS
+    with pytest.raises(ValueError):
+        sync.aggregate([g[0][:n]] * 9, (1,) * 9)
+    span = sync.SpanSpec([g[0][:n], g[1][:n]], param=None)
+    args = sync.make_step_args((1, 1), torch.float32, opt=SGD)
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.sync_bucket(span, args)                                          # optimizer without weights
+    assert e.value.status == L.ERR_NULL
