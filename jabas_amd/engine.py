@@ -96,10 +96,11 @@ class VSWFlatSync:
 
     def bucket_stats(self, stats):
         """Per-bucket rows from per-span rows (spans of one bucket summed in span order)."""
-        nb = len(self.layout.buckets)
-        idx = torch.tensor(self.span_bucket, device=stats.device)
-        out = torch.zeros(nb, L.STATS_STRIDE, dtype=torch.float64, device=stats.device)
-        return out.index_add_(0, idx, stats)
+        rows = stats.detach().cpu()
+        out = torch.zeros(len(self.layout.buckets), L.STATS_STRIDE, dtype=torch.float64)
+        for i, b in enumerate(self.span_bucket):
+            out[b] += rows[i]
+        return out
 
     @staticmethod
     def cosine(stats):
