@@ -126,13 +126,14 @@ typedef struct JabasStepArgs {
 const char* jabas_sync_version(void);
 const char* jabas_status_string(int status);
 
-/* Bytes of device workspace a fused or statistics call over n_span spans needs
- * (per-block partial sums of the two-level reduction). */
-size_t jabas_sync_workspace_bytes(uint32_t n_span);
+/* Bytes of device workspace a single-span call (jabas_sync_bucket, jabas_stats) over
+ * numel elements needs when statistics are requested: one partial row per workgroup of
+ * the two-level reduction. No reference counterpart. */
+size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype);
 
 /* --- multi-span plan --------------------------------------------------------------
  * A plan is the launch-invariant description of a set of spans (pointer table, tile
- * prefix sums, group bounds). jabas_plan_encode validates the spans and writes the
+ * chunk table, group bounds). jabas_plan_encode validates the spans and writes the
  * blob into host memory; the caller copies the same bytes to the device once and
  * passes both copies to jabas_sync_fused at every step. Pure host code: runs without
  * a GPU.
@@ -140,17 +141,22 @@ size_t jabas_sync_workspace_bytes(uint32_t n_span);
  * step in the reference: jabas/train/trainer.py:327-337 (hook registration per local
  * model), examples/gnmt/seq2seq/train/shard_optimizer.py:40-73 (per-parameter loop
  * matching gradients to parameters by .index). */
-size_t jabas_plan_bytes(uint32_t n_span, uint32_t n_bounds);
+size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds,
+                        int32_t grad_dtype);
 int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span,
                       const JabasBound* bounds, uint32_t n_bounds,
                       int32_t K, int32_t grad_dtype, int32_t opt_kind,
                       void* host_blob, size_t blob_bytes);
-/* Number of 16-byte-line tiles the plan covers (grid sizing, diagnostics). */
-int64_t jabas_plan_tiles(const void* host_blob);
+/* Number of workgroups (chunks) one launch of the plan uses; negative JabasStatus on a
+ * malformed blob. */
+int64_t jabas_plan_chunks(const void* host_blob);
+/* Bytes of device workspace jabas_sync_fused needs for this plan when statistics are
+ * requested (0 on a malformed blob). */
+size_t jabas_plan_workspace_bytes(const void* host_blob);
 
 /* --- the fused sync step ------------------------------------------------------------
  * Aggregate + statistics + optimizer (+ fan-out) over every span of a plan, one
- * launch (plus a one-block-per-span finalize launch when args->stats is set).
+ * launch (plus a one-workgroup-per-span finalize launch when args->stats is set).
  * stats_out: n_span * JABAS_STATS_STRIDE doubles (device), required when stats != 0.
  * Replaces, for one GPU:
  *   - the local aggregation of the K VSW buckets inside IIDPTrainer.compute()/step()
@@ -169,9 +175,10 @@ int jabas_sync_fused(const void* plan_host, const void* plan_dev,
                      void* workspace, size_t workspace_bytes, jabas_stream_t stream);
 
 /* The same step over ONE span passed by value (no plan, no device table): what a
- * comm hook calls for the bucket it was handed. bounds_dev is a device array of
- * span->bound_count entries starting at span->bound_begin, or NULL when
- * bound_count == 0. stats_out: JABAS_STATS_STRIDE doubles or NULL.
+ * comm hook calls for the bucket it was handed. bounds_dev is a device array holding
+ * the span's bound_count entries (span->bound_begin is ignored), or NULL when
+ * bound_count == 0; its contents cannot be checked on the host and must obey the
+ * JabasBound rules. stats_out: JABAS_STATS_STRIDE doubles or NULL.
  * Replaces hook_with_allreduce for one bucket
  * (jabas/ddp_comm_hooks/similarity_allreduce.py:38-45) and, with an optimizer kind,
  * the optimizer hook of the overlap weight-sync mode (jabas/train/trainer.py:327-333). */

@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libjabas_sync.so")
+# JABAS_SYNC_LIB points at another build of the same library (kernel tuning experiments)
+LIB_PATH = os.environ.get("JABAS_SYNC_LIB") or os.path.join(_HERE, "csrc", "libjabas_sync.so")
 
 MAX_K = 8
 MAX_GROUPS = 16
@@ -74,11 +75,12 @@ class JabasStepArgs(C.Structure):
 SIGNATURES = {
     "jabas_sync_version": (C.c_char_p, []),
     "jabas_status_string": (C.c_char_p, [C.c_int]),
-    "jabas_sync_workspace_bytes": (C.c_size_t, [C.c_uint32]),
-    "jabas_plan_bytes": (C.c_size_t, [C.c_uint32, C.c_uint32]),
+    "jabas_sync_workspace_bytes": (C.c_size_t, [C.c_uint64, C.c_int32]),
+    "jabas_plan_bytes": (C.c_size_t, [C.POINTER(JabasSpan), C.c_uint32, C.c_uint32, C.c_int32]),
     "jabas_plan_encode": (C.c_int, [C.POINTER(JabasSpan), C.c_uint32, C.POINTER(JabasBound), C.c_uint32,
                                     C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_size_t]),
-    "jabas_plan_tiles": (C.c_int64, [C.c_void_p]),
+    "jabas_plan_chunks": (C.c_int64, [C.c_void_p]),
+    "jabas_plan_workspace_bytes": (C.c_size_t, [C.c_void_p]),
     "jabas_sync_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(JabasStepArgs), C.c_void_p,
                                    C.c_void_p, C.c_size_t, C.c_void_p]),
     "jabas_sync_bucket": (C.c_int, [C.POINTER(JabasSpan), C.c_void_p, C.POINTER(JabasStepArgs), C.c_void_p,

@@ -15,19 +15,20 @@ int launch_gram_finalize(int K, const double* partials, unsigned grid, double* g
 
 namespace {
 
+constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 1;
+constexpr uint32_t kPlanVersion = 2;
 
 struct PlanHeader {
     uint32_t magic, version;
-    uint32_t n_span, n_bounds, n_tiles;
+    uint32_t n_span, n_bounds, n_chunks;
     int32_t K, grad_dtype, opt_kind;
     uint32_t max_group;       // largest group index any bound names
-    uint32_t all_have_s1;     // every span carries a state1 pointer
-    uint64_t off_spans, off_prefix, off_bounds, total_bytes;
+    uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
+    uint64_t off_spans, off_prefix, off_chunks, off_bounds, total_bytes;
 };
-static_assert(sizeof(PlanHeader) == 72, "plan header layout");
-constexpr size_t kHeaderBytes = 80;
+static_assert(sizeof(PlanHeader) == 80, "plan header layout");
+constexpr size_t kHeaderBytes = 96;
 
 inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
 
@@ -45,6 +46,16 @@ inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
     const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
     return a0 < b0 + nb && b0 < a0 + na;
 }
+
+// Tiles a span occupies, counted from the 16-byte line its first element falls in.
+inline uint64_t span_tiles(const JabasSpan& in, int grad_dtype) {
+    if (in.numel == 0) return 0;
+    const int gs = grad_dtype == JABAS_BF16 ? 2 : 4;
+    const uint64_t skew = (reinterpret_cast<uintptr_t>(in.grads[0]) / gs) % ept_of(grad_dtype);
+    const uint64_t te = tile_elems(grad_dtype);
+    return (skew + in.numel + te - 1) / te;
+}
+inline uint64_t chunks_of_tiles(uint64_t tiles) { return (tiles + kChunkTiles - 1) / kChunkTiles; }
 
 // Validates one span and produces the rebased device view. Host-only logic.
 int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDev* out, uint32_t* tiles) {
@@ -177,67 +188,37 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
     return JABAS_OK;
 }
 
-int cu_count() {
-    static int cache[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    if (cache[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
-        cache[dev] = n;
-    }
-    return cache[dev];
-}
-
 typedef int (*LaunchFn)(int, int, int, const KArgs&, unsigned, hipStream_t);
-typedef int (*OccFn)(int, int, int);
 const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_fused_k3, launch_fused_k4,
                                        launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
-const OccFn kOcc[JABAS_MAX_K] = {occupancy_k1, occupancy_k2, occupancy_k3, occupancy_k4,
-                                 occupancy_k5, occupancy_k6, occupancy_k7, occupancy_k8};
 
-unsigned pick_grid(int K, int grad_dtype, int oc, int stats, uint32_t n_tiles) {
-    const int occ = kOcc[K - 1](grad_dtype, oc, stats);
-    uint64_t g = static_cast<uint64_t>(cu_count()) * static_cast<uint64_t>(occ);
-    if (g > static_cast<uint64_t>(kMaxGrid)) g = kMaxGrid;
-    if (g > n_tiles) g = n_tiles;
-    if (g < 1) g = 1;
-    return static_cast<unsigned>(g);
-}
-
-// Second level of the statistics reduction: one wave per span sums, in increasing
-// workgroup order, the partial rows the workgroups that touched the span left behind.
-__global__ void __launch_bounds__(64) finalize_stats_kernel(const uint32_t* tile_prefix, uint32_t n_tiles,
-                                                            uint32_t use_inline, uint32_t grid, int ns,
-                                                            const double* partials, double* stats_out) {
-    const uint32_t s = blockIdx.x, lane = threadIdx.x;
-    uint32_t ts0 = 0, ts1 = n_tiles;
-    if (!use_inline) { ts0 = tile_prefix[s]; ts1 = tile_prefix[s + 1]; }
+// Second level of the statistics reduction: one workgroup per span sums the partial rows
+// of the span's chunks. Thread t adds rows t, t+256, ... in increasing order, then the 256
+// per-thread sums are added in thread order: a fixed tree, independent of the machine.
+constexpr int kFinalizeBlock = 256;
+__global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
+                                                                        uint32_t use_inline, int ns,
+                                                                        const double* partials, double* stats_out) {
+    __shared__ double red[kStatsStride][kFinalizeBlock + 1];
+    const uint32_t s = blockIdx.x, t = threadIdx.x;
+    uint32_t c0 = 0, c1 = n_chunks;
+    if (!use_inline) { c0 = chunk_prefix[s]; c1 = chunk_prefix[s + 1]; }
     double acc[kStatsStride];
 #pragma unroll
     for (int i = 0; i < kStatsStride; ++i) acc[i] = 0.0;
-    if (ts1 > ts0) {
-        // workgroup b owns tiles [b*T/G, (b+1)*T/G): owner(t) = ((t+1)*G - 1) / T
-        const uint64_t T = n_tiles, G = grid;
-        const uint32_t b_lo = static_cast<uint32_t>(((static_cast<uint64_t>(ts0) + 1) * G - 1) / T);
-        const uint32_t b_hi = static_cast<uint32_t>((static_cast<uint64_t>(ts1) * G - 1) / T);
-        for (uint32_t b = b_lo + lane; b <= b_hi; b += 64) {
-            const double* row = partials + static_cast<uint64_t>(b + s) * kStatsStride;
+    for (uint32_t c = c0 + t; c < c1; c += kFinalizeBlock) {
+        const double* row = partials + static_cast<uint64_t>(c) * kStatsStride;
 #pragma unroll
-            for (int i = 0; i < kStatsStride; ++i)
-                if (i < ns) acc[i] += row[i];
-        }
+        for (int i = 0; i < kStatsStride; ++i)
+            if (i < ns) acc[i] += row[i];
     }
 #pragma unroll
-    for (int i = 0; i < kStatsStride; ++i) {
-        double v = acc[i];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-        acc[i] = v;
-    }
-    if (lane == 0) {
-#pragma unroll
-        for (int i = 0; i < kStatsStride; ++i) stats_out[static_cast<uint64_t>(s) * kStatsStride + i] = acc[i];
+    for (int i = 0; i < kStatsStride; ++i) red[i][t] = acc[i];
+    __syncthreads();
+    if (t < kStatsStride) {
+        double sum = 0.0;
+        for (int j = 0; j < kFinalizeBlock; ++j) sum += red[t][j];
+        stats_out[static_cast<uint64_t>(s) * kStatsStride + t] = sum;
     }
 }
 
@@ -248,19 +229,17 @@ int run_fused(KArgs& a, const JabasStepArgs* s, double* stats_out, void* workspa
     if (stats) {
         if (!stats_out) return JABAS_ERR_NULL;
         if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
-        if (workspace_bytes < jabas_sync_workspace_bytes(a.n_span)) return JABAS_ERR_WORKSPACE;
+        if (workspace_bytes < static_cast<size_t>(a.n_chunks) * kStatsStride * sizeof(double)) return JABAS_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(stats_out) % 8) return JABAS_ERR_ALIGN;
     }
     a.partials = static_cast<double*>(workspace);
-    unsigned grid = 0;
-    if (a.n_tiles) {
-        grid = pick_grid(s->K, s->grad_dtype, oc, stats, a.n_tiles);
-        const int err = kLaunch[s->K - 1](s->grad_dtype, oc, stats, a, grid, stream);
+    if (a.n_chunks) {
+        const int err = kLaunch[s->K - 1](s->grad_dtype, oc, stats, a, a.n_chunks, stream);
         if (err != 0) return JABAS_ERR_LAUNCH;
     }
     if (stats) {
-        hipLaunchKernelGGL(finalize_stats_kernel, dim3(a.n_span), dim3(64), 0, stream, a.tile_prefix, a.n_tiles,
-                           a.use_inline, grid ? grid : 1u, 4 + s->K, a.partials, stats_out);
+        hipLaunchKernelGGL(finalize_stats_kernel, dim3(a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
+                           a.n_chunks, a.use_inline, 4 + s->K, a.partials, stats_out);
         if (hipGetLastError() != hipSuccess) return JABAS_ERR_LAUNCH;
     }
     return JABAS_OK;
@@ -291,14 +270,31 @@ JABAS_API const char* jabas_status_string(int status) {
     }
 }
 
-JABAS_API size_t jabas_sync_workspace_bytes(uint32_t n_span) {
-    return (static_cast<size_t>(kMaxGrid) + n_span) * kStatsStride * sizeof(double);
+JABAS_API size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype) {
+    // chunks of a single span whose first element may sit anywhere in a 16-byte line
+    const int dt = grad_dtype == JABAS_BF16 ? JABAS_BF16 : JABAS_F32;
+    const uint64_t te = tile_elems(dt);
+    const uint64_t tiles = (numel + ept_of(dt) - 1 + te - 1) / te;
+    return static_cast<size_t>(chunks_of_tiles(tiles) + 1) * kStatsStride * sizeof(double);
 }
 
-JABAS_API size_t jabas_plan_bytes(uint32_t n_span, uint32_t n_bounds) {
+namespace {
+uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype) {
+    uint64_t n = 0;
+    for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype));
+    return n;
+}
+size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
     return kHeaderBytes + align16(static_cast<size_t>(n_span) * sizeof(SpanDev)) +
            align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t)) +
+           align16(static_cast<size_t>(n_chunks) * sizeof(ChunkDesc)) +
            align16(static_cast<size_t>(n_bounds) * sizeof(BoundDev));
+}
+}  // namespace
+
+JABAS_API size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds, int32_t grad_dtype) {
+    if (!spans || (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16)) return 0;
+    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype));
 }
 
 JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
@@ -311,29 +307,38 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
     if (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
     if (opt_class_of(opt_kind) < 0) return JABAS_ERR_OPT;
-    if (blob_bytes < jabas_plan_bytes(n_span, n_bounds)) return JABAS_ERR_PLAN;
+    for (uint32_t i = 0; i < n_span; ++i)
+        if (spans[i].numel && !spans[i].grads[0]) return JABAS_ERR_NULL;
+    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype);
+    if (n_chunks > 0x7fffffffull) return JABAS_ERR_SIZE;
+    const size_t need = plan_bytes_for(n_span, n_bounds, n_chunks);
+    if (blob_bytes < need) return JABAS_ERR_PLAN;
     if (reinterpret_cast<uintptr_t>(host_blob) % 8) return JABAS_ERR_ALIGN;
 
     char* base = static_cast<char*>(host_blob);
-    memset(base, 0, jabas_plan_bytes(n_span, n_bounds));
+    memset(base, 0, need);
     PlanHeader h;
     memset(&h, 0, sizeof(h));
     h.magic = kPlanMagic;
     h.version = kPlanVersion;
     h.n_span = n_span;
     h.n_bounds = n_bounds;
+    h.n_chunks = static_cast<uint32_t>(n_chunks);
     h.K = K;
     h.grad_dtype = grad_dtype;
     h.opt_kind = opt_kind;
     h.off_spans = kHeaderBytes;
     h.off_prefix = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
-    h.off_bounds = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
-    h.total_bytes = jabas_plan_bytes(n_span, n_bounds);
+    h.off_chunks = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
+    h.off_bounds = h.off_chunks + align16(static_cast<size_t>(n_chunks) * sizeof(ChunkDesc));
+    h.total_bytes = need;
     h.all_have_s1 = 1;
 
     SpanDev* sd = reinterpret_cast<SpanDev*>(base + h.off_spans);
     uint32_t* prefix = reinterpret_cast<uint32_t*>(base + h.off_prefix);
-    uint64_t total = 0;
+    ChunkDesc* cd = reinterpret_cast<ChunkDesc*>(base + h.off_chunks);
+    const uint64_t te = tile_elems(grad_dtype);
+    uint32_t c = 0;
     for (uint32_t i = 0; i < n_span; ++i) {
         uint32_t tiles = 0;
         int rc = encode_span(spans[i], K, grad_dtype, opt_kind, &sd[i], &tiles);
@@ -341,23 +346,38 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
         rc = check_bounds_host(spans[i], bounds, n_bounds, &h.max_group);
         if (rc != JABAS_OK) return rc;
         if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
-        prefix[i] = static_cast<uint32_t>(total);
-        total += tiles;
-        if (total > 0x7fffffffull) return JABAS_ERR_SIZE;
+        prefix[i] = c;
+        uint32_t j = 0;
+        for (uint32_t t0 = 0; t0 < tiles; t0 += kChunkTiles, ++c) {
+            cd[c].span = i;
+            cd[c].tile0 = t0;
+            if (spans[i].bound_count) {       // bound entry covering the chunk's first live element
+                const uint64_t e0 = static_cast<uint64_t>(t0) * te;
+                const uint64_t rel = (e0 > sd[i].lo ? e0 : sd[i].lo) - sd[i].lo;
+                const JabasBound* b = bounds + spans[i].bound_begin;
+                while (j + 1 < spans[i].bound_count && b[j + 1].start <= rel) ++j;
+            }
+            cd[c].bound0 = j;
+        }
     }
-    prefix[n_span] = static_cast<uint32_t>(total);
-    h.n_tiles = static_cast<uint32_t>(total);
+    prefix[n_span] = c;
+    if (c != h.n_chunks) return JABAS_ERR_PLAN;
     if (n_bounds) memcpy(base + h.off_bounds, bounds, static_cast<size_t>(n_bounds) * sizeof(JabasBound));
     memcpy(base, &h, sizeof(h));
     return JABAS_OK;
 }
 
-JABAS_API int64_t jabas_plan_tiles(const void* host_blob) {
+JABAS_API int64_t jabas_plan_chunks(const void* host_blob) {
     if (!host_blob) return JABAS_ERR_NULL;
     PlanHeader h;
     memcpy(&h, host_blob, sizeof(h));
     if (h.magic != kPlanMagic || h.version != kPlanVersion) return JABAS_ERR_PLAN;
-    return h.n_tiles;
+    return h.n_chunks;
+}
+
+JABAS_API size_t jabas_plan_workspace_bytes(const void* host_blob) {
+    const int64_t n = jabas_plan_chunks(host_blob);
+    return n < 0 ? 0 : static_cast<size_t>(n + 1) * kStatsStride * sizeof(double);
 }
 
 JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, const JabasStepArgs* args,
@@ -380,10 +400,11 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     }
     const char* dev = static_cast<const char*>(plan_dev);
     a.spans = reinterpret_cast<const SpanDev*>(dev + h.off_spans);
-    a.tile_prefix = reinterpret_cast<const uint32_t*>(dev + h.off_prefix);
+    a.chunk_prefix = reinterpret_cast<const uint32_t*>(dev + h.off_prefix);
+    a.chunks = reinterpret_cast<const ChunkDesc*>(dev + h.off_chunks);
     a.bounds = h.n_bounds ? reinterpret_cast<const BoundDev*>(dev + h.off_bounds) : nullptr;
     a.n_span = h.n_span;
-    a.n_tiles = h.n_tiles;
+    a.n_chunks = h.n_chunks;
     a.use_inline = 0;
     return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
@@ -405,9 +426,10 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.span0.bound_begin = 0;
     a.bounds = reinterpret_cast<const BoundDev*>(bounds_dev);
     a.spans = nullptr;
-    a.tile_prefix = nullptr;
+    a.chunks = nullptr;
+    a.chunk_prefix = nullptr;
     a.n_span = 1;
-    a.n_tiles = tiles;
+    a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles));
     a.use_inline = 1;
     return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
@@ -467,10 +489,9 @@ JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype
     uint32_t tiles = 0;
     const int rc = encode_span(sp, K, grad_dtype, JABAS_OPT_NONE, &sd, &tiles);
     if (rc != JABAS_OK) return rc;
-    uint64_t g = static_cast<uint64_t>(cu_count()) * 4;
+    uint64_t g = kGramGrid;
     if (g > tiles) g = tiles;
     if (g < 1) g = 1;
-    if (g > static_cast<uint64_t>(kMaxGrid)) g = kMaxGrid;
     if (workspace_bytes < g * JABAS_GRAM_STRIDE * sizeof(double)) return JABAS_ERR_WORKSPACE;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (launch_gram(K, grad_dtype, sd, static_cast<double*>(workspace), static_cast<unsigned>(g), st) != 0)

@@ -3,15 +3,19 @@
 // streams are fully unrolled into independent 128-bit loads.
 //
 // Execution shape
-//   - persistent grid of 256-thread workgroups (4 wave64); workgroup b owns the
-//     contiguous tile range [b*T/G, (b+1)*T/G) of the launch, T = tiles, G = gridDim.x;
-//   - a tile is 256 threads x one 16-byte gradient vector (4 fp32 or 8 bf16 elements);
+//   - one 256-thread workgroup (4 wave64) per chunk of kChunkTiles consecutive tiles of
+//     one span; a tile is 256 threads x one 16-byte gradient vector (4 fp32 or 8 bf16
+//     elements). Small, short-lived workgroups dispatched in order keep the part of every
+//     buffer that is being streamed at any moment compact, which on MI355X sustains a
+//     markedly higher HBM rate than a persistent grid that spreads over the whole buffers;
+//   - every global access is a 128-bit vector access with the nontemporal hint (each byte
+//     is touched exactly once per step);
 //   - tiles that lie wholly inside the live range of a span and inside one parameter
 //     group take the vector path (all loads of U tiles issued before any arithmetic);
 //     the few tiles that straddle a span end or a group change take a scalar path;
-//   - statistics: per-thread fp64 accumulators -> wave64 shuffle tree -> LDS across
-//     the 4 waves -> one partial row per (workgroup, span) in the workspace, summed in
-//     fixed order by the finalize kernel. Same grid => same bits, run to run.
+//   - statistics: per-thread fp64 accumulators -> wave64 DPP tree -> LDS across the
+//     4 waves -> one partial row per workgroup in the workspace, summed in fixed order by
+//     the finalize kernel. The tree is fixed, so results are bit-identical run to run.
 //
 // Arithmetic is compiled with -ffp-contract=off: every fp32 product and sum of the
 // aggregate and of the optimizer formulas is rounded on its own, so results can be
@@ -135,13 +139,13 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
 
 template <int NV> __device__ __forceinline__ void load_vec(f32x4 (&r)[NV], const float* base, uint64_t e) {
 #pragma unroll
-    for (int v = 0; v < NV; ++v) r[v] = *reinterpret_cast<const f32x4*>(base + e + 4 * v);
+    for (int v = 0; v < NV; ++v) r[v] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + e + 4 * v));
 }
 template <int NV> __device__ __forceinline__ void store_vec(const float (&x)[4 * NV], float* base, uint64_t e) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         f32x4 r = {x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
-        *reinterpret_cast<f32x4*>(base + e + 4 * v) = r;
+        __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(base + e + 4 * v));
     }
 }
 template <int NV> __device__ __forceinline__ void unpack_vec(const f32x4 (&r)[NV], float (&x)[4 * NV]) {
@@ -149,44 +153,54 @@ template <int NV> __device__ __forceinline__ void unpack_vec(const f32x4 (&r)[NV
     for (int v = 0; v < NV; ++v) { x[4 * v] = r[v].x; x[4 * v + 1] = r[v].y; x[4 * v + 2] = r[v].z; x[4 * v + 3] = r[v].w; }
 }
 
-// Vector path over U consecutive full tiles of one parameter group. e is the (rebased)
-// index of this thread's first element in the first tile.
-template <int K, int DT, int OPT, bool STATS, int U>
-__device__ __forceinline__ void fast_tiles(const SpanDev& sp, uint64_t e, const KArgs& a, const GroupDev& G,
-                                           double (&acc)[NStats<K, STATS>::value]) {
+// Registers of U consecutive full tiles: the raw 16-byte vectors as loaded.
+template <int K, int DT, int U> struct TileRegs {
+    typename Grad<DT>::Raw g[U][K];
+    f32x4 p[U][Grad<DT>::EPT / 4], s1[U][Grad<DT>::EPT / 4], s2[U][Grad<DT>::EPT / 4];
+};
+
+// Issues every load of U consecutive full tiles. e is the (rebased) index of this
+// thread's first element in the first tile.
+template <int K, int DT, int OPT, int U>
+__device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
-    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
-    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
-
-    typename GR::Raw rg[U][K];
-    f32x4 rp[U][NV], r1[U][NV], r2[U][NV];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
 #pragma unroll
-        for (int k = 0; k < K; ++k) rg[u][k] = GR::load(sp.g[k], eu);
+        for (int k = 0; k < K; ++k) r.g[u][k] = GR::load(sp.g[k], eu);
         if constexpr (OPT != OPT_NONE) {
-            load_vec<NV>(rp[u], sp.p, eu);
-            if (load_s1) load_vec<NV>(r1[u], sp.s1, eu);
-            if constexpr (OPT == OPT_ADAM) load_vec<NV>(r2[u], sp.s2, eu);
+            load_vec<NV>(r.p[u], sp.p, eu);
+            if (load_s1) load_vec<NV>(r.s1[u], sp.s1, eu);
+            if constexpr (OPT == OPT_ADAM) load_vec<NV>(r.s2[u], sp.s2, eu);
         }
     }
+}
+
+// Arithmetic and stores of U tiles whose loads were issued by issue_loads.
+template <int K, int DT, int OPT, bool STATS, int U>
+__device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const KArgs& a,
+                                        const GroupDev& G, bool use_s1, bool load_s1,
+                                        double (&acc)[NStats<K, STATS>::value]) {
+    using GR = Grad<DT>;
+    constexpr int EPT = GR::EPT, NV = EPT / 4;
+    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
         float g[K][EPT], p[EPT], s1[EPT], s2[EPT], agg[EPT];
 #pragma unroll
-        for (int k = 0; k < K; ++k) GR::widen(rg[u][k], g[k]);
+        for (int k = 0; k < K; ++k) GR::widen(r.g[u][k], g[k]);
         if constexpr (OPT != OPT_NONE) {
-            unpack_vec<NV>(rp[u], p);
-            if (load_s1) unpack_vec<NV>(r1[u], s1);
+            unpack_vec<NV>(r.p[u], p);
+            if (load_s1) unpack_vec<NV>(r.s1[u], s1);
             else {
 #pragma unroll
                 for (int i = 0; i < EPT; ++i) s1[i] = 0.0f;
             }
-            if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r2[u], s2);
+            if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r.s2[u], s2);
         }
         compute<K, EPT, OPT, STATS>(g, p, s1, s2, agg, a, G, acc);
         if (sp.out) store_vec<NV>(agg, sp.out, eu);
@@ -194,7 +208,29 @@ __device__ __forceinline__ void fast_tiles(const SpanDev& sp, uint64_t e, const 
             store_vec<NV>(p, sp.p, eu);
             if (use_s1) store_vec<NV>(s1, sp.s1, eu);
             if constexpr (OPT == OPT_ADAM) store_vec<NV>(s2, sp.s2, eu);
-            for (uint32_t r = 0; r < sp.n_fan; ++r) store_vec<NV>(p, sp.fan[r], eu);
+            for (uint32_t f = 0; f < sp.n_fan; ++f) store_vec<NV>(p, sp.fan[f], eu);
+        }
+    }
+}
+
+// Vector path over nfull consecutive full tiles of one parameter group.
+template <int K, int DT, int OPT, bool STATS, int U>
+__device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
+                                         const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
+    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
+    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
+    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
+    uint32_t i = 0;
+    for (; i + U <= nfull; i += U, e += U * TE) {
+        TileRegs<K, DT, U> r;
+        issue_loads<K, DT, OPT, U>(r, sp, e, load_s1);
+        consume<K, DT, OPT, STATS, U>(r, sp, e, a, G, use_s1, load_s1, acc);
+    }
+    if constexpr (U > 1) {
+        for (; i < nfull; ++i, e += TE) {
+            TileRegs<K, DT, 1> r;
+            issue_loads<K, DT, OPT, 1>(r, sp, e, load_s1);
+            consume<K, DT, OPT, STATS, 1>(r, sp, e, a, G, use_s1, load_s1, acc);
         }
     }
 }
@@ -243,15 +279,15 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 
 // Tiles [lt0, lt1) of one span (tile indices local to the span).
 template <int K, int DT, int OPT, bool STATS>
-__device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, const KArgs& a,
-                                           double (&acc)[NStats<K, STATS>::value]) {
+__device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
+                                           const KArgs& a, double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
     constexpr int U = (DT == JABAS_BF16) ? JABAS_UNROLL_BF16 : JABAS_UNROLL_F32;
     const uint32_t nb = sp.bound_count;
     const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
-    uint32_t lt = lt0, j = 0;
+    uint32_t lt = lt0, j = j0;
     while (lt < lt1) {
         const uint64_t e0 = static_cast<uint64_t>(lt) * TE;
         const uint64_t cur = e0 > sp.lo ? e0 : sp.lo;
@@ -271,12 +307,7 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
         }
         if (nfull) {
             const GroupDev G = a.groups[gid];
-            uint64_t e = e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
-            uint32_t i = 0;
-            for (; i + U <= nfull; i += U, e += U * TE) fast_tiles<K, DT, OPT, STATS, U>(sp, e, a, G, acc);
-            if constexpr (U > 1) {
-                for (; i < nfull; ++i, e += TE) fast_tiles<K, DT, OPT, STATS, 1>(sp, e, a, G, acc);
-            }
+            fast_run<K, DT, OPT, STATS, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, acc);
             lt += nfull;
         } else {
             careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, acc);
@@ -285,17 +316,34 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     }
 }
 
+// Sum over the 64 lanes of a wave with DPP moves (no LDS traffic); the total lands in
+// lane 63. Pairing order is fixed: lane^1, lane^2, mirror within 8, mirror within 16,
+// row 0->1 and 2->3, rows 0..1 -> 2..3.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double wave_sum_to_lane63(double v) {
+    v += dpp_move<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(v);   // row_half_mirror
+    v += dpp_move<0x140, 0xf>(v);   // row_mirror
+    v += dpp_move<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_move<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
 template <int NS>
 __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
     __shared__ double red[kWaves][NS];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
-        double v = acc[i];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-        if (lane == 0) red[wave][i] = v;
-        acc[i] = 0.0;
+        const double v = wave_sum_to_lane63(acc[i]);
+        if (lane == 63) red[wave][i] = v;
     }
     __syncthreads();
     if (threadIdx.x < NS) {
@@ -304,55 +352,49 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
         for (int w = 1; w < kWaves; ++w) s += red[w][threadIdx.x];
         row[threadIdx.x] = s;
     }
-    __syncthreads();
 }
 
 template <int K, int DT, int OPT, bool STATS>
 __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
     constexpr int NS = NStats<K, STATS>::value;
-    const uint32_t G = gridDim.x, b = blockIdx.x;
-    uint32_t t = static_cast<uint32_t>(static_cast<uint64_t>(b) * a.n_tiles / G);
-    const uint32_t t1 = static_cast<uint32_t>(static_cast<uint64_t>(b + 1) * a.n_tiles / G);
-    uint32_t s = 0;
-    if (!a.use_inline) {                      // largest s with tile_prefix[s] <= t
-        uint32_t lo = 0, hi = a.n_span;       // invariant: prefix[lo] <= t < prefix[hi]
-        while (hi - lo > 1) {
-            const uint32_t mid = (lo + hi) >> 1;
-            if (a.tile_prefix[mid] <= t) lo = mid; else hi = mid;
-        }
-        s = lo;
-    }
+    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
+    const uint32_t b = blockIdx.x;
     double acc[NS];
 #pragma unroll
     for (int i = 0; i < NS; ++i) acc[i] = 0.0;
 
-    while (t < t1) {
-        uint32_t ts0 = 0, ts1 = a.n_tiles;
-        if (!a.use_inline) { ts0 = a.tile_prefix[s]; ts1 = a.tile_prefix[s + 1]; }
-        const uint32_t te = t1 < ts1 ? t1 : ts1;
-        if (te > t) {
-            if (a.use_inline) span_range<K, DT, OPT, STATS>(a.span0, t - ts0, te - ts0, a, acc);
-            else span_range<K, DT, OPT, STATS>(a.spans[s], t - ts0, te - ts0, a, acc);
-            if constexpr (STATS)
-                flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b + s) * kStatsStride);
+    if (a.use_inline) {
+        const SpanDev& sp = a.span0;
+        const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
+        const uint32_t lt0 = b * kChunkTiles;
+        const uint32_t lt1 = lt0 + kChunkTiles < tiles ? lt0 + kChunkTiles : tiles;
+        uint32_t j0 = 0;
+        if (sp.bound_count) {                  // largest j with bounds[j].start <= first live element
+            const BoundDev* bd = a.bounds + sp.bound_begin;
+            const uint64_t e0 = static_cast<uint64_t>(lt0) * TE;
+            const uint64_t rel = (e0 > sp.lo ? e0 : sp.lo) - sp.lo;
+            uint32_t lo = 0, hi = sp.bound_count;
+            while (hi - lo > 1) {
+                const uint32_t mid = (lo + hi) >> 1;
+                if (bd[mid].start <= rel) lo = mid; else hi = mid;
+            }
+            j0 = lo;
         }
-        t = te;
-        ++s;
+        span_range<K, DT, OPT, STATS>(sp, lt0, lt1, j0, a, acc);
+    } else {
+        const ChunkDesc c = a.chunks[b];
+        const SpanDev& sp = a.spans[c.span];
+        const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
+        const uint32_t lt1 = c.tile0 + kChunkTiles < tiles ? c.tile0 + kChunkTiles : tiles;
+        span_range<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
+    if constexpr (STATS) flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);
 }
 
 template <int K, int DT, int OPT, bool STATS>
 int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
     hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(kBlock), 0, stream, a);
     return static_cast<int>(hipGetLastError());
-}
-
-template <int K, int DT, int OPT, bool STATS>
-int occupancy_one() {
-    int n = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fused_kernel<K, DT, OPT, STATS>, kBlock, 0) != hipSuccess || n < 1)
-        n = 2;
-    return n;
 }
 
 }  // namespace
@@ -381,17 +423,6 @@ int occupancy_one() {
 int JABAS_CAT(launch_fused_k, JABAS_K)(int grad_dtype, int opt_class, int stats, const KArgs& a,
                                        unsigned grid, hipStream_t stream) {
     JABAS_DISPATCH(launch_one, a, grid, stream)
-}
-
-int JABAS_CAT(occupancy_k, JABAS_K)(int grad_dtype, int opt_class, int stats) {
-    static int cache[12] = {0};
-    const int k = (grad_dtype == JABAS_BF16 ? 6 : 0) + opt_class * 2 + (stats ? 1 : 0);
-    if (k < 0 || k >= 12) return 1;
-    if (cache[k] == 0) {
-        auto query = [&]() -> int { JABAS_DISPATCH(occupancy_one) };
-        cache[k] = query();
-    }
-    return cache[k];
 }
 
 }  // namespace jabas

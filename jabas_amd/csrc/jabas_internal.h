@@ -10,12 +10,13 @@ namespace jabas {
 
 constexpr int kBlock = 256;                 // threads per workgroup = 4 wave64
 constexpr int kWaves = kBlock / 64;
-constexpr int kMaxGrid = 4096;              // upper bound of persistent workgroups
+constexpr int kChunkTiles = 4;              // tiles one workgroup processes (a "chunk")
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
 // Elements one thread handles per tile: one 16-byte gradient vector.
 __host__ __device__ constexpr int ept_of(int grad_dtype) { return grad_dtype == JABAS_BF16 ? 8 : 4; }
 __host__ __device__ constexpr int tile_elems(int grad_dtype) { return kBlock * ept_of(grad_dtype); }
+__host__ __device__ constexpr int chunk_elems(int grad_dtype) { return kChunkTiles * tile_elems(grad_dtype); }
 
 // A span as the kernels see it. Pointers are rebased downwards by `lo` elements so that
 // element index 0 of every buffer is 16-byte aligned; [lo, hi) is the live range.
@@ -56,14 +57,23 @@ struct OptDev {
     int32_t has_momentum, first_step, nesterov, adamw;
 };
 
+// One workgroup's share of a planned launch: kChunkTiles consecutive tiles of one span.
+struct ChunkDesc {
+    uint32_t span;                           // index into the span table
+    uint32_t tile0;                          // first tile, local to the span
+    uint32_t bound0;                         // bound entry (local to the span) covering the chunk's first live element
+    uint32_t pad;
+};
+
 struct KArgs {
-    const SpanDev* spans;                    // device table (n_span > 1 or planned launch)
-    const uint32_t* tile_prefix;             // n_span + 1 entries, device
+    const SpanDev* spans;                    // device table (planned launch)
+    const ChunkDesc* chunks;                 // one per workgroup (planned launch)
+    const uint32_t* chunk_prefix;            // n_span + 1 entries: first chunk of each span (planned launch)
     const BoundDev* bounds;                  // device, may be NULL
-    double* partials;                        // (grid + n_span) * kStatsStride doubles
+    double* partials;                        // one row of kStatsStride doubles per workgroup
     uint32_t n_span;
-    uint32_t n_tiles;
-    uint32_t use_inline;                     // 1: the only span is `span0`
+    uint32_t n_chunks;
+    uint32_t use_inline;                     // 1: the only span is `span0`, chunk b starts at tile b*kChunkTiles
     uint32_t half_mask;                      // bit k set: VSW k belongs to half B
     SpanDev span0;
     float w[JABAS_MAX_K];
@@ -76,8 +86,7 @@ struct KArgs {
 // opt_class: 0 none, 1 SGD, 2 Adam/AdamW. Returns hipError_t as int.
 #define JABAS_DECLARE_K(k)                                                                   \
     int launch_fused_k##k(int grad_dtype, int opt_class, int stats, const KArgs& a,          \
-                          unsigned grid, hipStream_t stream);                                \
-    int occupancy_k##k(int grad_dtype, int opt_class, int stats);
+                          unsigned grid, hipStream_t stream);
 JABAS_DECLARE_K(1) JABAS_DECLARE_K(2) JABAS_DECLARE_K(3) JABAS_DECLARE_K(4)
 JABAS_DECLARE_K(5) JABAS_DECLARE_K(6) JABAS_DECLARE_K(7) JABAS_DECLARE_K(8)
 #undef JABAS_DECLARE_K

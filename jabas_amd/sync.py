@@ -177,13 +177,19 @@ def _stream_ptr(stream=None):
 
 
 class Workspace:
-    """Device scratch of the two-level statistics reduction plus the stats rows."""
+    """Device scratch of the two-level statistics reduction plus the stats rows.
 
-    def __init__(self, n_span, device):
-        nbytes = L.lib().jabas_sync_workspace_bytes(n_span)
-        self.buf = torch.empty(nbytes // 8, dtype=torch.float64, device=device)
+    ``Workspace.for_span(numel, dtype, device)`` sizes it for single-span calls over up to
+    ``numel`` elements; plans size their own."""
+
+    def __init__(self, nbytes, n_span, device):
+        self.buf = torch.empty(max(1, nbytes // 8), dtype=torch.float64, device=device)
         self.nbytes = nbytes
         self.stats = torch.zeros(n_span, L.STATS_STRIDE, dtype=torch.float64, device=device)
+
+    @classmethod
+    def for_span(cls, numel, grad_dtype, device):
+        return cls(L.lib().jabas_sync_workspace_bytes(int(numel), grad_dtype_code(grad_dtype)), 1, device)
 
 
 class SyncPlan:
@@ -208,14 +214,14 @@ class SyncPlan:
             c_spans[i] = sp.to_c(bound_begin=len(all_bounds))
             all_bounds += sp.bounds
         c_bounds = _bounds_array(all_bounds)
-        nbytes = lib.jabas_plan_bytes(n_span, len(all_bounds))
+        nbytes = lib.jabas_plan_bytes(c_spans, n_span, len(all_bounds), grad_dtype_code(gdt))
         self._host = np.zeros((nbytes + 7) // 8, dtype=np.uint64)        # 8-byte aligned blob
         L.check(lib.jabas_plan_encode(c_spans, n_span, c_bounds if all_bounds else None, len(all_bounds),
                                       self.K, grad_dtype_code(gdt), opt_kind_code,
                                       self._host.ctypes.data, nbytes), "jabas_plan_encode")
-        self.n_tiles = int(lib.jabas_plan_tiles(self._host.ctypes.data))
+        self.n_chunks = int(lib.jabas_plan_chunks(self._host.ctypes.data))
         self._dev = torch.from_numpy(self._host.view(np.int64)).to(dev)
-        self.ws = Workspace(n_span, dev)
+        self.ws = Workspace(lib.jabas_plan_workspace_bytes(self._host.ctypes.data), n_span, dev)
         self.n_span = n_span
 
     def run(self, args, stream=None):
@@ -242,7 +248,7 @@ def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
     ws_bytes = 0
     if args.stats:
         if workspace is None:
-            workspace = Workspace(1, span.grads[0].device)
+            workspace = Workspace.for_span(span.grads[0].numel(), span.grads[0].dtype, span.grads[0].device)
         stats_ptr, ws_ptr, ws_bytes = workspace.stats.data_ptr(), workspace.buf.data_ptr(), workspace.nbytes
     L.check(L.lib().jabas_sync_bucket(C.byref(c_span), None if bounds_dev is None else bounds_dev.data_ptr(),
                                       C.byref(args), stats_ptr, ws_ptr, ws_bytes, _stream_ptr(stream)),
@@ -283,7 +289,7 @@ def gradient_stats(grads, batches, half_id=None, workspace=None, stream=None):
     if len(w) != len(grads):
         raise ValueError("one batch size per gradient buffer")
     if workspace is None:
-        workspace = Workspace(1, dev)
+        workspace = Workspace.for_span(n, gdt, dev)
     K = len(w)
     L.check(L.lib().jabas_stats(_ptr_array(grads), K, grad_dtype_code(gdt),
                                 (C.c_float * K)(*[float(x) for x in w]),

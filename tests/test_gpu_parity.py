@@ -227,7 +227,7 @@ def test_sync_bucket_fused(gpu, K, dtype, opt):
     adam = opt["kind"] != "sgd"
     span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d, state1=s1_d, state2=s2_d if adam else None, fanout=fan,
                          bounds=bounds)
-    ws = sync.Workspace(1, gpu)
+    ws = sync.Workspace.for_span(n, dtype, gpu)
     for step in (1, 2, 3):
         args = sync.make_step_args(BATCHES[K], dtype, stats=True, opt=opt, step=step, first_step=(step == 1))
         row = sync.sync_bucket(span, args, workspace=ws)
