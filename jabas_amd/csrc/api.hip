@@ -193,32 +193,38 @@ const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_
                                        launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
 
 // Second level of the statistics reduction: one workgroup per span sums the partial rows
-// of the span's chunks. Thread t adds rows t, t+256, ... in increasing order, then the 256
-// per-thread sums are added in thread order: a fixed tree, independent of the machine.
+// of the span's chunks. Thread t adds rows t, t+256, ... in increasing order; the 256
+// per-thread sums then go through the same fixed wave tree and wave-order sum as the
+// first level, so the result does not depend on the machine or on timing.
 constexpr int kFinalizeBlock = 256;
 __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
                                                                         uint32_t use_inline, int ns,
                                                                         const double* partials, double* stats_out) {
-    __shared__ double red[kStatsStride][kFinalizeBlock + 1];
+    __shared__ double red[kFinalizeBlock / 64][kStatsStride];
     const uint32_t s = blockIdx.x, t = threadIdx.x;
     uint32_t c0 = 0, c1 = n_chunks;
     if (!use_inline) { c0 = chunk_prefix[s]; c1 = chunk_prefix[s + 1]; }
     double acc[kStatsStride];
 #pragma unroll
     for (int i = 0; i < kStatsStride; ++i) acc[i] = 0.0;
+#pragma unroll 4
     for (uint32_t c = c0 + t; c < c1; c += kFinalizeBlock) {
         const double* row = partials + static_cast<uint64_t>(c) * kStatsStride;
 #pragma unroll
-        for (int i = 0; i < kStatsStride; ++i)
-            if (i < ns) acc[i] += row[i];
+        for (int i = 0; i < kStatsStride; ++i) acc[i] += row[i];
     }
+    const int lane = t & 63, wave = t >> 6;
 #pragma unroll
-    for (int i = 0; i < kStatsStride; ++i) red[i][t] = acc[i];
+    for (int i = 0; i < kStatsStride; ++i) {
+        const double v = wave_sum_to_lane63(acc[i]);
+        if (lane == 63) red[wave][i] = v;
+    }
     __syncthreads();
     if (t < kStatsStride) {
-        double sum = 0.0;
-        for (int j = 0; j < kFinalizeBlock; ++j) sum += red[t][j];
-        stats_out[static_cast<uint64_t>(s) * kStatsStride + t] = sum;
+        double sum = red[0][t];
+#pragma unroll
+        for (int w = 1; w < kFinalizeBlock / 64; ++w) sum += red[w][t];
+        stats_out[static_cast<uint64_t>(s) * kStatsStride + t] = t < static_cast<uint32_t>(ns) ? sum : 0.0;
     }
 }
 

@@ -4,8 +4,8 @@
 //
 // Execution shape
 //   - one 256-thread workgroup (4 wave64) per chunk of kChunkTiles consecutive tiles of
-//     one span; a tile is 256 threads x one 16-byte gradient vector (4 fp32 or 8 bf16
-//     elements). Small, short-lived workgroups dispatched in order keep the part of every
+//     one span; a tile is 256 threads x 4 elements (one 16-byte vector of every fp32
+//     buffer, one 8-byte vector of a bf16 gradient buffer). Small, short-lived workgroups dispatched in order keep the part of every
 //     buffer that is being streamed at any moment compact, which on MI355X sustains a
 //     markedly higher HBM rate than a persistent grid that spreads over the whole buffers;
 //   - every global access is a 128-bit vector access with the nontemporal hint (each byte
@@ -27,18 +27,20 @@
 #ifndef JABAS_K
 #error "compile with -DJABAS_K=<1..8>"
 #endif
-#ifndef JABAS_UNROLL_F32
-#define JABAS_UNROLL_F32 2
+// Tiles whose loads are in flight together: the whole chunk without statistics, half of
+// it with (the fp64 accumulators need the registers).
+#ifndef JABAS_UNROLL_PLAIN
+#define JABAS_UNROLL_PLAIN 4
 #endif
-#ifndef JABAS_UNROLL_BF16
-#define JABAS_UNROLL_BF16 1
+#ifndef JABAS_UNROLL_STATS
+#define JABAS_UNROLL_STATS 2
 #endif
 
 namespace jabas {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 
@@ -59,17 +61,15 @@ template <> struct Grad<JABAS_F32> {
 };
 
 template <> struct Grad<JABAS_BF16> {
-    static constexpr int EPT = 8;
-    using Raw = u32x4;
+    static constexpr int EPT = 4;
+    using Raw = u32x2;
     static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
-        return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + e));
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(base) + e));
     }
     // bf16 -> fp32 is exact: the 16 bits become the high half of the fp32 pattern.
-    static __device__ __forceinline__ void widen(const Raw& r, float (&x)[8]) {
+    static __device__ __forceinline__ void widen(const Raw& r, float (&x)[4]) {
         x[0] = bits_to_float(r.x << 16); x[1] = bits_to_float(r.x & 0xffff0000u);
         x[2] = bits_to_float(r.y << 16); x[3] = bits_to_float(r.y & 0xffff0000u);
-        x[4] = bits_to_float(r.z << 16); x[5] = bits_to_float(r.z & 0xffff0000u);
-        x[6] = bits_to_float(r.w << 16); x[7] = bits_to_float(r.w & 0xffff0000u);
     }
     static __device__ __forceinline__ float load1(const void* base, uint64_t e) {
         return bits_to_float(static_cast<uint32_t>(static_cast<const uint16_t*>(base)[e]) << 16);
@@ -104,7 +104,7 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
 }
 
 // Aggregate, statistics and optimizer for N consecutive elements held in registers.
-template <int K, int N, int OPT, bool STATS>
+template <int K, int N, int OPT, bool STATS, bool HD>
 __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
                                         float (&s2)[N], float (&agg)[N], const KArgs& a,
                                         const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
@@ -119,9 +119,13 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
 #pragma unroll
             for (int k = 0; k < K; ++k) {
                 const float t = g[k][i] * a.wh[k];
-                const bool in_b = (a.half_mask >> k) & 1u;
-                gb = in_b ? gb + t : gb;
-                ga = in_b ? ga : ga + t;
+                if constexpr (HD) {            // default halves: even worker -> A, odd -> B
+                    if (k & 1) gb = gb + t; else ga = ga + t;
+                } else {
+                    const bool in_b = (a.half_mask >> k) & 1u;
+                    gb = in_b ? gb + t : gb;
+                    ga = in_b ? ga : ga + t;
+                }
                 const double gk = static_cast<double>(g[k][i]);
                 acc[JABAS_STAT_NORM_VSW0 + k] = __builtin_fma(gk, gk, acc[JABAS_STAT_NORM_VSW0 + k]);
             }
@@ -134,6 +138,9 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
             acc[JABAS_STAT_NORM_AGG] = __builtin_fma(ds, ds, acc[JABAS_STAT_NORM_AGG]);
         }
         if constexpr (OPT != OPT_NONE) opt_elem<OPT>(s, p[i], s1[i], s2[i], G, a.opt);
+        // keep the elements' dependency chains apart: interleaving them costs the statistics
+        // kernels a third of their occupancy in registers and buys nothing in a memory-bound loop
+        if constexpr (STATS) __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -180,7 +187,7 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev
 }
 
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
-template <int K, int DT, int OPT, bool STATS, int U>
+template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const KArgs& a,
                                         const GroupDev& G, bool use_s1, bool load_s1,
                                         double (&acc)[NStats<K, STATS>::value]) {
@@ -202,7 +209,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
             }
             if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r.s2[u], s2);
         }
-        compute<K, EPT, OPT, STATS>(g, p, s1, s2, agg, a, G, acc);
+        compute<K, EPT, OPT, STATS, HD>(g, p, s1, s2, agg, a, G, acc);
         if (sp.out) store_vec<NV>(agg, sp.out, eu);
         if constexpr (OPT != OPT_NONE) {
             store_vec<NV>(p, sp.p, eu);
@@ -214,7 +221,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 }
 
 // Vector path over nfull consecutive full tiles of one parameter group.
-template <int K, int DT, int OPT, bool STATS, int U>
+template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
                                          const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
@@ -224,13 +231,13 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
     for (; i + U <= nfull; i += U, e += U * TE) {
         TileRegs<K, DT, U> r;
         issue_loads<K, DT, OPT, U>(r, sp, e, load_s1);
-        consume<K, DT, OPT, STATS, U>(r, sp, e, a, G, use_s1, load_s1, acc);
+        consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, use_s1, load_s1, acc);
     }
     if constexpr (U > 1) {
         for (; i < nfull; ++i, e += TE) {
             TileRegs<K, DT, 1> r;
             issue_loads<K, DT, OPT, 1>(r, sp, e, load_s1);
-            consume<K, DT, OPT, STATS, 1>(r, sp, e, a, G, use_s1, load_s1, acc);
+            consume<K, DT, OPT, STATS, HD, 1>(r, sp, e, a, G, use_s1, load_s1, acc);
         }
     }
 }
@@ -266,7 +273,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
             if (load_s1) s1[0] = sp.s1[e];
             if constexpr (OPT == OPT_ADAM) s2[0] = sp.s2[e];
         }
-        compute<K, 1, OPT, STATS>(g, p, s1, s2, agg, a, G, acc);
+        compute<K, 1, OPT, STATS, false>(g, p, s1, s2, agg, a, G, acc);
         if (sp.out) sp.out[e] = agg[0];
         if constexpr (OPT != OPT_NONE) {
             sp.p[e] = p[0];
@@ -278,13 +285,14 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 }
 
 // Tiles [lt0, lt1) of one span (tile indices local to the span).
-template <int K, int DT, int OPT, bool STATS>
+template <int K, int DT, int OPT, bool STATS, bool HD>
 __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
                                            const KArgs& a, double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
-    constexpr int U = (DT == JABAS_BF16) ? JABAS_UNROLL_BF16 : JABAS_UNROLL_F32;
+    constexpr int U = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
+    static_assert(U <= kChunkTiles, "a chunk is the unit of work of one workgroup");
     const uint32_t nb = sp.bound_count;
     const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
     uint32_t lt = lt0, j = j0;
@@ -307,7 +315,7 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
         }
         if (nfull) {
             const GroupDev G = a.groups[gid];
-            fast_run<K, DT, OPT, STATS, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, acc);
+            fast_run<K, DT, OPT, STATS, HD, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, acc);
             lt += nfull;
         } else {
             careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, acc);
@@ -316,24 +324,18 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     }
 }
 
-// Sum over the 64 lanes of a wave with DPP moves (no LDS traffic); the total lands in
-// lane 63. Pairing order is fixed: lane^1, lane^2, mirror within 8, mirror within 16,
-// row 0->1 and 2->3, rows 0..1 -> 2..3.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ double dpp_move(double v) {
-    int lo = __double2loint(v), hi = __double2hiint(v);
-    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
-    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
-    return __hiloint2double(hi, lo);
-}
-__device__ __forceinline__ double wave_sum_to_lane63(double v) {
-    v += dpp_move<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
-    v += dpp_move<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
-    v += dpp_move<0x141, 0xf>(v);   // row_half_mirror
-    v += dpp_move<0x140, 0xf>(v);   // row_mirror
-    v += dpp_move<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
-    v += dpp_move<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
-    return v;
+// Statistics kernels carry two copies of the arithmetic: one with the default halves
+// (even worker -> A, odd -> B) resolved at compile time, one driven by the half mask.
+template <int K, int DT, int OPT, bool STATS>
+__device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const KArgs& a,
+                                          double (&acc)[NStats<K, STATS>::value]) {
+    if constexpr (STATS) {
+        constexpr uint32_t kDefaultMask = 0xAAu & ((1u << K) - 1u);
+        if (a.half_mask == kDefaultMask) span_range<K, DT, OPT, true, true>(sp, lt0, lt1, j0, a, acc);
+        else span_range<K, DT, OPT, true, false>(sp, lt0, lt1, j0, a, acc);
+    } else {
+        span_range<K, DT, OPT, false, true>(sp, lt0, lt1, j0, a, acc);
+    }
 }
 
 template <int NS>
@@ -346,10 +348,13 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
         if (lane == 63) red[wave][i] = v;
     }
     __syncthreads();
-    if (threadIdx.x < NS) {
-        double s = red[0][threadIdx.x];
+    if (threadIdx.x < kStatsStride) {          // unused slots of the row are written as zero
+        double s = 0.0;
+        if (threadIdx.x < NS) {
+            s = red[0][threadIdx.x];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) s += red[w][threadIdx.x];
+            for (int w = 1; w < kWaves; ++w) s += red[w][threadIdx.x];
+        }
         row[threadIdx.x] = s;
     }
 }
@@ -380,13 +385,13 @@ __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
             }
             j0 = lo;
         }
-        span_range<K, DT, OPT, STATS>(sp, lt0, lt1, j0, a, acc);
+        run_chunk<K, DT, OPT, STATS>(sp, lt0, lt1, j0, a, acc);
     } else {
         const ChunkDesc c = a.chunks[b];
         const SpanDev& sp = a.spans[c.span];
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
         const uint32_t lt1 = c.tile0 + kChunkTiles < tiles ? c.tile0 + kChunkTiles : tiles;
-        span_range<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
+        run_chunk<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
     if constexpr (STATS) flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);
 }

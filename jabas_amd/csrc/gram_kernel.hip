@@ -1,5 +1,5 @@
 // K x K Gram matrix of the K worker gradients of one span: gram[a][b] = sum_e g_a[e]*g_b[e].
-// fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums. Grid-stride over 16-byte
+// fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums. Grid-stride over 4-element
 // vectors, K(K+1)/2 accumulators per thread, wave64 shuffle tree -> LDS -> one packed
 // partial row per workgroup, then a single-workgroup finalize that sums the rows in
 // workgroup order and mirrors the lower triangle.
@@ -9,7 +9,7 @@ namespace jabas {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 
@@ -23,13 +23,11 @@ template <> struct GramLoad<JABAS_F32> {
     static __device__ __forceinline__ float one(const void* base, uint64_t e) { return static_cast<const float*>(base)[e]; }
 };
 template <> struct GramLoad<JABAS_BF16> {
-    static constexpr int EPT = 8;
-    static __device__ __forceinline__ void vec(const void* base, uint64_t e, float (&x)[8]) {
-        const u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + e));
+    static constexpr int EPT = 4;
+    static __device__ __forceinline__ void vec(const void* base, uint64_t e, float (&x)[4]) {
+        const u32x2 r = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(base) + e));
         x[0] = bits_to_float(r.x << 16); x[1] = bits_to_float(r.x & 0xffff0000u);
         x[2] = bits_to_float(r.y << 16); x[3] = bits_to_float(r.y & 0xffff0000u);
-        x[4] = bits_to_float(r.z << 16); x[5] = bits_to_float(r.z & 0xffff0000u);
-        x[6] = bits_to_float(r.w << 16); x[7] = bits_to_float(r.w & 0xffff0000u);
     }
     static __device__ __forceinline__ float one(const void* base, uint64_t e) {
         return bits_to_float(static_cast<uint32_t>(static_cast<const uint16_t*>(base)[e]) << 16);

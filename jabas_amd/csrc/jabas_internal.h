@@ -13,8 +13,10 @@ constexpr int kWaves = kBlock / 64;
 constexpr int kChunkTiles = 4;              // tiles one workgroup processes (a "chunk")
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
-// Elements one thread handles per tile: one 16-byte gradient vector.
-__host__ __device__ constexpr int ept_of(int grad_dtype) { return grad_dtype == JABAS_BF16 ? 8 : 4; }
+// Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer
+// (bf16 gradients are then read as 8-byte vectors, which keeps every access of a wave
+// contiguous).
+__host__ __device__ constexpr int ept_of(int /*grad_dtype*/) { return 4; }
 __host__ __device__ constexpr int tile_elems(int grad_dtype) { return kBlock * ept_of(grad_dtype); }
 __host__ __device__ constexpr int chunk_elems(int grad_dtype) { return kChunkTiles * tile_elems(grad_dtype); }
 
@@ -81,6 +83,29 @@ struct KArgs {
     OptDev opt;
     GroupDev groups[JABAS_MAX_GROUPS];
 };
+
+#if defined(__HIPCC__)
+// Sum over the 64 lanes of a wave with DPP moves (no LDS traffic); the total lands in
+// lane 63. Pairing order is fixed: lane^1, lane^2, mirror within 8, mirror within 16,
+// row 0->1 and 2->3, rows 0..1 -> 2..3.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double v) {
+    int lo = __double2loint(v), hi = __double2hiint(v);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double wave_sum_to_lane63(double v) {
+    v += dpp_move<0xB1, 0xf>(v);    // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xf>(v);    // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(v);   // row_half_mirror
+    v += dpp_move<0x140, 0xf>(v);   // row_mirror
+    v += dpp_move<0x142, 0xa>(v);   // row_bcast:15 into rows 1 and 3
+    v += dpp_move<0x143, 0xc>(v);   // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+#endif
 
 // Per-K launchers, one translation unit each (fused_kernel.hip with -DJABAS_K=k).
 // opt_class: 0 none, 1 SGD, 2 Adam/AdamW. Returns hipError_t as int.
