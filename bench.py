@@ -31,8 +31,11 @@ HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published peak
 ROTATE_TARGET_BYTES = 1.5e9   # minimum total working set per configuration
 
 # HBM bytes per launch of the fused kernel measured with rocprofv3 --pmc (FETCH_SIZE and
-# WRITE_SIZE runs, scaled by a copy kernel of known size); see profiles/. None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+# WRITE_SIZE runs, scaled by a copy kernel of known size; profiles/fused_kernel_hbm_traffic_pmc.md).
+MEASURED_TRAFFIC_BYTES = {
+    "vit_b16": 3813.9e6, "resnet50": 716.7e6, "faster_rcnn_r50_fpn": 1341.9e6, "gnmt": 7078.1e6,
+    "vit_l16": 13406.9e6,
+}
 
 
 def algorithmic_bytes_per_elem(cfg):
@@ -148,6 +151,10 @@ def main():
     ap.add_argument("--workload", default="vit_b16")
     ap.add_argument("--no-all", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB copy 5 times (the K=1, weight-1 aggregate: same 16-byte "
+                         "nontemporal loads and stores as the fused kernel, known traffic) for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures the one-GPU share of the gradient-sync path; "
@@ -161,6 +168,15 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     head_cfg = W.config(args.workload)
+    if args.calibrate_copy:
+        from jabas_amd import sync
+        src = torch.ones(1 << 28, dtype=torch.float32, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            sync.aggregate([src], (1,), out=dst)       # fused_kernel<1, f32, none, no stats>: out = src * 1.0f
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
     results = {}
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
     for cfg in order:
