@@ -1,0 +1,153 @@
+"""Per-GPU rendezvous of the K virtual stream workers (VSWs) around one fused launch.
+
+In IIDP every VSW runs its own DDP reducer on its own thread and stream; only VSW 0's
+comm hook communicates, the others register ``dummy_hook``
+(jabas/train/trainer.py:452-468). ``LocalBucketSync`` is where those K hooks meet on one
+GPU: each hook publishes the flat bucket it was handed; when the K buckets with the same
+index are in, whichever thread arrived last queues ONE fused kernel on VSW 0's stream
+(aggregate into VSW 0's bucket, statistics when asked, optimizer update when the weights
+are laid out like the buckets) and resolves the futures. No hook ever blocks, so the
+scheme also works when the VSWs are driven from a single thread one after the other.
+"""
+import threading
+
+import torch
+
+from . import sync
+from . import _lib as L
+
+
+class BucketStats:
+    """Statistics row of one bucket on the device (what a stat step leaves in
+    ``GradientSimilarityState.grad_placeholder`` instead of a full gradient copy)."""
+
+    def __init__(self, index, row):
+        self.index, self.row = index, row
+
+    def cpu(self):
+        return self.row.detach().to("cpu")
+
+
+class _Slot:
+    def __init__(self, K):
+        self.tensors = [None] * K
+        self.events = [None] * K
+        self.futures = [None] * K
+        self.values = [None] * K
+        self.want_stats = False
+        self.on_done = None
+        self.count = 0
+
+
+class LocalBucketSync:
+    """batches: local batch size of each VSW on this GPU (defines K and the weights).
+
+    launcher(bucket_index, tensors, want_stats) -> stats row or None replaces the C-ABI
+    call (CPU tests of the protocol inject a recorder); the default queues
+    ``jabas_sync_bucket`` on VSW 0's stream.
+    """
+
+    def __init__(self, batches, launcher=None, opt=None, param_buckets=None):
+        self.batches = tuple(batches)
+        self.K = len(self.batches)
+        self.opt = opt
+        self.param_buckets = param_buckets or {}     # bucket index -> dict(param=, state1=, state2=, bounds=, fanout=)
+        self.step_count = 0
+        self.lr_scale = 1.0
+        self._launcher = launcher or self._launch_fused
+        self._lock = threading.Lock()
+        self._slots = {}
+        self._main_stream = None
+        self._workspaces = {}
+        self._done_events = []
+
+    # ------------------------------------------------------------------ hooks call this
+    def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None):
+        """Hands VSW k's bucket ``bucket_index`` over. Returns a Future that resolves (to
+        ``value``, default the tensor) once the fused launch for that bucket is queued."""
+        if not 0 <= k < self.K:
+            raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
+        fut = torch.futures.Future()
+        event = stream = None
+        if tensor.is_cuda:
+            stream = torch.cuda.current_stream(tensor.device)
+            event = torch.cuda.Event()
+            event.record(stream)
+        with self._lock:
+            slot = self._slots.setdefault(bucket_index, _Slot(self.K))
+            if slot.tensors[k] is not None:
+                raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
+            slot.tensors[k], slot.events[k], slot.futures[k] = tensor, event, fut
+            slot.values[k] = tensor if value is None else value
+            slot.count += 1
+            if k == 0:
+                slot.want_stats, slot.on_done = want_stats, on_done
+                self._main_stream = stream
+            ready = slot.count == self.K
+            if ready:
+                del self._slots[bucket_index]
+        if ready:
+            self._fire(bucket_index, slot)
+        return fut
+
+    def _fire(self, bucket_index, slot):
+        main = self._main_stream
+        try:
+            if main is not None:
+                with torch.cuda.stream(main):
+                    for ev in slot.events[1:]:
+                        main.wait_event(ev)
+                    row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
+                    done = torch.cuda.Event()
+                    done.record(main)
+                    self._done_events.append(done)
+            else:
+                row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
+        except Exception as exc:                       # surface the failure in every waiting hook
+            for f in slot.futures:
+                f.set_exception(exc)
+            return
+        if slot.on_done is not None:
+            slot.on_done(BucketStats(bucket_index, row) if row is not None else None)
+        for f, v in zip(slot.futures, slot.values):
+            f.set_result(v)
+
+    # ------------------------------------------------------------- the default launcher
+    def _launch_fused(self, bucket_index, tensors, want_stats):
+        g0 = tensors[0]
+        pb = self.param_buckets.get(bucket_index)
+        opt = self.opt if pb is not None else None
+        span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
+                             param=pb and pb.get("param"), state1=pb and pb.get("state1"),
+                             state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
+                             bounds=(pb or {}).get("bounds", ()) if opt else ())
+        args = sync.make_step_args(self.batches, g0.dtype, stats=want_stats, opt=opt, step=self.step_count + 1,
+                                   first_step=self.step_count == 0, lr_scale=self.lr_scale)
+        ws = None
+        if want_stats:
+            key = (bucket_index, g0.numel())
+            ws = self._workspaces.get(key)
+            if ws is None:
+                ws = self._workspaces[key] = sync.Workspace.for_span(g0.numel(), g0.dtype, g0.device)
+        bd = None
+        if span.bounds:
+            bd = (pb or {}).get("_bounds_dev")
+        row = sync.sync_bucket(span, args, workspace=ws, bounds_dev=bd)
+        return row.clone() if row is not None else None
+
+    # ------------------------------------------------------------------ trainer calls this
+    def pending(self):
+        with self._lock:
+            return sorted(self._slots)
+
+    def finish_step(self, streams=()):
+        """End of a sync step: every VSW stream waits for the fused launches that read its
+        buckets, and the step count (Adam's t, SGD's first-step flag) advances."""
+        left = self.pending()
+        if left:
+            raise RuntimeError(f"buckets {left} were not published by every VSW")
+        for s in streams:
+            for ev in self._done_events:
+                s.wait_event(ev)
+        self._done_events = []
+        self.step_count += 1

@@ -1,0 +1,147 @@
+"""The part of the IIDP/JABAS trainer that sits on the gradient-sync path, for one GPU.
+
+``VSWSyncTrainer`` mirrors the attributes and call order through which the reference
+reaches the path (jabas/train/trainer.py: ``prepare_stream_parallel`` :82-86,
+``prepare_weight_sync_method`` :88-98, ``compute`` :171-174, ``step`` :176-197,
+``_compute_cosine_similarity`` :470-483, ``_adjust_adaptive_lr`` :693-700; attributes
+``local_models``, ``main_model``, ``model_streams``, ``num_models``, ``similarity_state``,
+``cos_placeholder``): K model replicas on K HIP streams, one sync step per iteration.
+It is not the reference's trainer: data loading, the configuration solver, elastic
+restarts and the cross-GPU all-reduce are outside this build.
+
+Memory layout (MI355X-first): the weights, their optimizer state, the aggregated gradient
+and every VSW's gradients live in flat arenas with one common bucket layout
+(``VSWFlatSync``); module parameters and their ``.grad`` are views into the arenas, so
+backward writes straight into the buckets (what ``gradient_as_bucket_view=True`` gives
+the reference) and the whole sync step is one fused launch that also refreshes the
+replicas' weights.
+"""
+import copy
+
+import torch
+
+from ..engine import VSWFlatSync
+from ..workloads import ParamSpec
+from ..ddp_comm_hooks import GradientSimilarityState
+from .. import sync
+
+
+def create_optimizer_hook(hook, optimizer):
+    """Counterpart of IIDPTrainer._create_optimizer_hook (call site
+    jabas/train/trainer.py:332): run ``hook`` and, once its Future resolves, apply
+    ``optimizer.step(gradients)`` to the parameters of that bucket. Gradients are taken
+    from ``bucket.gradients()`` / ``bucket.parameters()`` (torch >= 1.10 GradBucket) and
+    tagged with ``.index`` the way the reference matches them
+    (examples/gnmt/seq2seq/train/shard_optimizer.py:41-46)."""
+    def hook_then_step(state, bucket):
+        fut = hook(state, bucket)
+
+        def run(done):
+            value = done.value()
+            params, grads = bucket.parameters(), bucket.gradients()
+            for p, g in zip(params, grads):
+                if not isinstance(getattr(p, "index", None), int):
+                    raise RuntimeError("parameters need an .index attribute (see tag_parameter_indices)")
+                g.index = p.index
+            optimizer.step(grads)
+            return value
+
+        return fut.then(run)
+    return hook_then_step
+
+
+def tag_parameter_indices(model):
+    """Gives every parameter the ``.index`` the Shard optimizers match on."""
+    for i, p in enumerate(model.parameters()):
+        p.index = i
+    return model
+
+
+class VSWSyncTrainer:
+    def __init__(self, gpu, local_batch_sizes, opt, interval=100, grad_dtype=torch.float32,
+                 param_groups_func=None, similarity_target=None):
+        self.gpu = torch.device("cuda", gpu) if isinstance(gpu, int) else torch.device(gpu)
+        self.local_batch_sizes = tuple(local_batch_sizes)
+        self.num_models = len(self.local_batch_sizes)
+        self.total_num_decoupled_workers = self.num_models
+        self.opt = opt
+        self.grad_dtype = grad_dtype
+        self.param_groups_func = param_groups_func
+        self.similarity_target = similarity_target
+        self.global_lr_modifier = 1.0
+        self.local_models, self.model_streams = [], []
+        self.main_model = None
+        self.engine = None
+        self.cos_placeholder = None
+        self.grad_placeholders = [[], []]
+        workers = self.num_models if self.num_models % 2 == 0 else self.num_models + 1
+        self.similarity_state = GradientSimilarityState(None, workers, None, self.grad_placeholders[0], interval)
+
+    # ---------------------------------------------------------------------- set-up
+    def prepare_stream_parallel(self, model, criterion):
+        model = model.to(self.gpu)
+        names = [n for n, _ in model.named_parameters()]
+        params = [p for _, p in model.named_parameters()]
+        group_of = {}
+        if self.param_groups_func is not None:
+            for gi, group in enumerate(self.param_groups_func(model)):
+                for p in group["params"]:
+                    group_of[id(p)] = gi
+        specs = [ParamSpec(n, p.numel(), group_of.get(id(p), 0)) for n, p in zip(names, params)]
+        self.engine = VSWFlatSync(specs, self.local_batch_sizes, grad_dtype=self.grad_dtype, opt=self.opt,
+                                  device=self.gpu, n_fanout=self.num_models - 1)
+        self.criterion = criterion
+        self.local_models = [model] + [copy.deepcopy(model) for _ in range(self.num_models - 1)]
+        self.main_model = self.local_models[0]
+        self.model_streams = [torch.cuda.Stream(self.gpu) for _ in range(self.num_models)]
+        eng = self.engine
+        with torch.no_grad():
+            for k, m in enumerate(self.local_models):
+                weights = eng.param if k == 0 else eng.fanout[k - 1]
+                for i, p in enumerate(m.parameters()):
+                    view = eng._view(weights, i).view(p.shape)
+                    view.copy_(p.data)
+                    p.data = view
+                    if self.grad_dtype == torch.float32:
+                        p.grad = eng.grad_view(k, i).view(p.shape)     # backward accumulates into the bucket
+        torch.cuda.synchronize(self.gpu)
+
+    # ------------------------------------------------------------------- one iteration
+    def compute(self, data):
+        """data: one (input, target) pair per VSW, already on the GPU."""
+        if len(data) != self.num_models:
+            raise ValueError(f"expected {self.num_models} local batches, got {len(data)}")
+        cur = torch.cuda.current_stream(self.gpu)
+        losses = []
+        for k, ((x, y), m, s) in enumerate(zip(data, self.local_models, self.model_streams)):
+            s.wait_stream(cur)
+            with torch.cuda.stream(s):
+                loss = self.criterion(m(x), y)
+                loss.backward()
+                if self.grad_dtype != torch.float32:
+                    for i, p in enumerate(m.parameters()):
+                        self.engine.grad_view(k, i).copy_(p.grad.reshape(-1))
+                        p.grad = None
+                losses.append(loss.detach())
+        return losses
+
+    def step(self):
+        cur = torch.cuda.current_stream(self.gpu)
+        for s in self.model_streams:
+            cur.wait_stream(s)
+        st = self.similarity_state
+        want = st.step % st.interval == 0
+        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier)
+        if want:
+            self._compute_cosine_similarity(rows)
+        for k in range(self.num_models):
+            self.engine.grads[k].zero_()
+        for s in self.model_streams:
+            s.wait_stream(cur)
+        st.step += 1
+        return True
+
+    def _compute_cosine_similarity(self, rows):
+        self.cos_placeholder = torch.tensor([sync.cosine_from_stats(rows)])
+        self.similarity_state.grad_placeholder = []
+        return self.cos_placeholder

@@ -1,0 +1,184 @@
+"""CPU-only checks of the C ABI: the shared library loads, exports every symbol the header
+declares, and its pure-host entry points (plan encoding, size queries, status strings)
+behave as documented. No kernel is launched here.
+"""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from jabas_amd import _lib as L
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "jabas_sync.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(jabas_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert len(names) >= 14
+    lib = L.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in jabas_sync.h but not exported"
+    assert set(names) == set(L.SIGNATURES), "ctypes signature table and header disagree"
+
+
+def test_struct_layouts_match_the_header():
+    # sizes a C compiler gives the header's structs on x86-64 / amdgcn host ABI
+    assert C.sizeof(L.JabasSpan) == 8 * 8 + 4 * 8 + 7 * 8 + 8 + 4 * 4
+    assert C.sizeof(L.JabasBound) == 16
+    assert C.sizeof(L.JabasGroup) == 24
+    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 32 + 4 + 8 + 32 + 4 * 4 + 4 + 5 * 8 + 16 * 24
+    assert L.JabasStepArgs.groups.offset % 8 == 0 and L.JabasStepArgs.momentum.offset % 8 == 0
+
+
+def test_version_and_status_strings():
+    lib = L.lib()
+    assert b"jabas_sync" in lib.jabas_sync_version()
+    assert lib.jabas_status_string(0) == b"ok"
+    seen = {lib.jabas_status_string(s) for s in range(-11, 0)}
+    assert len(seen) == 11 and b"unknown status" not in seen
+    assert lib.jabas_status_string(-99) == b"unknown status"
+
+
+def _span(numel, base=0x7f0000000000, K=2, gs=4, skew=0, opt=False, stride=1 << 32):
+    s = L.JabasSpan()
+    for k in range(K):
+        s.grads[k] = base + k * stride + skew * gs
+    s.agg_out = base + 8 * stride + skew * 4
+    if opt:
+        s.param = base + 9 * stride + skew * 4
+        s.state1 = base + 10 * stride + skew * 4
+        s.state2 = base + 11 * stride + skew * 4
+    s.numel = numel
+    return s
+
+
+def _encode(spans, bounds=(), K=2, dtype=L.F32, opt=L.OPT_NONE):
+    lib = L.lib()
+    arr = (L.JabasSpan * len(spans))(*spans)
+    barr = (L.JabasBound * max(1, len(bounds)))()
+    for i, (st, g) in enumerate(bounds):
+        barr[i].start, barr[i].group = st, g
+    nbytes = lib.jabas_plan_bytes(arr, len(spans), len(bounds), dtype)
+    blob = np.zeros(nbytes // 8 + 1, dtype=np.uint64)
+    rc = lib.jabas_plan_encode(arr, len(spans), barr if bounds else None, len(bounds), K, dtype, opt,
+                               blob.ctypes.data, nbytes)
+    return rc, blob, nbytes
+
+
+def test_plan_encode_counts_chunks_of_4096_elements():
+    lib = L.lib()
+    rc, blob, _ = _encode([_span(4096), _span(4097), _span(1), _span(0), _span(10 * 4096 + 5)])
+    assert rc == L.OK
+    assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
+    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) == (15 + 1) * 12 * 8
+    # a span that starts 3 elements into a 16-byte line needs one more tile when it is exactly full
+    rc, blob, _ = _encode([_span(4096, skew=3)])
+    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data) == 2
+
+
+def test_plan_encode_bf16_positions_are_counted_in_elements():
+    # bf16 gradients 2 elements into an 8-byte line, fp32 buffers 2 elements into a 16-byte line: congruent
+    rc, _, _ = _encode([_span(5000, gs=2, skew=2)], dtype=L.BF16)
+    assert rc == L.OK
+    s = _span(5000, gs=2, skew=2)
+    s.agg_out += 4                      # now 3 elements in: not congruent with the gradients
+    rc, _, _ = _encode([s], dtype=L.BF16)
+    assert rc == L.ERR_ALIGN
+
+
+def test_plan_encode_rejects_bad_spans():
+    s = _span(4096)
+    s.grads[1] += 4
+    assert _encode([s])[0] == L.ERR_ALIGN                       # gradients not mutually congruent
+    s = _span(4096)
+    s.grads[1] = 0
+    assert _encode([s])[0] == L.ERR_NULL
+    assert _encode([_span(4096)], K=9)[0] == L.ERR_K
+    assert _encode([_span(4096)], dtype=7)[0] == L.ERR_DTYPE
+    assert _encode([_span(4096)], opt=9)[0] == L.ERR_OPT
+    assert _encode([_span(4096)], opt=L.OPT_SGD)[0] == L.ERR_NULL    # optimizer without weights
+    s = _span(4096, opt=True)
+    s.state2 = 0
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_NULL
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.OK
+    s = _span(4096)
+    s.agg_out = s.grads[0] + 16                                 # overlaps VSW 0's buffer, not in place
+    assert _encode([s])[0] == L.ERR_ALIAS
+    s = _span(4096)
+    s.agg_out = s.grads[0]                                      # exactly in place: allowed for fp32
+    assert _encode([s])[0] == L.OK
+    s = _span(4096, gs=2)
+    s.agg_out = s.grads[0]
+    assert _encode([s], dtype=L.BF16)[0] == L.ERR_ALIAS          # fp32 output over bf16 input
+    s = _span(4096, opt=True)
+    s.n_fanout = 8
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_SIZE
+
+
+def test_plan_encode_checks_bounds():
+    def with_bounds(bounds, count=None, begin=0):
+        s = _span(10000, opt=True)
+        s.bound_begin, s.bound_count = begin, len(bounds) if count is None else count
+        return _encode([s], bounds=bounds, opt=L.OPT_SGD)[0]
+    assert with_bounds([(0, 0), (100, 1), (9999, 0)]) == L.OK
+    assert with_bounds([(1, 0)]) == L.ERR_GROUP                 # first bound must start at 0
+    assert with_bounds([(0, 0), (100, 1), (100, 0)]) == L.ERR_GROUP   # not strictly increasing
+    assert with_bounds([(0, 0), (10000, 1)]) == L.ERR_GROUP     # starts past the end
+    assert with_bounds([(0, 16)]) == L.ERR_GROUP                # group index out of range
+    assert with_bounds([(0, 0)], count=2) == L.ERR_GROUP        # table shorter than claimed
+
+
+def test_plan_blob_too_small_and_garbage_header():
+    lib = L.lib()
+    spans = (L.JabasSpan * 1)(_span(4096))
+    nbytes = lib.jabas_plan_bytes(spans, 1, 0, L.F32)
+    blob = np.zeros(nbytes // 8 + 1, dtype=np.uint64)
+    assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, nbytes - 8) == L.ERR_PLAN
+    junk = np.zeros(64, dtype=np.uint64)
+    assert lib.jabas_plan_chunks(junk.ctypes.data) == L.ERR_PLAN
+    assert lib.jabas_plan_workspace_bytes(junk.ctypes.data) == 0
+    args = L.JabasStepArgs()
+    args.K = 2
+    assert lib.jabas_sync_fused(junk.ctypes.data, 0x1000, C.byref(args), None, None, 0, None) == L.ERR_PLAN
+    assert lib.jabas_sync_fused(None, None, C.byref(args), None, None, 0, None) == L.ERR_NULL
+
+
+def test_workspace_bytes_cover_any_line_position():
+    lib = L.lib()
+    assert lib.jabas_sync_workspace_bytes(0, L.F32) >= 96
+    assert lib.jabas_sync_workspace_bytes(4096, L.F32) >= 2 * 96      # a shifted start can straddle two chunks
+    assert lib.jabas_sync_workspace_bytes(1 << 30, L.BF16) >= ((1 << 30) // 4096) * 96
+
+
+def test_entry_points_validate_before_launching():
+    """Argument errors are reported on a machine without a GPU because nothing is launched."""
+    lib = L.lib()
+    w = (C.c_float * 2)(0.5, 0.5)
+    g = (C.c_void_p * 2)(0x7f0000000000, 0x7f0100000000)
+    assert lib.jabas_aggregate(g, 0, L.F32, w, 0x7f0200000000, 100, None) == L.ERR_K
+    assert lib.jabas_aggregate(g, 2, L.F32, w, None, 100, None) == L.ERR_NULL
+    assert lib.jabas_aggregate(g, 2, 5, w, 0x7f0200000000, 100, None) == L.ERR_DTYPE
+    g[1] = 0x7f0100000004
+    assert lib.jabas_aggregate(g, 2, L.F32, w, 0x7f0200000000, 100, None) == L.ERR_ALIGN
+    assert lib.jabas_sgd(None, 0x7f0000000000, None, 10, 0.1, 0.0, 0.0, 0.0, 0, 0, None) == L.ERR_NULL
+    # momentum without a buffer
+    assert lib.jabas_sgd(0x7f0000000000, 0x7f0100000000, None, 10, 0.1, 0.0, 0.9, 0.0, 0, 0, None) == L.ERR_NULL
+    # nesterov needs momentum and zero dampening
+    assert lib.jabas_sgd(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 10, 0.1, 0.0, 0.9, 0.1, 1, 0, None) == L.ERR_OPT
+    # Adam's step count is 1-based
+    assert lib.jabas_adam(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 0x7f0300000000, 10, 1e-3, 0.0, 0.9, 0.999,
+                          1e-8, 0, 0, None) == L.ERR_OPT
+    hid = (C.c_uint8 * 2)(0, 1)
+    assert lib.jabas_stats(g, 2, L.F32, w, hid, w, 100, 0x7f0400000000, None, 0, None) == L.ERR_ALIGN
+    g[1] = 0x7f0100000000
+    assert lib.jabas_stats(g, 2, L.F32, w, hid, w, 100, 0x7f0400000000, None, 0, None) == L.ERR_WORKSPACE
+    assert lib.jabas_gram(g, 2, L.F32, 100, 0x7f0400000000, None, 0, None) == L.ERR_WORKSPACE

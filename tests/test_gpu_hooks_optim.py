@@ -1,0 +1,201 @@
+"""GPU tests of the host layer above the C ABI: Shard optimizers against torch.optim,
+the K-VSW rendezvous with real streams and threads against the oracle, and the slim
+trainer end to end against a plain-torch restatement of one training step.
+Tolerances: weights 1e-6 relative (absolute floor of a few ulp of the operands),
+aggregate bit-exact, statistics 1e-6 relative.
+"""
+import copy
+import threading
+
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(a, b, rtol=1e-6, atol=1e-9):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    return bool(((a - b).abs() <= rtol * b.abs() + atol).all())
+
+
+def _mlp(seed):
+    torch.manual_seed(seed)
+    return torch.nn.Sequential(torch.nn.Linear(37, 64), torch.nn.ReLU(), torch.nn.Linear(64, 33, bias=True),
+                               torch.nn.ReLU(), torch.nn.Linear(33, 10))
+
+
+def _groups(model):
+    decay = [p for p in model.parameters() if p.dim() > 1]
+    no_decay = [p for p in model.parameters() if p.dim() <= 1]
+    return [{"params": no_decay, "weight_decay": 0.0}, {"params": decay, "weight_decay": 0.05}]
+
+
+@pytest.mark.parametrize("kind", ["sgd", "sgd_nesterov", "adam", "adamw"])
+def test_shard_optimizers_match_torch_optim(gpu, kind):
+    from jabas_amd import optim
+    ref_model, my_model = _mlp(0).to(gpu), _mlp(0).to(gpu)
+    if kind == "sgd":
+        ref = torch.optim.SGD(_groups(ref_model), lr=0.1, momentum=0.9, foreach=False)
+        mine = optim.ShardSGD(_groups(my_model), lr=0.1, momentum=0.9)
+    elif kind == "sgd_nesterov":
+        ref = torch.optim.SGD(_groups(ref_model), lr=0.05, momentum=0.8, nesterov=True, foreach=False)
+        mine = optim.ShardSGD(_groups(my_model), lr=0.05, momentum=0.8, nesterov=True)
+    elif kind == "adam":
+        ref = torch.optim.Adam(_groups(ref_model), lr=2e-3, foreach=False)
+        mine = optim.ShardAdam(_groups(my_model), lr=2e-3)
+    else:
+        ref = torch.optim.AdamW(_groups(ref_model), lr=5e-4, foreach=False)
+        mine = optim.ShardAdamW(_groups(my_model), lr=5e-4)
+    for step in range(4):
+        g = torch.Generator(device="cpu").manual_seed(step)
+        x = torch.randn(16, 37, generator=g).to(gpu)
+        for model in (ref_model, my_model):
+            model.zero_grad(set_to_none=True)
+            model(x).square().mean().backward()
+        ref.step()
+        mine.step()
+        torch.cuda.synchronize()
+        for pr, pm in zip(ref_model.parameters(), my_model.parameters()):
+            assert _close(pm, pr, 1e-6, 1e-8), f"{kind} step {step}"
+    key = "momentum_buffer" if kind.startswith("sgd") else "exp_avg"
+    for pr, pm in zip(ref_model.parameters(), my_model.parameters()):
+        assert _close(mine.state[pm][key], ref.state[pr][key], 1e-6, 1e-8)
+
+
+def test_shard_step_with_bucket_gradients_updates_only_matching_parameters(gpu):
+    from jabas_amd import optim
+    from jabas_amd.train.trainer import tag_parameter_indices
+    model = tag_parameter_indices(_mlp(1).to(gpu))
+    ref_model = copy.deepcopy(model)
+    params = list(model.parameters())
+    opt = optim.ShardAdamW(_groups(model), lr=5e-4)
+    ref = torch.optim.AdamW(_groups(ref_model), lr=5e-4, foreach=False)
+    before = [p.detach().clone() for p in params]
+    # a "bucket": one flat buffer carrying the gradients of parameters 2..5, views tagged by index;
+    # parameter 3 has 33 elements, so the views after it start off a 16-byte line
+    chosen = [2, 3, 4, 5]
+    flat = torch.randn(sum(params[i].numel() for i in chosen), device=gpu) * 1e-2
+    grads, off = [], 0
+    for i in chosen:
+        v = flat[off:off + params[i].numel()].view_as(params[i])
+        v.index = i
+        grads.append(v)
+        off += params[i].numel()
+    opt.step(grads)
+    torch.cuda.synchronize()
+    for i, (p, rp) in enumerate(zip(params, ref_model.parameters())):
+        rp.grad = grads[chosen.index(i)].clone() if i in chosen else None
+    ref.step()
+    for i, (p, rp) in enumerate(zip(params, ref_model.parameters())):
+        if i in chosen:
+            assert _close(p, rp, 1e-6, 1e-8), i
+            assert not torch.equal(p, before[i])
+        else:
+            assert torch.equal(p, before[i]), i
+            assert len(opt.state[p]) == 0
+
+
+def test_k_vsw_rendezvous_with_streams_and_threads(gpu):
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+
+    class Bucket:
+        def __init__(self, i, t):
+            self._i, self._t = i, t
+
+        def index(self):
+            return self._i
+
+        def buffer(self):
+            return self._t
+
+    K, batches, sizes = 3, (4, 2, 2), [40001, 7, 250000]
+    host = [[torch.randn(n, generator=torch.Generator().manual_seed(100 * b + k)) * 1e-3 for k in range(K)]
+            for b, n in enumerate(sizes)]
+    local = LocalBucketSync(batches)
+    st = H.GradientSimilarityState(None, 4, None, [], 1).attach_local(local)
+    main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    dev = [[None] * K for _ in sizes]
+    futs = {}
+
+    def vsw(k):
+        with torch.cuda.stream(streams[k]):
+            order = range(len(sizes)) if k % 2 == 0 else reversed(range(len(sizes)))
+            for b in order:
+                dev[b][k] = host[b][k].to(gpu, non_blocking=False)          # "backward" fills the bucket on this stream
+                bucket = Bucket(b, dev[b][k])
+                futs[(k, b)] = main_hook(st, bucket) if k == 0 else H.dummy_hook(H.VSWPeerState(local, k), bucket)
+
+    threads = [threading.Thread(target=vsw, args=(k,)) for k in range(K)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for f in futs.values():
+        f.wait()
+    local.finish_step(streams)
+    torch.cuda.synchronize()
+    for b in range(len(sizes)):
+        want = O.aggregate(host[b], batches)
+        assert torch.equal(dev[b][0].cpu().view(torch.int32), want.view(torch.int32)), b
+        for k in range(1, K):
+            assert torch.equal(dev[b][k].cpu(), host[b][k])
+    rows = {s.index: s.cpu() for s in st.grad_placeholder}
+    assert sorted(rows) == [0, 1, 2]
+    for b in range(len(sizes)):
+        want = O.stats(host[b], batches)
+        assert _close(rows[b][:4 + K], want[:4 + K], 1e-6, 0.0)
+    whole = O.cosine_from_rows(torch.stack([O.stats(host[b], batches) for b in range(len(sizes))]))
+    assert H.cosine_similarity_from_placeholder(st.grad_placeholder) == pytest.approx(whole, rel=1e-9)
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind):
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (6, 2)
+    if kind == "sgd":
+        opt = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+                   groups=[dict(lr=0.05, weight_decay=0.0), dict(lr=0.05, weight_decay=0.05)])
+    else:
+        opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+                   groups=[dict(lr=1e-3, weight_decay=0.0), dict(lr=1e-3, weight_decay=0.05)])
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, opt, interval=2, param_groups_func=_groups)
+    trainer.prepare_stream_parallel(_mlp(3), crit)
+    ref_model = _mlp(3).to(gpu)
+    groups = _groups(ref_model)
+    if kind == "sgd":
+        ref_opt = torch.optim.SGD(groups, lr=0.05, momentum=0.9, foreach=False)
+    else:
+        ref_opt = torch.optim.AdamW(groups, lr=1e-3, foreach=False)
+    w, _, _ = O.batch_weights(batches)
+    for step in range(1, 5):
+        gen = torch.Generator().manual_seed(step)
+        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        trainer.compute(data)
+        # plain torch: per-VSW gradients with the same weights, batch-weighted sum, optimizer step
+        per_vsw = []
+        for x, y in data:
+            ref_model.zero_grad(set_to_none=True)
+            crit(ref_model(x), y).backward()
+            per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(per_vsw[0][i], w[0]), torch.mul(per_vsw[1][i], w[1]))
+        if trainer.similarity_state.step % 2 == 0:
+            flat = [torch.cat([g.reshape(-1) for g in gs]) for gs in per_vsw]
+            want_cos = torch.nn.functional.cosine_similarity(flat[0].double(), flat[1].double(), dim=0).item()
+        ref_opt.step()
+        stat_step = trainer.similarity_state.step % 2 == 0
+        trainer.step()
+        torch.cuda.synchronize()
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), f"{kind} step {step}"
+        for m in trainer.local_models[1:]:
+            for p, q in zip(m.parameters(), trainer.main_model.parameters()):
+                assert torch.equal(p, q)                       # replicas refreshed by the same launch
+        if stat_step:
+            assert float(trainer.cos_placeholder) == pytest.approx(want_cos, rel=1e-6)
+    assert trainer.similarity_state.step == 5

@@ -1,0 +1,258 @@
+"""Comm-hook protocol on the CPU: gating, placeholders, future chaining and the K-VSW
+rendezvous, with fake bucket objects and a recording launcher in place of the kernel
+(restated from jabas/ddp_comm_hooks/similarity_allreduce.py:8-45 and
+jabas/train/trainer.py:184-195,452-468,480)."""
+import random
+import threading
+
+import pytest
+import torch
+
+from jabas_amd import ddp_comm_hooks as H
+from jabas_amd.local_sync import LocalBucketSync, BucketStats
+from jabas_amd.train import create_optimizer_hook
+from jabas_amd import optim
+
+
+class NewBucket:
+    """torch >= 1.10 GradBucket flavour."""
+
+    def __init__(self, index, tensor, params=()):
+        self._i, self._t, self._p = index, tensor, list(params)
+
+    def index(self):
+        return self._i
+
+    def buffer(self):
+        return self._t
+
+    def parameters(self):
+        return self._p
+
+    def gradients(self):
+        out, off = [], 0
+        for p in self._p:
+            out.append(self._t[off:off + p.numel()].view_as(p))
+            off += p.numel()
+        return out
+
+
+class OldBucket:
+    """torch 1.8.1 _GradBucket flavour the reference was written against."""
+
+    def __init__(self, index, tensor):
+        self._i, self._t = index, tensor
+
+    def get_index(self):
+        return self._i
+
+    def get_tensors(self):
+        return [self._t]
+
+
+class Recorder:
+    def __init__(self):
+        self.calls = []
+
+    def __call__(self, bucket_index, tensors, want_stats):
+        self.calls.append((bucket_index, [t.clone() for t in tensors], want_stats))
+        tensors[0].copy_(sum(tensors))                     # stands in for the in-place aggregate
+        return torch.full((12,), float(bucket_index), dtype=torch.float64) if want_stats else None
+
+
+def test_similarity_state_fields_follow_the_reference():
+    st = H.GradientSimilarityState("pg", 8, "sub", [], 100)
+    assert st.step == 1 and st.interval == 100
+    assert st.subgroup_total_num_decoupled_workers == 4
+    assert st.total_num_decoupled_workers == 8 and st.sub_group == "sub" and st.process_group == "pg"
+    with pytest.raises(AssertionError):
+        H.GradientSimilarityState("pg", 3, "sub", [], 100)
+
+
+@pytest.mark.parametrize("make", [NewBucket, OldBucket])
+def test_subgroup_hook_is_pass_through_off_interval(make):
+    st = H.GradientSimilarityState(None, 2, None, [], 5)
+    t = torch.arange(4.0)
+    b = make(0, t)
+    for step in (1, 2, 3, 4):
+        st.step = step
+        v = H.subgroup_allreduce_hook(st, b).wait()
+        v = v[0] if isinstance(v, list) else v
+        assert v is t and st.grad_placeholder == []
+    assert isinstance(H.subgroup_allreduce_hook(st, OldBucket(0, t)).wait(), list)
+    assert isinstance(H.subgroup_allreduce_hook(st, NewBucket(0, t)).wait(), torch.Tensor)
+
+
+def test_dummy_hook_without_state_passes_the_bucket_through():
+    t = torch.ones(3)
+    assert H.dummy_hook(None, NewBucket(0, t)).wait() is t
+    assert H.dummy_hook(None, OldBucket(0, t)).wait()[0] is t
+
+
+def test_allreduce_sum_fut_single_process_is_identity():
+    t = torch.ones(3)
+    out = H._allreduce_sum_fut(None, t).wait()
+    assert isinstance(out, list) and out[0] is t
+
+
+def test_iidp_hook_needs_a_local_sync_unless_there_is_one_worker():
+    t = torch.ones(3)
+    assert H.iidp_allreduce_hook(H.IIDPState(None, 1), NewBucket(0, t)).wait() is t
+    with pytest.raises(RuntimeError):
+        H.iidp_allreduce_hook(H.IIDPState(None, 4), NewBucket(0, t))
+
+
+def _wire(K, interval, recorder):
+    local = LocalBucketSync([4] * K, launcher=recorder)
+    st = H.GradientSimilarityState(None, K if K % 2 == 0 else K + 1, None, [], interval).attach_local(local)
+    main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
+    peers = [H.VSWPeerState(local, k) for k in range(1, K)]
+    return local, st, main_hook, peers
+
+
+def test_main_vsw_first_does_not_block_and_fires_once_when_all_arrived():
+    K, rec = 3, Recorder()
+    local, st, main_hook, peers = _wire(K, 2, rec)
+    grads = [torch.full((5,), float(k + 1)) for k in range(K)]
+    st.step = 2                                            # statistic step
+    fut0 = main_hook(st, NewBucket(7, grads[0]))
+    assert not fut0.done() and rec.calls == [] and local.pending() == [7]
+    f1 = H.dummy_hook(peers[0], NewBucket(7, grads[1]))
+    assert not f1.done() and rec.calls == []
+    f2 = H.dummy_hook(peers[1], NewBucket(7, grads[2]))
+    assert fut0.done() and f1.done() and f2.done()
+    assert len(rec.calls) == 1
+    idx, seen, want = rec.calls[0]
+    assert idx == 7 and want is True
+    assert [float(t[0]) for t in seen] == [1.0, 2.0, 3.0]   # VSW order, whatever the arrival order
+    assert torch.equal(fut0.value(), torch.full((5,), 6.0)) and fut0.value() is grads[0]
+    assert f1.value() is grads[1]
+    assert len(st.grad_placeholder) == 1 and isinstance(st.grad_placeholder[0], BucketStats)
+    assert st.grad_placeholder[0].index == 7
+    local.finish_step()
+    assert local.step_count == 1
+
+
+def test_off_interval_steps_do_not_ask_for_statistics_nor_fill_the_placeholder():
+    K, rec = 2, Recorder()
+    local, st, main_hook, peers = _wire(K, 100, rec)
+    for step in (1, 2, 3):
+        st.step = step
+        g = [torch.ones(4), torch.ones(4)]
+        H.dummy_hook(peers[0], OldBucket(0, g[1]))
+        out = main_hook(st, OldBucket(0, g[0])).wait()
+        assert isinstance(out, list) and torch.equal(out[0], torch.full((4,), 2.0))
+        local.finish_step()
+    assert [c[2] for c in rec.calls] == [False, False, False]
+    assert st.grad_placeholder == []
+
+
+def test_trainer_side_placeholder_reset_and_step_counter():
+    # the trainer empties grad_placeholder after reading it and bumps state.step (trainer.py:480,194-195)
+    K, rec = 2, Recorder()
+    local, st, main_hook, peers = _wire(K, 3, rec)
+    stat_steps = []
+    for step in range(1, 10):
+        st.step = step
+        for b in (0, 1):
+            H.dummy_hook(peers[0], NewBucket(b, torch.ones(2)))
+            main_hook(st, NewBucket(b, torch.ones(2))).wait()
+        local.finish_step()
+        if st.step % st.interval == 0:
+            assert [s.index for s in st.grad_placeholder] == [0, 1]
+            stat_steps.append(step)
+            st.grad_placeholder.clear()
+        else:
+            assert st.grad_placeholder == []
+    assert stat_steps == [3, 6, 9]
+
+
+def test_threads_in_random_order_over_many_buckets():
+    K, nb, rec = 4, 12, Recorder()
+    local, st, main_hook, peers = _wire(K, 1, rec)
+    grads = [[torch.full((3,), float(10 * b + k)) for k in range(K)] for b in range(nb)]
+    futures, lock = {}, threading.Lock()
+
+    def vsw(k):
+        order = list(range(nb))
+        random.Random(k).shuffle(order)
+        for b in order:
+            if k == 0:
+                f = main_hook(st, NewBucket(b, grads[b][0]))
+            else:
+                f = H.dummy_hook(peers[k - 1], NewBucket(b, grads[b][k]))
+            with lock:
+                futures[(k, b)] = f
+
+    threads = [threading.Thread(target=vsw, args=(k,)) for k in range(K)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert all(f.done() for f in futures.values())
+    assert sorted(c[0] for c in rec.calls) == list(range(nb))
+    for b in range(nb):
+        assert float(grads[b][0][0]) == sum(10 * b + k for k in range(K))
+    assert sorted(s.index for s in st.grad_placeholder) == list(range(nb))
+    local.finish_step()
+
+
+def test_finish_step_reports_missing_vsws_and_double_publish_is_an_error():
+    local = LocalBucketSync([1, 1], launcher=Recorder())
+    local.publish(0, 3, torch.ones(2))
+    with pytest.raises(RuntimeError, match="not published"):
+        local.finish_step()
+    with pytest.raises(RuntimeError, match="twice"):
+        local.publish(0, 3, torch.ones(2))
+    with pytest.raises(ValueError):
+        local.publish(2, 3, torch.ones(2))
+
+
+def test_launcher_failure_reaches_every_waiting_hook():
+    def boom(*a):
+        raise RuntimeError("launch refused")
+    local = LocalBucketSync([1, 1], launcher=boom)
+    f0 = local.publish(0, 0, torch.ones(2))
+    f1 = local.publish(1, 0, torch.ones(2))
+    for f in (f0, f1):
+        with pytest.raises(RuntimeError, match="launch refused"):
+            f.wait()
+
+
+def test_optimizer_hook_steps_the_bucket_parameters_after_the_comm_hook():
+    class FakeOpt:
+        def __init__(self):
+            self.seen = []
+
+        def step(self, gradients):
+            self.seen.append([(g.index, g.clone()) for g in gradients])
+
+    p0, p1 = torch.nn.Parameter(torch.zeros(2, 2)), torch.nn.Parameter(torch.zeros(3))
+    p0.index, p1.index = 5, 6
+    flat = torch.arange(7.0)
+    opt = FakeOpt()
+    hook = create_optimizer_hook(lambda state, bucket: H.dummy_hook(None, bucket), opt)
+    out = hook(None, NewBucket(0, flat, [p0, p1])).wait()
+    assert out is flat
+    assert [i for i, _ in opt.seen[0]] == [5, 6]
+    assert torch.equal(opt.seen[0][0][1], flat[:4].view(2, 2)) and torch.equal(opt.seen[0][1][1], flat[4:])
+
+
+def test_shard_optimizer_constructors_validate_like_torch():
+    p = [torch.nn.Parameter(torch.zeros(4))]
+    with pytest.raises(ValueError):
+        optim.ShardSGD(p, lr=-1.0)
+    with pytest.raises(ValueError):
+        optim.ShardSGD(p, lr=0.1, momentum=0.0, nesterov=True)
+    with pytest.raises(ValueError):
+        optim.ShardAdam(p, betas=(1.0, 0.999))
+    with pytest.raises(ValueError):
+        optim.ShardAdamW(p, eps=-1e-8)
+    o = optim.ShardAdamW(p)
+    assert o.defaults["weight_decay"] == 1e-2 and optim.ShardAdam(p).defaults["weight_decay"] == 0
+    p[0].grad = torch.ones(4)
+    with pytest.raises(RuntimeError, match="GPU"):
+        optim.ShardSGD(p, lr=0.1).step()                       # no CPU fallback
+    g = torch.ones(4)
+    with pytest.raises(ValueError, match="index"):
+        optim.ShardSGD(p, lr=0.1).step([g])
