@@ -44,7 +44,7 @@ typedef enum JabasStatus {
     JABAS_OK = 0,
     JABAS_ERR_NULL = -1,        /* a required pointer is NULL                          */
     JABAS_ERR_K = -2,           /* K outside 1..JABAS_MAX_K                            */
-    JABAS_ERR_ALIGN = -3,       /* buffers of a span are not mutually 16-byte congruent*/
+    JABAS_ERR_ALIGN = -3,       /* buffers of a span sit at different line positions   */
     JABAS_ERR_DTYPE = -4,       /* grad_dtype is neither JABAS_F32 nor JABAS_BF16      */
     JABAS_ERR_OPT = -5,         /* unknown optimizer kind or inconsistent state ptrs   */
     JABAS_ERR_GROUP = -6,       /* group index / count out of range, unsorted bounds   */
@@ -71,9 +71,10 @@ enum {
 };
 
 /* One contiguous stretch of the flat layout. All buffers hold `numel` elements and are
- * indexed alike. Their addresses must be congruent modulo 16 bytes in element terms
- * (element e of every buffer falls at the same position of a 16-byte line), which holds
- * whenever they are views at one element offset into 16-byte aligned arenas.
+ * indexed alike. Element e of every fp32 buffer must fall at the same position of a
+ * 16-byte line, and of every bf16 gradient buffer at the same position of an 8-byte line
+ * ((address / element size) mod 4 equal for all buffers), which holds whenever they are
+ * views at one element offset into 16-byte aligned arenas.
  * agg_out may alias grads[0] when the gradients are fp32 (in-place bucket update).
  * Unused pointers are NULL. */
 typedef struct JabasSpan {
