@@ -1,0 +1,181 @@
+"""The five benchmark configurations at their full sizes on the GPU, checked through
+size-independent properties and through the oracle on sampled windows:
+
+  * sampled windows (8 x 64 Ki elements, incl. the first and last of the arena): aggregate
+    bit-exact, weights/state within 1e-6 of the oracle after two steps;
+  * power-of-two scaling of every gradient scales the aggregate exactly (linearity);
+  * checksum: sum(aggregate) = sum_k w_k sum(g_k) within rounding;
+  * statistics: per-bucket rows add up to the row of one whole-arena span; per-worker norms
+    equal a float64 library reduction; bit-identical across two runs;
+  * exact-zero gradient rows (GNMT embedding) stay +0 in the aggregate and leave Adam's
+    weights untouched on the first step;
+  * first Adam step is the closed-form sign step where weight decay is 0;
+  * every replica's weights equal the main weights (fan-out).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+WINDOW = 65536
+
+
+def _fill(eng, cfg, seed):
+    from jabas_amd import workloads as W
+    dev = eng.device
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    live = torch.zeros(eng.layout.total, dtype=torch.bool, device=dev)       # padding between buckets stays zero
+    for off, n, _, _ in eng.layout.spans:
+        live[off:off + n] = True
+    for k in range(eng.K):
+        t = torch.randn(eng.layout.total, generator=gen, device=dev) * cfg.grad_std
+        eng.grads[k].copy_(torch.where(live, t, torch.zeros((), device=dev)).to(eng.grad_dtype))
+    eng.param.copy_(torch.where(live, torch.randn(eng.layout.total, generator=gen, device=dev) * 0.05,
+                                torch.zeros((), device=dev)))
+    if cfg.name == "gnmt":
+        i = [s.name for s in cfg.specs].index(W.GNMT_EMBEDDING)
+        keep = (torch.rand(W.GNMT_EMBEDDING_ROWS, generator=torch.Generator().manual_seed(0)) < 0.1).to(dev)
+        for k in range(eng.K):
+            v = eng.grad_view(k, i).view(W.GNMT_EMBEDDING_ROWS, W.GNMT_EMBEDDING_COLS)
+            v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=dev, dtype=v.dtype)))
+        return i, keep
+    return None, None
+
+
+def _windows(eng):
+    """Windows inside spans (so the oracle sees the same group bounds)."""
+    rng = np.random.RandomState(7)
+    out = []
+    spans = eng.layout.spans
+    picks = [0, len(spans) - 1] + list(rng.randint(0, len(spans), size=6))
+    for si in picks:
+        off, n, bounds, _ = spans[si]
+        w = min(WINDOW, n)
+        start = 0 if si == 0 else (n - w if si == len(spans) - 1 else int(rng.randint(0, n - w + 1)))
+        out.append((off, n, bounds, start, w))
+    return out
+
+
+def _window_bounds(bounds, start, w):
+    """Group bounds of span-local range [start, start+w), rebased to the window."""
+    b = [(0, [g for s, g in bounds if s <= start][-1])] if bounds else [(0, 0)]
+    for s, g in bounds:
+        if start < s < start + w:
+            b.append((s - start, g))
+    return tuple(b)
+
+
+def _close(a, b, rtol, atol):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    return bool(((a - b).abs() <= rtol * b.abs() + atol).all())
+
+
+@pytest.mark.parametrize("name", ["resnet50", "vit_b16", "faster_rcnn_r50_fpn", "gnmt", "vit_l16"])
+def test_full_size_configuration(gpu, name):
+    from jabas_amd import workloads as W, sync
+    from jabas_amd.engine import VSWFlatSync
+    cfg = W.config(name)
+    gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
+    print(f"full size {name}: {sum(s.numel for s in cfg.specs)} elements K={cfg.K}", flush=True)
+    eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=gpu, n_fanout=1)
+    emb, keep = _fill(eng, cfg, 11)
+    wins = _windows(eng)
+    adam = cfg.opt["kind"] != "sgd"
+    # host copies of the sampled windows before the step
+    host = []
+    for off, n, bounds, start, w in wins:
+        sl = slice(off + start, off + start + w)
+        host.append(dict(g=[g[sl].cpu() for g in eng.grads], p=eng.param[sl].cpu(),
+                         s1=torch.zeros(w), s2=torch.zeros(w), bounds=_window_bounds(bounds, start, w)))
+    g_sums = [g.double().sum().item() for g in eng.grads]
+    g_abs = sum(g.double().abs().sum().item() * wk for g, wk in zip(eng.grads, O.batch_weights(cfg.batches)[0]))
+    norms = [(g.double() ** 2).sum().item() for g in eng.grads]
+    p0 = eng.param.clone()
+    g_before = [g.clone() for g in eng.grads]
+
+    rows = eng.step(stats=True)
+    torch.cuda.synchronize()
+    rows1 = rows.cpu().clone()
+
+    # ---- sampled windows against the oracle, step 1
+    for h, (off, n, bounds, start, w) in zip(host, wins):
+        sl = slice(off + start, off + start + w)
+        agg_h, _ = O.sync_step(h["g"], cfg.batches, [(0, w, h["bounds"])], cfg.opt, h["p"], h["s1"],
+                               h["s2"] if adam else None, step=1, first_step=True)
+        assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h.view(torch.int32)), (name, off, start)
+        assert _close(eng.param[sl], h["p"], 1e-6, 1e-9)
+        assert _close(eng.state1[sl], h["s1"], 1e-6, 2e-9)
+        if adam:
+            assert _close(eng.state2[sl], h["s2"], 1e-6, 1e-16)
+        h["agg"] = agg_h
+
+    # ---- checksum of the aggregate
+    w = O.batch_weights(cfg.batches)[0]
+    want_sum = sum(wk * s for wk, s in zip(w, g_sums))
+    got_sum = eng.agg.double().sum().item()
+    assert abs(got_sum - want_sum) <= 1e-6 * g_abs + 1e-12
+
+    # ---- statistics
+    whole = rows1.sum(0)
+    for k in range(cfg.K):
+        assert whole[4 + k].item() == pytest.approx(norms[k], rel=1e-10)
+    assert whole[3].item() == pytest.approx((eng.agg.double() ** 2).sum().item(), rel=1e-10)
+    one_span = sync.gradient_stats(g_before, cfg.batches).cpu()          # one span over the whole arena
+    assert torch.allclose(whole[:4 + cfg.K], one_span[:4 + cfg.K], rtol=1e-11, atol=0.0)
+    cos = sync.cosine_from_stats(rows1)
+    assert -1.0 <= cos <= 1.0
+
+    # ---- fan-out and closed forms
+    assert torch.equal(eng.fanout[0], eng.param)
+    if adam:
+        # groups without weight decay: p1 = p0 - lr * g / (|g| + eps); AdamW scales p0 by (1 - lr*wd) elsewhere
+        for off, n, bounds, _ in eng.layout.spans[:3]:
+            for j, (s, grp) in enumerate(bounds):
+                e = bounds[j + 1][0] if j + 1 < len(bounds) else n
+                hp = cfg.opt["groups"][grp]
+                if hp["weight_decay"] != 0.0:
+                    continue
+                sl = slice(off + s, off + e)
+                g = eng.agg[sl].double()
+                want = p0[sl].double() - hp["lr"] * g / (g.abs() + 1e-8)
+                assert torch.allclose(eng.param[sl].double(), want, rtol=2e-6, atol=1e-9)
+    if emb is not None:
+        rows_, cols_ = keep.numel(), W.GNMT_EMBEDDING_COLS
+        a = eng.agg_view(emb).view(rows_, cols_)
+        assert torch.all(a[~keep].view(torch.int32) == 0)                # exact +0 rows
+        pv, p0v = eng.param_view(emb).view(rows_, cols_), eng._view(p0, emb).view(rows_, cols_)
+        assert torch.equal(pv[~keep], p0v[~keep])                        # zero gradient, zero moments: no update
+        assert torch.count_nonzero(eng._view(eng.state1, emb).view(rows_, cols_)[~keep]) == 0
+
+    # ---- second step on the sampled windows (moments now non-zero)
+    if gdt == torch.float32:
+        for h, (off, n, bounds, start, w_) in zip(host, wins):
+            h["g"][0] = h["agg"].clone()                                 # in place: VSW 0's bucket holds the aggregate
+    eng.step(stats=False)
+    torch.cuda.synchronize()
+    for h, (off, n, bounds, start, w_) in zip(host, wins):
+        sl = slice(off + start, off + start + w_)
+        agg_h, _ = O.sync_step(h["g"], cfg.batches, [(0, w_, h["bounds"])], cfg.opt, h["p"], h["s1"],
+                               h["s2"] if adam else None, step=2, first_step=False)
+        assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h.view(torch.int32))
+        assert _close(eng.param[sl], h["p"], 1e-6, 1e-9)
+        assert _close(eng.state1[sl], h["s1"], 1e-6, 2e-9)
+
+    # ---- linearity under power-of-two scaling and run-to-run determinism, on fresh engines
+    del eng
+    torch.cuda.empty_cache()
+    a = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=None, device=gpu, in_place=False)
+    for k in range(cfg.K):
+        a.grads[k].copy_(g_before[k])
+    r1 = a.step(stats=True).cpu().clone()
+    agg1 = a.agg.clone()
+    r2 = a.step(stats=True).cpu().clone()
+    assert torch.equal(r1.view(torch.int64), r2.view(torch.int64))       # same plan, same bits
+    for k in range(cfg.K):
+        a.grads[k].mul_(4.0)
+    a.step(stats=False)
+    torch.cuda.synchronize()
+    assert torch.equal((agg1 * 4.0).view(torch.int32), a.agg.view(torch.int32))
