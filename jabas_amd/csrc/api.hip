@@ -17,7 +17,7 @@ namespace {
 
 constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 2;
+constexpr uint32_t kPlanVersion = 3;
 
 struct PlanHeader {
     uint32_t magic, version;
@@ -25,9 +25,11 @@ struct PlanHeader {
     int32_t K, grad_dtype, opt_kind;
     uint32_t max_group;       // largest group index any bound names
     uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
+    uint32_t chunk_tiles;     // tiles per workgroup the chunk table was cut for
+    uint32_t pad;
     uint64_t off_spans, off_prefix, off_chunks, off_bounds, total_bytes;
 };
-static_assert(sizeof(PlanHeader) == 80, "plan header layout");
+static_assert(sizeof(PlanHeader) == 88, "plan header layout");
 constexpr size_t kHeaderBytes = 96;
 
 inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
@@ -55,7 +57,7 @@ inline uint64_t span_tiles(const JabasSpan& in, int grad_dtype) {
     const uint64_t te = tile_elems(grad_dtype);
     return (skew + in.numel + te - 1) / te;
 }
-inline uint64_t chunks_of_tiles(uint64_t tiles) { return (tiles + kChunkTiles - 1) / kChunkTiles; }
+inline uint64_t chunks_of_tiles(uint64_t tiles, uint64_t ct) { return (tiles + ct - 1) / ct; }
 
 // Validates one span and produces the rebased device view. Host-only logic.
 int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDev* out, uint32_t* tiles) {
@@ -281,13 +283,13 @@ JABAS_API size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype) 
     const int dt = grad_dtype == JABAS_BF16 ? JABAS_BF16 : JABAS_F32;
     const uint64_t te = tile_elems(dt);
     const uint64_t tiles = (numel + ept_of(dt) - 1 + te - 1) / te;
-    return static_cast<size_t>(chunks_of_tiles(tiles) + 1) * kStatsStride * sizeof(double);
+    return static_cast<size_t>(chunks_of_tiles(tiles, kMinChunkTiles) + 1) * kStatsStride * sizeof(double);
 }
 
 namespace {
-uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype) {
+uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype, uint64_t ct) {
     uint64_t n = 0;
-    for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype));
+    for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype), ct);
     return n;
 }
 size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
@@ -300,7 +302,7 @@ size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
 
 JABAS_API size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds, int32_t grad_dtype) {
     if (!spans || (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16)) return 0;
-    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype));
+    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype, kMinChunkTiles));
 }
 
 JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
@@ -315,7 +317,8 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     if (opt_class_of(opt_kind) < 0) return JABAS_ERR_OPT;
     for (uint32_t i = 0; i < n_span; ++i)
         if (spans[i].numel && !spans[i].grads[0]) return JABAS_ERR_NULL;
-    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype);
+    const uint32_t ct = pick_chunk_tiles(K);
+    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype, ct);
     if (n_chunks > 0x7fffffffull) return JABAS_ERR_SIZE;
     const size_t need = plan_bytes_for(n_span, n_bounds, n_chunks);
     if (blob_bytes < need) return JABAS_ERR_PLAN;
@@ -333,6 +336,7 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     h.K = K;
     h.grad_dtype = grad_dtype;
     h.opt_kind = opt_kind;
+    h.chunk_tiles = ct;
     h.off_spans = kHeaderBytes;
     h.off_prefix = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
     h.off_chunks = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
@@ -354,7 +358,7 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
         if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
         prefix[i] = c;
         uint32_t j = 0;
-        for (uint32_t t0 = 0; t0 < tiles; t0 += kChunkTiles, ++c) {
+        for (uint32_t t0 = 0; t0 < tiles; t0 += ct, ++c) {
             cd[c].span = i;
             cd[c].tile0 = t0;
             if (spans[i].bound_count) {       // bound entry covering the chunk's first live element
@@ -411,6 +415,7 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     a.bounds = h.n_bounds ? reinterpret_cast<const BoundDev*>(dev + h.off_bounds) : nullptr;
     a.n_span = h.n_span;
     a.n_chunks = h.n_chunks;
+    a.chunk_tiles = h.chunk_tiles;
     a.use_inline = 0;
     return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
@@ -435,7 +440,8 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.chunks = nullptr;
     a.chunk_prefix = nullptr;
     a.n_span = 1;
-    a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles));
+    a.chunk_tiles = pick_chunk_tiles(args->K);
+    a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, a.chunk_tiles));
     a.use_inline = 1;
     return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }

@@ -3,7 +3,7 @@
 // streams are fully unrolled into independent 128-bit loads.
 //
 // Execution shape
-//   - one 256-thread workgroup (4 wave64) per chunk of kChunkTiles consecutive tiles of
+//   - one 256-thread workgroup (4 wave64) per chunk of 2 or 4 consecutive tiles of
 //     one span; a tile is 256 threads x 4 elements (one 16-byte vector of every fp32
 //     buffer, one 8-byte vector of a bf16 gradient buffer). Small, short-lived workgroups dispatched in order keep the part of every
 //     buffer that is being streamed at any moment compact, which on MI355X sustains a
@@ -27,8 +27,8 @@
 #ifndef JABAS_K
 #error "compile with -DJABAS_K=<1..8>"
 #endif
-// Tiles whose loads are in flight together: the whole chunk without statistics, half of
-// it with (the fp64 accumulators need the registers).
+// Most tiles whose loads are in flight together: a whole 4-tile chunk without statistics,
+// 2 tiles with (the fp64 accumulators need the registers).
 #ifndef JABAS_UNROLL_PLAIN
 #define JABAS_UNROLL_PLAIN 4
 #endif
@@ -220,7 +220,8 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
     }
 }
 
-// Vector path over nfull consecutive full tiles of one parameter group.
+// Vector path over nfull consecutive full tiles of one parameter group: groups of U tiles,
+// then U/2, ... down to single tiles.
 template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
                                          const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
@@ -233,13 +234,7 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
         issue_loads<K, DT, OPT, U>(r, sp, e, load_s1);
         consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, use_s1, load_s1, acc);
     }
-    if constexpr (U > 1) {
-        for (; i < nfull; ++i, e += TE) {
-            TileRegs<K, DT, 1> r;
-            issue_loads<K, DT, OPT, 1>(r, sp, e, load_s1);
-            consume<K, DT, OPT, STATS, HD, 1>(r, sp, e, a, G, use_s1, load_s1, acc);
-        }
-    }
+    if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, acc);
 }
 
 // Scalar path for one tile that touches a span edge or a group change. tile_e0 is the
@@ -291,8 +286,9 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
-    constexpr int U = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
-    static_assert(U <= kChunkTiles, "a chunk is the unit of work of one workgroup");
+    constexpr int UW = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
+    constexpr int U = UW < pick_chunk_tiles(K) ? UW : pick_chunk_tiles(K);   // never more than a chunk holds
+    static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
     const uint32_t nb = sp.bound_count;
     const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
     uint32_t lt = lt0, j = j0;
@@ -338,24 +334,31 @@ __device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint3
     }
 }
 
+// Workgroup sum of NS per-thread accumulators -> one partial row. Through LDS rather than
+// wave shuffles: 12 stores + 16 loads per thread instead of ~18 DPP-and-add instructions per
+// value, which matters because a workgroup only covers a few thousand elements.
+//   stage 1  thread (v, part) adds entries part, part+16, ..., part+240 of value v (in order);
+//   stage 2  the 16 parts of a value sit in one 16-lane row: DPP row reduction.
+// The order is fixed, so the row is bit-identical from run to run.
 template <int NS>
 __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
-    __shared__ double red[kWaves][NS];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ double buf[NS][kBlock];
+    const int tid = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < NS; ++i) {
-        const double v = wave_sum_to_lane63(acc[i]);
-        if (lane == 63) red[wave][i] = v;
-    }
+    for (int i = 0; i < NS; ++i) buf[i][tid] = acc[i];
     __syncthreads();
-    if (threadIdx.x < kStatsStride) {          // unused slots of the row are written as zero
-        double s = 0.0;
-        if (threadIdx.x < NS) {
-            s = red[0][threadIdx.x];
+    if (tid < NS * 16) {
+        const int v = tid >> 4, part = tid & 15;
+        double s = buf[v][part];
 #pragma unroll
-            for (int w = 1; w < kWaves; ++w) s += red[w][threadIdx.x];
-        }
-        row[threadIdx.x] = s;
+        for (int i = 1; i < 16; ++i) s += buf[v][i * 16 + part];
+        s += dpp_move<0xB1, 0xf>(s);     // quad_perm [1,0,3,2]
+        s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
+        s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
+        s += dpp_move<0x140, 0xf>(s);    // row_mirror
+        if (part == 0) row[v] = s;
+    } else if (tid >= kBlock - (kStatsStride - NS)) {
+        row[NS + (tid - (kBlock - (kStatsStride - NS)))] = 0.0;     // unused slots of the row
     }
 }
 
@@ -371,8 +374,8 @@ __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
     if (a.use_inline) {
         const SpanDev& sp = a.span0;
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
-        const uint32_t lt0 = b * kChunkTiles;
-        const uint32_t lt1 = lt0 + kChunkTiles < tiles ? lt0 + kChunkTiles : tiles;
+        const uint32_t lt0 = b * a.chunk_tiles;
+        const uint32_t lt1 = lt0 + a.chunk_tiles < tiles ? lt0 + a.chunk_tiles : tiles;
         uint32_t j0 = 0;
         if (sp.bound_count) {                  // largest j with bounds[j].start <= first live element
             const BoundDev* bd = a.bounds + sp.bound_begin;
@@ -390,7 +393,7 @@ __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
         const ChunkDesc c = a.chunks[b];
         const SpanDev& sp = a.spans[c.span];
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
-        const uint32_t lt1 = c.tile0 + kChunkTiles < tiles ? c.tile0 + kChunkTiles : tiles;
+        const uint32_t lt1 = c.tile0 + a.chunk_tiles < tiles ? c.tile0 + a.chunk_tiles : tiles;
         run_chunk<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
     if constexpr (STATS) flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);

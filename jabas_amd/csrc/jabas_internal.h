@@ -10,7 +10,12 @@ namespace jabas {
 
 constexpr int kBlock = 256;                 // threads per workgroup = 4 wave64
 constexpr int kWaves = kBlock / 64;
-constexpr int kChunkTiles = 4;              // tiles one workgroup processes (a "chunk")
+constexpr int kMinChunkTiles = 2;           // a chunk = the tiles one workgroup processes: 2 or 4
+constexpr int kMaxChunkTiles = 4;
+// Small chunks keep the streamed window of every buffer compact (higher HBM rate) and cut
+// the ramp-up / drain of a launch; kernels with many gradient streams and statistics have
+// low occupancy and a long prologue, and do better with twice the work per workgroup.
+__host__ __device__ constexpr int pick_chunk_tiles(int K) { return K > 4 ? kMaxChunkTiles : kMinChunkTiles; }
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
 // Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer
@@ -18,7 +23,6 @@ constexpr int kStatsStride = JABAS_STATS_STRIDE;
 // contiguous).
 __host__ __device__ constexpr int ept_of(int /*grad_dtype*/) { return 4; }
 __host__ __device__ constexpr int tile_elems(int grad_dtype) { return kBlock * ept_of(grad_dtype); }
-__host__ __device__ constexpr int chunk_elems(int grad_dtype) { return kChunkTiles * tile_elems(grad_dtype); }
 
 // A span as the kernels see it. Pointers are rebased downwards by `lo` elements so that
 // element index 0 of every buffer is 16-byte aligned; [lo, hi) is the live range.
@@ -59,7 +63,7 @@ struct OptDev {
     int32_t has_momentum, first_step, nesterov, adamw;
 };
 
-// One workgroup's share of a planned launch: kChunkTiles consecutive tiles of one span.
+// One workgroup's share of a planned launch: chunk_tiles consecutive tiles of one span.
 struct ChunkDesc {
     uint32_t span;                           // index into the span table
     uint32_t tile0;                          // first tile, local to the span
@@ -75,8 +79,10 @@ struct KArgs {
     double* partials;                        // one row of kStatsStride doubles per workgroup
     uint32_t n_span;
     uint32_t n_chunks;
-    uint32_t use_inline;                     // 1: the only span is `span0`, chunk b starts at tile b*kChunkTiles
+    uint32_t chunk_tiles;                    // tiles per workgroup
+    uint32_t use_inline;                     // 1: the only span is `span0`, chunk b starts at tile b*chunk_tiles
     uint32_t half_mask;                      // bit k set: VSW k belongs to half B
+    uint32_t pad0;
     SpanDev span0;
     float w[JABAS_MAX_K];
     float wh[JABAS_MAX_K];

@@ -74,15 +74,20 @@ def _encode(spans, bounds=(), K=2, dtype=L.F32, opt=L.OPT_NONE):
     return rc, blob, nbytes
 
 
-def test_plan_encode_counts_chunks_of_4096_elements():
+def test_plan_encode_counts_chunks():
+    """A tile is 1024 elements; a workgroup takes 2 tiles for K <= 4 and 4 tiles above."""
     lib = L.lib()
-    rc, blob, _ = _encode([_span(4096), _span(4097), _span(1), _span(0), _span(10 * 4096 + 5)])
+    sizes = [4096, 4097, 1, 0, 10 * 4096 + 5]
+    rc, blob, _ = _encode([_span(n) for n in sizes])
+    assert rc == L.OK
+    assert lib.jabas_plan_chunks(blob.ctypes.data) == 2 + 3 + 1 + 0 + 21
+    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) == (27 + 1) * 12 * 8
+    rc, blob, _ = _encode([_span(n, K=8) for n in sizes], K=8)
     assert rc == L.OK
     assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
-    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) == (15 + 1) * 12 * 8
     # a span that starts 3 elements into a 16-byte line needs one more tile when it is exactly full
     rc, blob, _ = _encode([_span(4096, skew=3)])
-    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data) == 2
+    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data) == 3
 
 
 def test_plan_encode_bf16_positions_are_counted_in_elements():
@@ -155,8 +160,8 @@ def test_plan_blob_too_small_and_garbage_header():
 def test_workspace_bytes_cover_any_line_position():
     lib = L.lib()
     assert lib.jabas_sync_workspace_bytes(0, L.F32) >= 96
-    assert lib.jabas_sync_workspace_bytes(4096, L.F32) >= 2 * 96      # a shifted start can straddle two chunks
-    assert lib.jabas_sync_workspace_bytes(1 << 30, L.BF16) >= ((1 << 30) // 4096) * 96
+    assert lib.jabas_sync_workspace_bytes(4096, L.F32) >= 3 * 96      # a shifted start adds a chunk
+    assert lib.jabas_sync_workspace_bytes(1 << 30, L.BF16) >= ((1 << 30) // 2048) * 96
 
 
 def test_entry_points_validate_before_launching():
