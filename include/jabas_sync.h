@@ -121,6 +121,9 @@ typedef struct JabasStepArgs {
     double  momentum, dampening;        /* SGD                                         */
     double  beta1, beta2, eps;          /* Adam / AdamW                                */
     JabasGroup groups[JABAS_MAX_GROUPS];
+    const float* grad_scale;            /* device scalar c or NULL: when c < 1 the aggregate
+                                           is multiplied by c (one fp32 product) before it is
+                                           written and handed to the optimizer (clipping)  */
 } JabasStepArgs;
 
 /* Library identification. No reference counterpart. */
@@ -209,6 +212,16 @@ int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype,
 int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype,
                uint64_t numel, double* gram_out,
                void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* Global-norm clipping coefficient from statistics rows (device to device, no host sync):
+ *   total = sum over the n_rows rows of slot JABAS_STAT_NORM_AGG (in row order, fp64),
+ *   *coef_out = fp32(max_norm / (sqrt(total) + eps)).
+ * Feed coef_out to a later call as JabasStepArgs.grad_scale: the gradient is scaled only
+ * when the coefficient is below 1, as torch.nn.utils.clip_grad_norm_ does
+ * (examples/gnmt/seq2seq/train/trainer.py:157-161; clip_grad_norm_for_overlap in
+ * examples/gnmt/seq2seq/train/shard_optimizer.py:75-76). eps is 1e-6 there. */
+int jabas_clip_coef(const double* stats_rows, uint32_t n_rows, double max_norm, double eps,
+                    float* coef_out, jabas_stream_t stream);
 
 /* SGD step with a ready fp32 gradient (torch 1.8.1 optim/_functional.sgd as used by
  * examples/resnet50/main.py:351-359, examples/faster_r_cnn/train.py:266-276).

@@ -68,6 +68,7 @@ class JabasStepArgs(C.Structure):
         ("beta2", C.c_double),
         ("eps", C.c_double),
         ("groups", JabasGroup * MAX_GROUPS),
+        ("grad_scale", C.c_void_p),
     ]
 
 
@@ -92,6 +93,7 @@ SIGNATURES = {
                               C.c_void_p, C.c_size_t, C.c_void_p]),
     "jabas_gram": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.c_uint64, C.c_void_p,
                              C.c_void_p, C.c_size_t, C.c_void_p]),
+    "jabas_clip_coef": (C.c_int, [C.c_void_p, C.c_uint32, C.c_double, C.c_double, C.c_void_p, C.c_void_p]),
     "jabas_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double, C.c_double,
                             C.c_double, C.c_double, C.c_int32, C.c_int32, C.c_void_p]),
     "jabas_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double,

@@ -156,6 +156,7 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
         if (s->half_id[k]) mask |= 1u << k;
     }
     a->half_mask = mask;
+    a->grad_scale = s->grad_scale;
     if (oc == 0) return JABAS_OK;
     if (s->n_groups < 1 || s->n_groups > JABAS_MAX_GROUPS) return JABAS_ERR_GROUP;
     OptDev& o = a->opt;
@@ -228,6 +229,15 @@ __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const ui
         for (int w = 1; w < kFinalizeBlock / 64; ++w) sum += red[w][t];
         stats_out[static_cast<uint64_t>(s) * kStatsStride + t] = t < static_cast<uint32_t>(ns) ? sum : 0.0;
     }
+}
+
+// One wave: fixed-order sum of slot NORM_AGG over the rows, then the coefficient.
+__global__ void __launch_bounds__(64) clip_coef_kernel(const double* rows, uint32_t n_rows, double max_norm, double eps,
+                                                       float* coef_out) {
+    double acc = 0.0;
+    for (uint32_t r = threadIdx.x; r < n_rows; r += 64) acc += rows[static_cast<uint64_t>(r) * kStatsStride + JABAS_STAT_NORM_AGG];
+    const double total = wave_sum_to_lane63(acc);
+    if (threadIdx.x == 63) *coef_out = static_cast<float>(max_norm / (sqrt(total) + eps));
 }
 
 int run_fused(KArgs& a, const JabasStepArgs* s, double* stats_out, void* workspace, size_t workspace_bytes,
@@ -511,6 +521,17 @@ JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype
     if (launch_gram_finalize(K, static_cast<const double*>(workspace), static_cast<unsigned>(g), gram_out, st) != 0)
         return JABAS_ERR_LAUNCH;
     return JABAS_OK;
+}
+
+JABAS_API int jabas_clip_coef(const double* stats_rows, uint32_t n_rows, double max_norm, double eps, float* coef_out,
+                              jabas_stream_t stream) {
+    if (!stats_rows || !coef_out) return JABAS_ERR_NULL;
+    if (n_rows < 1) return JABAS_ERR_SIZE;
+    if (!(max_norm > 0.0) || eps < 0.0) return JABAS_ERR_OPT;
+    if (reinterpret_cast<uintptr_t>(stats_rows) % 8 || reinterpret_cast<uintptr_t>(coef_out) % 4) return JABAS_ERR_ALIGN;
+    hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), stats_rows, n_rows,
+                       max_norm, eps, coef_out);
+    return hipGetLastError() == hipSuccess ? JABAS_OK : JABAS_ERR_LAUNCH;
 }
 
 JABAS_API int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t numel, double lr,

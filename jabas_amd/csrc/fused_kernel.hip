@@ -107,12 +107,13 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
 template <int K, int N, int OPT, bool STATS, bool HD>
 __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
                                         float (&s2)[N], float (&agg)[N], const KArgs& a,
-                                        const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
+                                        const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         float s = g[0][i] * a.w[0];
 #pragma unroll
         for (int k = 1; k < K; ++k) s = s + g[k][i] * a.w[k];
+        if (clip < 1.0f) s = s * clip;         // global-norm clipping: only ever scales down
         agg[i] = s;
         if constexpr (STATS) {
             float ga = 0.0f, gb = 0.0f;
@@ -189,7 +190,7 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
 template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const KArgs& a,
-                                        const GroupDev& G, bool use_s1, bool load_s1,
+                                        const GroupDev& G, float clip, bool use_s1, bool load_s1,
                                         double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
@@ -209,7 +210,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
             }
             if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r.s2[u], s2);
         }
-        compute<K, EPT, OPT, STATS, HD>(g, p, s1, s2, agg, a, G, acc);
+        compute<K, EPT, OPT, STATS, HD>(g, p, s1, s2, agg, a, G, clip, acc);
         if (sp.out) store_vec<NV>(agg, sp.out, eu);
         if constexpr (OPT != OPT_NONE) {
             store_vec<NV>(p, sp.p, eu);
@@ -224,7 +225,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 // then U/2, ... down to single tiles.
 template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
-                                         const GroupDev& G, double (&acc)[NStats<K, STATS>::value]) {
+                                         const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
@@ -232,9 +233,9 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
     for (; i + U <= nfull; i += U, e += U * TE) {
         TileRegs<K, DT, U> r;
         issue_loads<K, DT, OPT, U>(r, sp, e, load_s1);
-        consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, use_s1, load_s1, acc);
+        consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, clip, use_s1, load_s1, acc);
     }
-    if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, acc);
+    if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, clip, acc);
 }
 
 // Scalar path for one tile that touches a span edge or a group change. tile_e0 is the
@@ -242,7 +243,7 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
 // first live element of the tile.
 template <int K, int DT, int OPT, bool STATS>
 __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const KArgs& a, uint32_t j,
-                                          double (&acc)[NStats<K, STATS>::value]) {
+                                             float clip, double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
@@ -268,7 +269,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
             if (load_s1) s1[0] = sp.s1[e];
             if constexpr (OPT == OPT_ADAM) s2[0] = sp.s2[e];
         }
-        compute<K, 1, OPT, STATS, false>(g, p, s1, s2, agg, a, G, acc);
+        compute<K, 1, OPT, STATS, false>(g, p, s1, s2, agg, a, G, clip, acc);
         if (sp.out) sp.out[e] = agg[0];
         if constexpr (OPT != OPT_NONE) {
             sp.p[e] = p[0];
@@ -283,6 +284,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 template <int K, int DT, int OPT, bool STATS, bool HD>
 __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
                                            const KArgs& a, double (&acc)[NStats<K, STATS>::value]) {
+    const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
@@ -311,10 +313,10 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
         }
         if (nfull) {
             const GroupDev G = a.groups[gid];
-            fast_run<K, DT, OPT, STATS, HD, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, acc);
+            fast_run<K, DT, OPT, STATS, HD, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, clip, acc);
             lt += nfull;
         } else {
-            careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, acc);
+            careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, clip, acc);
             lt += 1;
         }
     }

@@ -77,6 +77,7 @@ struct KArgs {
     const uint32_t* chunk_prefix;            // n_span + 1 entries: first chunk of each span (planned launch)
     const BoundDev* bounds;                  // device, may be NULL
     double* partials;                        // one row of kStatsStride doubles per workgroup
+    const float* grad_scale;                 // device scalar or NULL (clipping)
     uint32_t n_span;
     uint32_t n_chunks;
     uint32_t chunk_tiles;                    // tiles per workgroup

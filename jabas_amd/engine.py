@@ -12,7 +12,7 @@ import torch
 
 from . import _lib as L
 from .layout import FlatLayout
-from .sync import SpanSpec, SyncPlan, make_step_args, opt_kind, cosine_from_stats
+from .sync import SpanSpec, SyncPlan, make_step_args, opt_kind, cosine_from_stats, clip_coef
 
 
 class VSWFlatSync:
@@ -59,6 +59,7 @@ class VSWFlatSync:
                 bounds=bounds if kind != L.OPT_NONE else ()))
         self.span_bucket = [s[3] for s in self.layout.spans]
         self.plan = SyncPlan(spans, kind)
+        self._plan_agg = self._plan_opt = self._coef = None
         self.step_count = 0
 
     # ---- views -------------------------------------------------------------------
@@ -86,13 +87,41 @@ class VSWFlatSync:
         return make_step_args(self.batches, self.grad_dtype, stats=stats, opt=opt, step=self.step_count + 1,
                               first_step=first, lr_scale=lr_scale)
 
-    def step(self, stats=False, lr_scale=1.0, stream=None):
-        """One fused sync step over the whole gradient set. Returns the per-span stats
-        tensor when ``stats`` is set."""
-        args = self.step_args(stats=stats, lr_scale=lr_scale)
-        out = self.plan.run(args, stream=stream)
+    def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None):
+        """One sync step over the whole gradient set. Returns the per-span stats tensor
+        when ``stats`` is set.
+
+        Without ``clip_norm``: one fused launch. With it (global-norm clipping as
+        examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
+        clipping coefficient on the device, then the optimizer launch over the aggregate
+        scaled by it -- the norm has to be known before any weight moves."""
+        if clip_norm is None or self.opt is None:
+            args = self.step_args(stats=stats, lr_scale=lr_scale)
+            out = self.plan.run(args, stream=stream)
+            self.step_count += 1
+            return out
+        if self._plan_agg is None:
+            self._build_clip_plans()
+        rows = self._plan_agg.run(self.step_args(stats=True, with_opt=False), stream=stream)
+        coef = clip_coef(rows, clip_norm, out=self._coef, stream=stream)
+        args = make_step_args((1,), torch.float32, stats=False, opt=self.opt, step=self.step_count + 1,
+                              first_step=self.step_count == 0, lr_scale=lr_scale, grad_scale=coef)
+        self._plan_opt.run(args, stream=stream)
         self.step_count += 1
-        return out
+        return rows if stats else None
+
+    def _build_clip_plans(self):
+        agg_spans, opt_spans = [], []
+        for (off, numel, bounds, _bucket) in self.layout.spans:
+            sl = slice(off, off + numel)
+            agg_spans.append(SpanSpec([g[sl] for g in self.grads], agg_out=self.agg[sl]))
+            opt_spans.append(SpanSpec([self.agg[sl]], agg_out=self.agg[sl], param=self.param[sl],
+                                      state1=None if self.state1 is None else self.state1[sl],
+                                      state2=None if self.state2 is None else self.state2[sl],
+                                      fanout=[f[sl] for f in self.fanout], bounds=bounds))
+        self._plan_agg = SyncPlan(agg_spans, L.OPT_NONE)
+        self._plan_opt = SyncPlan(opt_spans, opt_kind(self.opt))
+        self._coef = torch.ones(1, dtype=torch.float32, device=self.device)
 
     def bucket_stats(self, stats):
         """Per-bucket rows from per-span rows (spans of one bucket summed in span order)."""

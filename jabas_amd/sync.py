@@ -65,7 +65,7 @@ def grad_dtype_code(dtype):
 
 
 def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_step=False, half_id=None,
-                   lr_scale=1.0):
+                   lr_scale=1.0, grad_scale=None):
     """Builds the JabasStepArgs of one call.
 
     ``opt``: None or dict(kind='sgd'|'adam'|'adamw', groups=[dict(lr=, weight_decay=)], plus
@@ -98,6 +98,11 @@ def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_ste
         b1, b2 = opt.get("betas", (0.9, 0.999))
         a.beta1, a.beta2 = float(b1), float(b2)
         a.eps = float(opt.get("eps", 1e-8))
+    if grad_scale is not None:
+        if grad_scale.dtype != torch.float32 or not grad_scale.is_cuda:
+            raise TypeError("grad_scale must be an fp32 scalar on the GPU")
+        a.grad_scale = grad_scale.data_ptr()
+        a._keep_grad_scale = grad_scale          # keeps the tensor alive as long as the args
     return a
 
 
@@ -329,6 +334,17 @@ def adam_step(grad, param, exp_avg, exp_avg_sq, lr, weight_decay, betas, eps, st
     L.check(L.lib().jabas_adam(grad.data_ptr(), param.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
                                lr, weight_decay, betas[0], betas[1], eps, int(step), int(bool(adamw)),
                                _stream_ptr(stream)), "jabas_adam")
+
+
+def clip_coef(stats_rows, max_norm, eps=1e-6, out=None, stream=None):
+    """Device scalar max_norm / (||aggregate|| + eps) from statistics rows (no host sync);
+    pass it as ``grad_scale`` of a later step to clip the aggregate by global norm."""
+    rows = stats_rows.reshape(-1, L.STATS_STRIDE)
+    if out is None:
+        out = torch.empty(1, dtype=torch.float32, device=rows.device)
+    L.check(L.lib().jabas_clip_coef(rows.data_ptr(), rows.shape[0], float(max_norm), float(eps), out.data_ptr(),
+                                    _stream_ptr(stream)), "jabas_clip_coef")
+    return out
 
 
 # ---------------------------------------------------------------------- cosine similarity

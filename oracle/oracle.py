@@ -168,9 +168,23 @@ def opt_step(opt, group, p, g, s1, s2, step, first_step, lr_scale=1.0):
         raise ValueError(opt["kind"])
 
 
+# -------------------------------------------------------------------------- clipping
+def clip_coef(total_sq, max_norm, eps=1e-6):
+    """torch.nn.utils.clip_grad_norm_: clip_coef = max_norm / (total_norm + 1e-6), applied
+    only when below 1 (examples/gnmt/seq2seq/train/trainer.py:157-161). The norm is formed
+    from the float64 sum of squares; the coefficient is an fp32 scalar."""
+    return float(np.float32(max_norm / (math.sqrt(total_sq) + eps)))
+
+
+def clip(agg, max_norm, eps=1e-6):
+    """Returns (clipped aggregate, coefficient); one fp32 product per element when clipping."""
+    c = clip_coef(float(torch.dot(agg.double(), agg.double())), max_norm, eps)
+    return (torch.mul(agg, c) if c < 1.0 else agg), c
+
+
 # ---------------------------------------------------------------------- whole sync step
 def sync_step(grads, batches, spans, opt=None, param=None, state1=None, state2=None, step=1, first_step=False,
-              want_stats=False, half_id=None, lr_scale=1.0):
+              want_stats=False, half_id=None, lr_scale=1.0, clip_norm=None):
     """Fused-step semantics over flat CPU arenas.
 
     grads: K flat tensors; spans: [(offset, numel, bounds)] with bounds [(start, group)].
@@ -184,6 +198,13 @@ def sync_step(grads, batches, spans, opt=None, param=None, state1=None, state2=N
         agg[sl] = aggregate(gs, batches)
         if want_stats:
             rows[si] = stats(gs, batches, half_id)
+    if clip_norm is not None:                  # global norm over every span, then one scale
+        total = sum(float(torch.dot(agg[o:o + n].double(), agg[o:o + n].double())) for o, n, _ in spans)
+        c = clip_coef(total, clip_norm)
+        if c < 1.0:
+            for o, n, _ in spans:
+                agg[o:o + n] = torch.mul(agg[o:o + n], c)
+    for si, (off, n, bounds) in enumerate(spans):
         if opt is not None:
             bl = list(bounds) if bounds else [(0, 0)]
             for j, (start, group) in enumerate(bl):

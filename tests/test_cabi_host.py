@@ -23,7 +23,7 @@ def _declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = _declared_functions()
-    assert len(names) >= 14
+    assert len(names) >= 15
     lib = L.lib()
     for n in names:
         assert hasattr(lib, n), f"{n} declared in jabas_sync.h but not exported"
@@ -35,7 +35,7 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(L.JabasSpan) == 8 * 8 + 4 * 8 + 7 * 8 + 8 + 4 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
-    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 32 + 4 + 8 + 32 + 4 * 4 + 4 + 5 * 8 + 16 * 24
+    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 32 + 4 + 8 + 32 + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8
     assert L.JabasStepArgs.groups.offset % 8 == 0 and L.JabasStepArgs.momentum.offset % 8 == 0
 
 

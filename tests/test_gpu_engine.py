@@ -1,0 +1,100 @@
+"""GPU tests of the flat-arena engine: multi-bucket plans with parameter groups, in-place
+aggregation, fan-out, per-tensor spans, and global-norm clipping (two launches with a
+device-side coefficient), against the oracle over the same arenas."""
+import math
+
+import pytest
+import torch
+
+from oracle import oracle as O
+from jabas_amd.workloads import ParamSpec
+
+pytestmark = pytest.mark.gpu
+
+SPECS = [ParamSpec("a.weight", 5000, 1), ParamSpec("a.bias", 77, 0), ParamSpec("b.weight", 300000, 1),
+         ParamSpec("b.bias", 1024, 0), ParamSpec("c.weight", 64 * 64 * 9, 1), ParamSpec("c.scale", 1, 0),
+         ParamSpec("d.weight", 123457, 1)]
+CAPS = (4096 * 4, 200000 * 4)
+SGD = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+           groups=[dict(lr=0.1, weight_decay=0.0), dict(lr=0.1, weight_decay=1e-4)])
+ADAM = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8,
+            groups=[dict(lr=2e-3, weight_decay=0.0), dict(lr=2e-3, weight_decay=1e-2)])
+
+
+def _close(a, b, rtol=1e-6, atol=1e-9):
+    a, b = a.detach().cpu().double(), b.detach().cpu().double()
+    return bool(((a - b).abs() <= rtol * b.abs() + atol).all())
+
+
+def _make(gpu, batches, opt, dtype=torch.float32, **kw):
+    from jabas_amd.engine import VSWFlatSync
+    eng = VSWFlatSync(SPECS, batches, grad_dtype=dtype, opt=opt, device=gpu, caps=CAPS, **kw)
+    gen = torch.Generator().manual_seed(3)
+    n = eng.layout.total
+    host = dict(g=[(torch.randn(n, generator=gen) * 1e-2).to(dtype) for _ in batches],
+                p=torch.randn(n, generator=gen) * 0.05, s1=torch.zeros(n), s2=torch.zeros(n))
+    for k, g in enumerate(host["g"]):
+        eng.grads[k].copy_(g)
+    eng.param.copy_(host["p"])
+    spans = [(off, cnt, bounds) for off, cnt, bounds, _ in eng.layout.spans]
+    return eng, host, spans
+
+
+@pytest.mark.parametrize("per_tensor", [False, True])
+@pytest.mark.parametrize("opt,dtype", [(SGD, torch.float32), (ADAM, torch.float32), (ADAM, torch.bfloat16)])
+def test_engine_steps_match_oracle(gpu, opt, dtype, per_tensor):
+    batches = (4, 2, 2)
+    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=2, per_tensor_spans=per_tensor)
+    assert len(eng.layout.buckets) >= 3
+    adam = opt["kind"] != "sgd"
+    for step in (1, 2, 3):
+        rows = eng.step(stats=True)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"] if adam else None,
+                                    step=step, first_step=(step == 1), want_stats=True)
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h[sl].view(torch.int32)), step
+        rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        assert _close(rows[:, :7], rows_h[:, :7], rtol, 1e-30)
+        assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
+        for f in eng.fanout:
+            for off, cnt, _ in spans:                             # padding between buckets is never touched
+                assert torch.equal(f[off:off + cnt], eng.param[off:off + cnt])
+        assert eng.cosine(rows) == pytest.approx(O.cosine_from_rows(rows_h), rel=1e-6)
+        if dtype == torch.float32:
+            for off, cnt, _ in spans:
+                host["g"][0][off:off + cnt] = agg_h[off:off + cnt]
+        per_bucket = eng.bucket_stats(rows)
+        assert per_bucket.shape[0] == len(eng.layout.buckets)
+        assert torch.allclose(per_bucket.sum(0), rows.cpu().sum(0), rtol=1e-12)
+
+
+@pytest.mark.parametrize("clip_norm", [0.05, 1e3])
+@pytest.mark.parametrize("opt", [SGD, ADAM])
+def test_global_norm_clipping(gpu, opt, clip_norm):
+    batches = (128, 128, 64, 64)
+    eng, host, spans = _make(gpu, batches, opt, n_fanout=1)
+    adam = opt["kind"] != "sgd"
+    for step in (1, 2):
+        rows = eng.step(stats=True, clip_norm=clip_norm)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"] if adam else None,
+                                    step=step, first_step=(step == 1), want_stats=True, clip_norm=clip_norm)
+        total = float(rows_h[:, O.NORM_AGG].sum())
+        c = O.clip_coef(total, clip_norm)
+        assert (c < 1.0) == (clip_norm < 1.0)                     # the small bound clips, the large one does not
+        assert float(eng._coef) == pytest.approx(c, rel=1e-6)
+        assert _close(rows[:, :8], rows_h[:, :8], 1e-6, 1e-30)     # statistics are of the unclipped aggregate
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            assert _close(eng.agg[sl], agg_h[sl], 1e-6, 1e-12), step
+            if c >= 1.0:
+                assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h[sl].view(torch.int32))
+        assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
+        for off, cnt, _ in spans:
+            assert torch.equal(eng.fanout[0][off:off + cnt], eng.param[off:off + cnt])
+            host["g"][0][off:off + cnt] = agg_h[off:off + cnt]
+    if clip_norm < 1.0:
+        norm = math.sqrt(sum(float(torch.dot(eng.agg[o:o + c_].double(), eng.agg[o:o + c_].double())) for o, c_, _ in spans))
+        assert norm == pytest.approx(clip_norm, rel=1e-4)

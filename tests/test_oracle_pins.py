@@ -309,3 +309,23 @@ def test_sync_step_composes_pieces_per_span_and_group():
     wd = slice(0, 700)
     assert torch.allclose(p[wd].double(), p0[wd].double() - 0.1 * (agg[wd].double() + 1e-4 * p0[wd].double()),
                           rtol=1e-6, atol=1e-10)
+
+
+# ----------------------------------------------------------------------------- clipping
+@pytest.mark.parametrize("max_norm", [0.01, 5.0])
+def test_clip_matches_torch_clip_grad_norm(max_norm):
+    shapes = [(300,), (17, 31), (1000,)]
+    gen = torch.Generator().manual_seed(5)
+    params = [torch.nn.Parameter(torch.zeros(s)) for s in shapes]
+    for p in params:
+        p.grad = torch.randn(p.shape, generator=gen) * 1e-2
+    flat = torch.cat([p.grad.reshape(-1) for p in params]).clone()
+    total = torch.nn.utils.clip_grad_norm_(params, max_norm)
+    got, c = O.clip(flat, max_norm)
+    want = torch.cat([p.grad.reshape(-1) for p in params])
+    assert float(total) == pytest.approx(math.sqrt(float(torch.dot(flat.double(), flat.double()))), rel=1e-6)
+    assert torch.allclose(got, want, rtol=1e-6, atol=1e-12)
+    if max_norm == 5.0:
+        assert c > 1.0 and torch.equal(got, flat)              # above the norm: untouched, bit for bit
+    else:
+        assert c < 1.0 and float(torch.linalg.vector_norm(got.double())) == pytest.approx(max_norm, rel=1e-4)
