@@ -47,6 +47,12 @@ class VSWFlatSync:
             if kind in (L.OPT_ADAM, L.OPT_ADAMW):
                 self.state2 = torch.zeros(n, dtype=torch.float32, device=self.device)
             self.fanout = [torch.zeros(n, dtype=torch.float32, device=self.device) for _ in range(n_fanout)]
+        self._fanout_wanted = n_fanout > 0
+        self._build_plan()
+        self.step_count = 0
+
+    def _build_plan(self):
+        kind = opt_kind(self.opt)
         spans = []
         for (off, numel, bounds, _bucket) in self.layout.spans:
             sl = slice(off, off + numel)
@@ -60,7 +66,33 @@ class VSWFlatSync:
         self.span_bucket = [s[3] for s in self.layout.spans]
         self.plan = SyncPlan(spans, kind)
         self._plan_agg = self._plan_opt = self._coef = None
-        self.step_count = 0
+
+    # ---- reconfiguration ---------------------------------------------------------
+    def reconfigure(self, batches):
+        """Changes the set of VSWs (adaptive batching adds or removes workers at run time,
+        jabas/train/trainer.py:485-575) without touching weights or optimizer state:
+        gradient and replica arenas are added or dropped, the plans rebuilt, the step
+        count kept."""
+        batches = tuple(batches)
+        new_k = len(batches)
+        if not 1 <= new_k <= L.MAX_K:
+            raise ValueError(f"number of VSWs must be in 1..{L.MAX_K}")
+        n = self.layout.total
+        in_place = self.agg is self.grads[0]
+        had_fanout = self._fanout_wanted
+        while len(self.grads) < new_k:
+            self.grads.append(torch.zeros(n, dtype=self.grad_dtype, device=self.device))
+        del self.grads[new_k:]
+        if had_fanout and self.param is not None:
+            while len(self.fanout) < new_k - 1:
+                f = torch.empty(n, dtype=torch.float32, device=self.device)
+                f.copy_(self.param)                     # a new replica starts from the main weights
+                self.fanout.append(f)
+            del self.fanout[max(0, new_k - 1):]
+        self.K, self.batches = new_k, batches
+        if in_place:
+            self.agg = self.grads[0]
+        self._build_plan()
 
     # ---- views -------------------------------------------------------------------
     def _view(self, arena, i):

@@ -59,7 +59,7 @@ def tag_parameter_indices(model):
 
 class VSWSyncTrainer:
     def __init__(self, gpu, local_batch_sizes, opt, interval=100, grad_dtype=torch.float32,
-                 param_groups_func=None, similarity_target=None):
+                 param_groups_func=None, similarity_target=None, controller=None, clip_norm=None):
         self.gpu = torch.device("cuda", gpu) if isinstance(gpu, int) else torch.device(gpu)
         self.local_batch_sizes = tuple(local_batch_sizes)
         self.num_models = len(self.local_batch_sizes)
@@ -68,6 +68,8 @@ class VSWSyncTrainer:
         self.grad_dtype = grad_dtype
         self.param_groups_func = param_groups_func
         self.similarity_target = similarity_target
+        self.controller = controller              # AdaptiveBatchController or None (enable_adjust off)
+        self.clip_norm = clip_norm
         self.global_lr_modifier = 1.0
         self.local_models, self.model_streams = [], []
         self.main_model = None
@@ -89,21 +91,48 @@ class VSWSyncTrainer:
                     group_of[id(p)] = gi
         specs = [ParamSpec(n, p.numel(), group_of.get(id(p), 0)) for n, p in zip(names, params)]
         self.engine = VSWFlatSync(specs, self.local_batch_sizes, grad_dtype=self.grad_dtype, opt=self.opt,
-                                  device=self.gpu, n_fanout=self.num_models - 1)
+                                  device=self.gpu, n_fanout=max(1, self.num_models - 1))
+        if self.num_models == 1:
+            self.engine.reconfigure(self.local_batch_sizes)       # keeps the fan-out slot for later replicas
         self.criterion = criterion
         self.local_models = [model] + [copy.deepcopy(model) for _ in range(self.num_models - 1)]
         self.main_model = self.local_models[0]
         self.model_streams = [torch.cuda.Stream(self.gpu) for _ in range(self.num_models)]
+        for k, m in enumerate(self.local_models):
+            self._bind_model(k, m, copy_weights=True)
+        torch.cuda.synchronize(self.gpu)
+
+    def _bind_model(self, k, m, copy_weights):
+        """Points replica k's parameters and gradients at its arenas."""
         eng = self.engine
+        weights = eng.param if k == 0 else eng.fanout[k - 1]
         with torch.no_grad():
-            for k, m in enumerate(self.local_models):
-                weights = eng.param if k == 0 else eng.fanout[k - 1]
-                for i, p in enumerate(m.parameters()):
-                    view = eng._view(weights, i).view(p.shape)
+            for i, p in enumerate(m.parameters()):
+                view = eng._view(weights, i).view(p.shape)
+                if copy_weights:
                     view.copy_(p.data)
-                    p.data = view
-                    if self.grad_dtype == torch.float32:
-                        p.grad = eng.grad_view(k, i).view(p.shape)     # backward accumulates into the bucket
+                p.data = view
+                if self.grad_dtype == torch.float32:
+                    p.grad = eng.grad_view(k, i).view(p.shape)         # backward accumulates into the bucket
+
+    def _change_local_models_state(self, new_num_models, local_batch_size):
+        """Adds or removes VSWs (counterpart of jabas/train/trainer.py:485-575): the engine
+        re-plans over the new set, new replicas start from the main weights, weights and
+        optimizer state of the main VSW are untouched."""
+        torch.cuda.synchronize(self.gpu)
+        self.local_batch_sizes = (local_batch_size,) * new_num_models
+        self.engine.reconfigure(self.local_batch_sizes)
+        while len(self.local_models) < new_num_models:
+            self.local_models.append(copy.deepcopy(self.main_model))
+            self.model_streams.append(torch.cuda.Stream(self.gpu))
+        del self.local_models[new_num_models:]
+        del self.model_streams[new_num_models:]
+        for k, m in enumerate(self.local_models):
+            self._bind_model(k, m, copy_weights=False)
+        self.num_models = self.total_num_decoupled_workers = new_num_models
+        workers = new_num_models if new_num_models % 2 == 0 else new_num_models + 1
+        self.similarity_state.total_num_decoupled_workers = workers
+        self.similarity_state.subgroup_total_num_decoupled_workers = workers / 2
         torch.cuda.synchronize(self.gpu)
 
     # ------------------------------------------------------------------- one iteration
@@ -131,15 +160,25 @@ class VSWSyncTrainer:
             cur.wait_stream(s)
         st = self.similarity_state
         want = st.step % st.interval == 0
-        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier)
+        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm)
         if want:
             self._compute_cosine_similarity(rows)
         for k in range(self.num_models):
             self.engine.grads[k].zero_()
         for s in self.model_streams:
             s.wait_stream(cur)
+        if want and self.controller is not None:
+            self._adjust_adaptive_global_batch_size()
         st.step += 1
         return True
+
+    def _adjust_adaptive_global_batch_size(self):
+        """jabas/train/trainer.py:702-718: new global batch size from the similarity, the
+        matching number of VSWs, and the square-root LR modifier for the following steps."""
+        workers, modifier = self.controller.update(float(self.cos_placeholder), step=self.similarity_state.step)
+        self.global_lr_modifier = modifier
+        if workers != self.num_models:
+            self._change_local_models_state(workers, self.controller.local_batch_size)
 
     def _compute_cosine_similarity(self, rows):
         self.cos_placeholder = torch.tensor([sync.cosine_from_stats(rows)])

@@ -98,3 +98,34 @@ def test_global_norm_clipping(gpu, opt, clip_norm):
     if clip_norm < 1.0:
         norm = math.sqrt(sum(float(torch.dot(eng.agg[o:o + c_].double(), eng.agg[o:o + c_].double())) for o, c_, _ in spans))
         assert norm == pytest.approx(clip_norm, rel=1e-4)
+
+
+def test_reconfigure_changes_k_and_keeps_weights_and_state(gpu):
+    batches = (4, 4)
+    eng, host, spans = _make(gpu, batches, ADAM, n_fanout=1)
+    eng.step()
+    O.sync_step(host["g"], batches, spans, ADAM, host["p"], host["s1"], host["s2"], step=1, first_step=True)
+    torch.cuda.synchronize()
+    p_before, m_before = eng.param.clone(), eng.state1.clone()
+    # grow to 3 workers, then shrink to 1
+    for new_batches, step in (((4, 4, 4), 2), ((4,), 3)):
+        eng.reconfigure(new_batches)
+        assert eng.K == len(new_batches) and len(eng.grads) == eng.K and len(eng.fanout) == eng.K - 1
+        assert torch.equal(eng.param, p_before) and torch.equal(eng.state1, m_before)
+        assert eng.step_count == step - 1
+        for f in eng.fanout:
+            for off, cnt, _ in spans:
+                assert torch.equal(f[off:off + cnt], eng.param[off:off + cnt])     # a new replica starts in sync
+        gen = torch.Generator().manual_seed(40 + step)
+        hg = [torch.randn(eng.layout.total, generator=gen) * 1e-2 for _ in new_batches]
+        for k, g in enumerate(hg):
+            eng.grads[k].copy_(g)
+        rows = eng.step(stats=True)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg, new_batches, spans, ADAM, host["p"], host["s1"], host["s2"], step=step,
+                                    first_step=False, want_stats=True)
+        for off, cnt, _ in spans:
+            assert torch.equal(eng.agg[off:off + cnt].cpu().view(torch.int32), agg_h[off:off + cnt].view(torch.int32))
+        assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
+        assert _close(rows[:, :4 + eng.K], rows_h[:, :4 + eng.K], 1e-6, 1e-30)
+        p_before, m_before = eng.param.clone(), eng.state1.clone()

@@ -199,3 +199,37 @@ def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind):
         if stat_step:
             assert float(trainer.cos_placeholder) == pytest.approx(want_cos, rel=1e-6)
     assert trainer.similarity_state.step == 5
+
+
+def test_trainer_adds_and_removes_workers_from_the_similarity(gpu):
+    from jabas_amd.train import VSWSyncTrainer
+    from jabas_amd.train.adaptive import AdaptiveBatchController
+    import math
+    opt = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+               groups=[dict(lr=0.05, weight_decay=0.0), dict(lr=0.05, weight_decay=0.05)])
+    crit = torch.nn.MSELoss()
+    ctl = AdaptiveBatchController(8, 4, similarity_target=2.0, adjust_rate=0.1)     # cos < 2 always: grow
+    trainer = VSWSyncTrainer(gpu, (4, 4), opt, interval=2, param_groups_func=_groups, controller=ctl)
+    trainer.prepare_stream_parallel(_mlp(5), crit)
+    sizes = []
+    for step in range(1, 7):
+        gen = torch.Generator().manual_seed(step)
+        data = [(torch.randn(4, 37, generator=gen).to(gpu), torch.randn(4, 10, generator=gen).to(gpu))
+                for _ in range(trainer.num_models)]
+        losses = trainer.compute(data)
+        assert len(losses) == trainer.num_models
+        trainer.step()
+        torch.cuda.synchronize()
+        sizes.append(trainer.num_models)
+        for m in trainer.local_models[1:]:
+            for p, q in zip(m.parameters(), trainer.main_model.parameters()):
+                assert torch.equal(p, q)
+    assert sizes == [2, 3, 3, 4, 4, 5]                       # statistic steps 2, 4, 6 each add a worker
+    assert trainer.global_lr_modifier == pytest.approx(math.sqrt(20 / 8))
+    assert trainer.similarity_state.total_num_decoupled_workers == 6      # kept even, as the reference asserts
+    ctl.similarity_target = -2.0                             # cos > target always: shrink
+    for step in range(7, 9):
+        data = [(torch.randn(4, 37).to(gpu), torch.randn(4, 10).to(gpu)) for _ in range(trainer.num_models)]
+        trainer.compute(data)
+        trainer.step()
+    assert trainer.num_models == 4 and len(trainer.model_streams) == 4 and trainer.engine.K == 4
