@@ -116,6 +116,47 @@ def time_config(cfg, device, steps, warmup, torch):
     return res
 
 
+def launch_modes(cfg, device, steps, torch):
+    """Small-span launch overhead (the Faster R-CNN configuration's point): the same step as
+    one launch over bucket spans, one launch over one span per tensor, one launch per
+    bucket, and one launch per tensor. ms per step from HIP events."""
+    from jabas_amd.engine import VSWFlatSync
+    from jabas_amd.sync import SyncPlan
+    gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
+    out = {}
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    for label, per_tensor in (("one_launch_bucket_spans", False), ("one_launch_tensor_spans", True)):
+        eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, per_tensor_spans=per_tensor)
+        for g in eng.grads:
+            g.normal_(0, cfg.grad_std)
+        eng.param.normal_(0, 0.05)
+        eng.step()
+        out[label] = dict(launches=1, spans=eng.plan.n_span, ms=timed(lambda: eng.step(), steps))
+        plans = [SyncPlan([sp], eng.plan.opt_kind) for sp in eng.plan.spans]
+        args = eng.step_args()
+
+        def many():
+            for p in plans:
+                p.run(args)
+        key = "one_launch_per_tensor" if per_tensor else "one_launch_per_bucket"
+        out[key] = dict(launches=len(plans), spans=len(plans), ms=timed(many, max(3, steps // 5)))
+        del eng, plans
+        torch.cuda.empty_cache()
+    return out
+
+
 def cpu_baseline(cfg, torch, budget_s=25.0):
     """Reference-structured unfused step on the host cores, bounded to about budget_s."""
     from jabas_amd.layout import FlatLayout
@@ -184,6 +225,9 @@ def main():
         print(f"# {cfg.name}: {results[cfg.name]['ms_per_step']:.4f} ms/step, "
               f"{results[cfg.name]['GBps']:.0f} GB/s, {results[cfg.name]['pct_hbm_peak']:.1f} % of HBM peak",
               file=sys.stderr, flush=True)
+    if "faster_rcnn_r50_fpn" in results:
+        results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
+                                                                      args.steps, torch)
     head = results[head_cfg.name]
     bytes_per_launch = head["GB_per_step"] * 1e9
     roofline = dict(bound="hbm", achieved=head["GBps_launch"], peak=HBM_PEAK_GBPS, unit="GB/s",
