@@ -196,10 +196,10 @@ const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_
                                        launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
 
 // Second level of the statistics reduction: one workgroup per span sums the partial rows
-// of the span's chunks. Thread t adds rows t, t+256, ... in increasing order; the 256
+// of the span's chunks. Thread t adds rows t, t+1024, ... in increasing order; the 1024
 // per-thread sums then go through the same fixed wave tree and wave-order sum as the
 // first level, so the result does not depend on the machine or on timing.
-constexpr int kFinalizeBlock = 256;
+constexpr int kFinalizeBlock = 1024;
 __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
                                                                         uint32_t use_inline, int ns,
                                                                         const double* partials, double* stats_out) {

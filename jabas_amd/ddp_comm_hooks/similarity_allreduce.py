@@ -47,8 +47,8 @@ def subgroup_allreduce_hook(state, bucket):
 
 def similimarity_allreduce_hook(hook):
     """hook -> hook that runs ``hook`` first and the all-group aggregation after it, as in
-    the reference (same misspelt name). Nothing blocks: the returned Future resolves when
-    the fused launch that covers this bucket has been queued."""
+    the reference (same misspelt name). Nothing blocks: the returned Future is complete as
+    soon as this VSW's bucket has been handed to the GPU's LocalBucketSync."""
     def hook_with_allreduce(state, bucket):
         future_work = hook(state, bucket)
         out = torch.futures.Future()

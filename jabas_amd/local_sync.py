@@ -6,8 +6,12 @@ comm hook communicates, the others register ``dummy_hook``
 GPU: each hook publishes the flat bucket it was handed; when the K buckets with the same
 index are in, whichever thread arrived last queues ONE fused kernel on VSW 0's stream
 (aggregate into VSW 0's bucket, statistics when asked, optimizer update when the weights
-are laid out like the buckets) and resolves the futures. No hook ever blocks, so the
-scheme also works when the VSWs are driven from a single thread one after the other.
+are laid out like the buckets). The Future a hook gets back is already complete: stock
+DDP waits on it at the end of that replica's backward on the autograd engine's device
+thread, which every replica on the GPU shares, so a Future that needed another replica's
+backward to make progress would deadlock. Ordering is by stream instead: the launch waits
+on an event from every VSW's stream, and ``finish_step`` makes every VSW stream wait for
+the launches (and reports anything that went wrong in them) before gradients are reused.
 """
 import threading
 
@@ -32,8 +36,6 @@ class _Slot:
     def __init__(self, K):
         self.tensors = [None] * K
         self.events = [None] * K
-        self.futures = [None] * K
-        self.values = [None] * K
         self.want_stats = False
         self.on_done = None
         self.count = 0
@@ -60,14 +62,18 @@ class LocalBucketSync:
         self._main_stream = None
         self._workspaces = {}
         self._done_events = []
+        self._errors = []
+        self.launched = 0                      # fused launches queued so far
 
     # ------------------------------------------------------------------ hooks call this
     def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None):
-        """Hands VSW k's bucket ``bucket_index`` over. Returns a Future that resolves (to
-        ``value``, default the tensor) once the fused launch for that bucket is queued."""
+        """Hands VSW k's bucket ``bucket_index`` over; the fused launch for that bucket is
+        queued by whichever VSW hands its bucket over last. Returns a completed Future
+        carrying ``value`` (default the tensor)."""
         if not 0 <= k < self.K:
             raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
         fut = torch.futures.Future()
+        fut.set_result(tensor if value is None else value)
         event = stream = None
         if tensor.is_cuda:
             stream = torch.cuda.current_stream(tensor.device)
@@ -77,8 +83,7 @@ class LocalBucketSync:
             slot = self._slots.setdefault(bucket_index, _Slot(self.K))
             if slot.tensors[k] is not None:
                 raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
-            slot.tensors[k], slot.events[k], slot.futures[k] = tensor, event, fut
-            slot.values[k] = tensor if value is None else value
+            slot.tensors[k], slot.events[k] = tensor, event
             slot.count += 1
             if k == 0:
                 slot.want_stats, slot.on_done = want_stats, on_done
@@ -103,14 +108,14 @@ class LocalBucketSync:
                     self._done_events.append(done)
             else:
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
-        except Exception as exc:                       # surface the failure in every waiting hook
-            for f in slot.futures:
-                f.set_exception(exc)
+        except Exception as exc:                       # reported by finish_step
+            with self._lock:
+                self._errors.append((bucket_index, exc))
             return
         if slot.on_done is not None:
             slot.on_done(BucketStats(bucket_index, row) if row is not None else None)
-        for f, v in zip(slot.futures, slot.values):
-            f.set_result(v)
+        with self._lock:
+            self.launched += 1
 
     # ------------------------------------------------------------- the default launcher
     def _launch_fused(self, bucket_index, tensors, want_stats):
@@ -146,6 +151,11 @@ class LocalBucketSync:
         left = self.pending()
         if left:
             raise RuntimeError(f"buckets {left} were not published by every VSW")
+        with self._lock:
+            errors, self._errors = self._errors, []
+        if errors:
+            idx, exc = errors[0]
+            raise RuntimeError(f"fused launch of bucket {idx} failed: {exc}") from exc
         for s in streams:
             for ev in self._done_events:
                 s.wait_event(ev)
