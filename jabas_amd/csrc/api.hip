@@ -26,7 +26,7 @@ struct PlanHeader {
     uint32_t max_group;       // largest group index any bound names
     uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
     uint32_t chunk_tiles;     // tiles per workgroup the chunk table was cut for
-    uint32_t pad;
+    uint32_t max_span_chunks; // chunks of the largest span (sizes the striped finalize)
     uint64_t off_spans, off_prefix, off_chunks, off_bounds, total_bytes;
 };
 static_assert(sizeof(PlanHeader) == 88, "plan header layout");
@@ -195,24 +195,43 @@ typedef int (*LaunchFn)(int, int, int, const KArgs&, unsigned, hipStream_t);
 const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_fused_k3, launch_fused_k4,
                                        launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
 
-// Second level of the statistics reduction: one workgroup per span sums the partial rows
-// of the span's chunks. Thread t adds rows t, t+1024, ... in increasing order; the 1024
-// per-thread sums then go through the same fixed wave tree and wave-order sum as the
-// first level, so the result does not depend on the machine or on timing.
-constexpr int kFinalizeBlock = 1024;
+// Second level of the statistics reduction: sums partial rows in a fixed order.
+//   stripes == 0  rows [s*in_stripes, (s+1)*in_stripes) of `in` -> row s of `out`
+//   stripes >= 1  stripe j = blockIdx.x of the chunk rows of span s = blockIdx.y -> row s*stripes + j
+// Thread t adds rows t, t+256, ... in increasing order; the 256 per-thread sums then go
+// through the fixed wave tree and a wave-order sum, so the result does not depend on the
+// machine or on timing. A span with many chunks is cut into stripes (one workgroup each,
+// then one more launch over the stripe rows) because a single workgroup reads its rows at
+// the bandwidth of one CU.
+constexpr int kFinalizeBlock = 256;
+constexpr uint32_t kStripeRows = 512;        // chunk rows one workgroup sums in the striped launch
+constexpr uint32_t kMaxStripes = 32;
+constexpr uint32_t kSingleLaunchRows = 2560; // up to here one workgroup per span finishes in about 6 us
 __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
-                                                                        uint32_t use_inline, int ns,
-                                                                        const double* partials, double* stats_out) {
+                                                                        uint32_t use_inline, uint32_t stripes,
+                                                                        uint32_t in_stripes, int ns, const double* in,
+                                                                        double* out) {
     __shared__ double red[kFinalizeBlock / 64][kStatsStride];
-    const uint32_t s = blockIdx.x, t = threadIdx.x;
-    uint32_t c0 = 0, c1 = n_chunks;
-    if (!use_inline) { c0 = chunk_prefix[s]; c1 = chunk_prefix[s + 1]; }
+    const uint32_t s = blockIdx.y, j = blockIdx.x, t = threadIdx.x;
+    uint32_t c0, c1, o;
+    if (stripes == 0) {
+        c0 = s * in_stripes;
+        c1 = c0 + in_stripes;
+        o = s;
+    } else {
+        uint32_t b0 = 0, b1 = n_chunks;
+        if (!use_inline) { b0 = chunk_prefix[s]; b1 = chunk_prefix[s + 1]; }
+        const uint32_t per = (b1 - b0 + stripes - 1) / stripes;
+        c0 = b0 + j * per < b1 ? b0 + j * per : b1;
+        c1 = c0 + per < b1 ? c0 + per : b1;
+        o = s * stripes + j;
+    }
     double acc[kStatsStride];
 #pragma unroll
     for (int i = 0; i < kStatsStride; ++i) acc[i] = 0.0;
-#pragma unroll 4
+#pragma unroll 2
     for (uint32_t c = c0 + t; c < c1; c += kFinalizeBlock) {
-        const double* row = partials + static_cast<uint64_t>(c) * kStatsStride;
+        const double* row = in + static_cast<uint64_t>(c) * kStatsStride;
 #pragma unroll
         for (int i = 0; i < kStatsStride; ++i) acc[i] += row[i];
     }
@@ -227,9 +246,17 @@ __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const ui
         double sum = red[0][t];
 #pragma unroll
         for (int w = 1; w < kFinalizeBlock / 64; ++w) sum += red[w][t];
-        stats_out[static_cast<uint64_t>(s) * kStatsStride + t] = t < static_cast<uint32_t>(ns) ? sum : 0.0;
+        out[static_cast<uint64_t>(o) * kStatsStride + t] = t < static_cast<uint32_t>(ns) ? sum : 0.0;
     }
 }
+
+inline uint32_t stripes_for(uint32_t max_span_chunks) {
+    if (max_span_chunks <= kSingleLaunchRows) return 1;      // a second launch costs more than it saves
+    const uint32_t st = (max_span_chunks + kStripeRows - 1) / kStripeRows;
+    return st > kMaxStripes ? kMaxStripes : st;
+}
+// workspace rows: one per chunk, then one per (span, stripe)
+inline size_t workspace_rows(uint64_t n_chunks, uint64_t n_span) { return n_chunks + n_span * kMaxStripes + 1; }
 
 // One wave: fixed-order sum of slot NORM_AGG over the rows, then the coefficient.
 __global__ void __launch_bounds__(64) clip_coef_kernel(const double* rows, uint32_t n_rows, double max_norm, double eps,
@@ -240,14 +267,14 @@ __global__ void __launch_bounds__(64) clip_coef_kernel(const double* rows, uint3
     if (threadIdx.x == 63) *coef_out = static_cast<float>(max_norm / (sqrt(total) + eps));
 }
 
-int run_fused(KArgs& a, const JabasStepArgs* s, double* stats_out, void* workspace, size_t workspace_bytes,
-              hipStream_t stream) {
+int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double* stats_out, void* workspace,
+              size_t workspace_bytes, hipStream_t stream) {
     const int oc = opt_class_of(s->opt_kind);
     const int stats = s->stats ? 1 : 0;
     if (stats) {
         if (!stats_out) return JABAS_ERR_NULL;
         if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
-        if (workspace_bytes < static_cast<size_t>(a.n_chunks) * kStatsStride * sizeof(double)) return JABAS_ERR_WORKSPACE;
+        if (workspace_bytes < workspace_rows(a.n_chunks, a.n_span) * kStatsStride * sizeof(double)) return JABAS_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(stats_out) % 8) return JABAS_ERR_ALIGN;
     }
     a.partials = static_cast<double*>(workspace);
@@ -256,8 +283,18 @@ int run_fused(KArgs& a, const JabasStepArgs* s, double* stats_out, void* workspa
         if (err != 0) return JABAS_ERR_LAUNCH;
     }
     if (stats) {
-        hipLaunchKernelGGL(finalize_stats_kernel, dim3(a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
-                           a.n_chunks, a.use_inline, 4 + s->K, a.partials, stats_out);
+        const uint32_t st = stripes_for(max_span_chunks);
+        const int ns = 4 + s->K;
+        if (st == 1) {
+            hipLaunchKernelGGL(finalize_stats_kernel, dim3(1, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
+                               a.n_chunks, a.use_inline, 1u, 0u, ns, a.partials, stats_out);
+        } else {
+            double* level2 = a.partials + static_cast<uint64_t>(a.n_chunks) * kStatsStride;
+            hipLaunchKernelGGL(finalize_stats_kernel, dim3(st, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
+                               a.n_chunks, a.use_inline, st, 0u, ns, a.partials, level2);
+            hipLaunchKernelGGL(finalize_stats_kernel, dim3(1, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
+                               a.n_chunks, a.use_inline, 0u, st, ns, level2, stats_out);
+        }
         if (hipGetLastError() != hipSuccess) return JABAS_ERR_LAUNCH;
     }
     return JABAS_OK;
@@ -293,7 +330,7 @@ JABAS_API size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype) 
     const int dt = grad_dtype == JABAS_BF16 ? JABAS_BF16 : JABAS_F32;
     const uint64_t te = tile_elems(dt);
     const uint64_t tiles = (numel + ept_of(dt) - 1 + te - 1) / te;
-    return static_cast<size_t>(chunks_of_tiles(tiles, kMinChunkTiles) + 1) * kStatsStride * sizeof(double);
+    return workspace_rows(chunks_of_tiles(tiles, kMinChunkTiles), 1) * kStatsStride * sizeof(double);
 }
 
 namespace {
@@ -367,6 +404,8 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
         if (rc != JABAS_OK) return rc;
         if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
         prefix[i] = c;
+        const uint32_t span_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, ct));
+        if (span_chunks > h.max_span_chunks) h.max_span_chunks = span_chunks;
         uint32_t j = 0;
         for (uint32_t t0 = 0; t0 < tiles; t0 += ct, ++c) {
             cd[c].span = i;
@@ -397,7 +436,10 @@ JABAS_API int64_t jabas_plan_chunks(const void* host_blob) {
 
 JABAS_API size_t jabas_plan_workspace_bytes(const void* host_blob) {
     const int64_t n = jabas_plan_chunks(host_blob);
-    return n < 0 ? 0 : static_cast<size_t>(n + 1) * kStatsStride * sizeof(double);
+    if (n < 0) return 0;
+    PlanHeader h;
+    memcpy(&h, host_blob, sizeof(h));
+    return workspace_rows(static_cast<uint64_t>(n), h.n_span) * kStatsStride * sizeof(double);
 }
 
 JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, const JabasStepArgs* args,
@@ -427,7 +469,7 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     a.n_chunks = h.n_chunks;
     a.chunk_tiles = h.chunk_tiles;
     a.use_inline = 0;
-    return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return run_fused(a, args, h.max_span_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev, const JabasStepArgs* args,
@@ -453,7 +495,7 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.chunk_tiles = pick_chunk_tiles(args->K);
     a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, a.chunk_tiles));
     a.use_inline = 1;
-    return run_fused(a, args, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return run_fused(a, args, a.n_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 JABAS_API int jabas_aggregate(const void* const* grads, int32_t K, int32_t grad_dtype, const float* weight,

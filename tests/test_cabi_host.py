@@ -81,7 +81,7 @@ def test_plan_encode_counts_chunks():
     rc, blob, _ = _encode([_span(n) for n in sizes])
     assert rc == L.OK
     assert lib.jabas_plan_chunks(blob.ctypes.data) == 2 + 3 + 1 + 0 + 21
-    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) == (27 + 1) * 12 * 8
+    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (27 + 5) * 12 * 8     # a row per chunk and per span, at least
     rc, blob, _ = _encode([_span(n, K=8) for n in sizes], K=8)
     assert rc == L.OK
     assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
