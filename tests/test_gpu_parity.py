@@ -327,3 +327,64 @@ def test_fused_rejects_bad_arguments(gpu):
     with pytest.raises(L.JabasSyncError) as e:
         sync.sync_bucket(span, args)                                          # optimizer without weights
     assert e.value.status == L.ERR_NULL
+
+
+def test_span_beyond_two_to_the_31_elements(gpu):
+    """64-bit element indexing: one span of 2^31 + 4099 elements (8.6 GB per buffer)."""
+    from jabas_amd import sync
+    n = (1 << 31) + 4099
+    g0 = torch.empty(n, dtype=torch.float32, device=gpu)
+    g1 = torch.empty(n, dtype=torch.float32, device=gpu)
+    step = 1 << 27
+    for lo in range(0, n, step):                       # value depends on the position, cheap to regenerate
+        hi = min(n, lo + step)
+        idx = torch.arange(lo, hi, device=gpu, dtype=torch.int64)
+        g0[lo:hi] = ((idx % 1021).float() - 510.0) * 2.0 ** -10
+        g1[lo:hi] = ((idx % 4093).float() - 2046.0) * 2.0 ** -12
+        del idx
+    out = torch.empty(n, dtype=torch.float32, device=gpu)
+    sync.aggregate([g0, g1], (1, 1), out=out)          # weights 0.5, 0.5: every product and the sum are exact
+    row = sync.gradient_stats([g0, g1], (1, 1)).cpu()
+    torch.cuda.synchronize()
+    norm0 = 0.0
+    for lo in range(0, n, step):
+        hi = min(n, lo + step)
+        want = g0[lo:hi] * 0.5 + g1[lo:hi] * 0.5
+        assert torch.equal(out[lo:hi].view(torch.int32), want.view(torch.int32)), lo
+        norm0 += float((g0[lo:hi].double() ** 2).sum())
+        del want
+    assert float(row[4]) == pytest.approx(norm0, rel=1e-10)
+
+
+def test_special_values_denormals_infinities_nans(gpu):
+    """Denormal inputs and results are kept (no flush to zero), infinities and NaNs stay in
+    the element they entered, signed zeros follow IEEE addition."""
+    from jabas_amd import sync
+    K, n = 3, 5000
+    hg = _host_grads(K, n, 99)
+    hg[0][:64] = torch.logspace(-45, -38, 64)                 # denormal inputs
+    hg[1][:64] = -torch.logspace(-44.5, -38.2, 64)
+    hg[2][:64] = 0.0
+    hg[0][100], hg[1][101], hg[2][102] = float("inf"), float("-inf"), float("nan")
+    hg[0][103], hg[1][103] = float("inf"), float("-inf")       # inf - inf -> nan
+    hg[0][200:210], hg[1][200:210], hg[2][200:210] = -0.0, -0.0, -0.0
+    hg[0][210:220], hg[1][210:220], hg[2][210:220] = -0.0, 0.0, -0.0
+    out = sync.aggregate([_dev(t, gpu) for t in hg], BATCHES[K]).cpu()
+    want = O.aggregate(hg, BATCHES[K])
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(out), nan) and int(nan.sum()) == 2
+    assert torch.equal(out[~nan].view(torch.int32), want[~nan].view(torch.int32))
+    assert torch.count_nonzero(out[:64]) > 32                  # denormal results survived
+    assert torch.all(out[200:210].view(torch.int32) == torch.tensor(-0.0).view(torch.int32))
+    assert torch.all(out[210:220].view(torch.int32) == 0)
+    # Adam on a gradient whose square is denormal: v stays denormal, the step is still the sign step
+    g = torch.full((2048,), 1e-21)
+    p_h, m_h, v_h = torch.ones(2048), torch.zeros(2048), torch.zeros(2048)
+    p_d, m_d, v_d = _dev(p_h, gpu), _dev(m_h, gpu), _dev(v_h, gpu)
+    hp = dict(lr=1e-3, weight_decay=0.0, betas=(0.9, 0.999), eps=1e-30, adamw=False)
+    O.adam_step(p_h, g, m_h, v_h, step=1, **hp)
+    sync.adam_step(_dev(g, gpu), p_d, m_d, v_d, step=1, **hp)
+    torch.cuda.synchronize()
+    assert 0 < float(v_h[0]) < 1.2e-38                         # denormal second moment
+    for a, b in ((p_d, p_h), (m_d, m_h), (v_d, v_h)):
+        assert torch.equal(_bits(a), _bits(b))
