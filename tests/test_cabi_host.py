@@ -187,3 +187,48 @@ def test_entry_points_validate_before_launching():
     g[1] = 0x7f0100000000
     assert lib.jabas_stats(g, 2, L.F32, w, hid, w, 100, 0x7f0400000000, None, 0, None) == L.ERR_WORKSPACE
     assert lib.jabas_gram(g, 2, L.F32, 100, 0x7f0400000000, None, 0, None) == L.ERR_WORKSPACE
+
+
+def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tmp_path):
+    """gcc -std=c99 compiles the header and a C client; the client links the library, reports the struct
+    layout its compiler sees (compared field by field with the ctypes mirror) and encodes a plan."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    libdir = os.path.dirname(os.path.abspath(L.LIB_PATH))
+    exe = str(tmp_path / "cabi_client")
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+           os.path.join(ROOT, "tests", "cabi_client.c"), "-o", exe, "-L", libdir, "-ljabas_sync",
+           "-Wl,-rpath," + libdir, "-Wl,--allow-shlib-undefined"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr
+    seen = {}
+    for line in out.stdout.splitlines():
+        kind, name, *rest = line.split(" ", 2)
+        seen[(kind, name)] = rest[0] if rest else ""
+    structs = {"JabasSpan": L.JabasSpan, "JabasBound": L.JabasBound, "JabasGroup": L.JabasGroup,
+               "JabasStepArgs": L.JabasStepArgs}
+    checked = 0
+    for (kind, name), val in seen.items():
+        if kind == "sizeof":
+            assert C.sizeof(structs[name]) == int(val), name
+            checked += 1
+        elif kind == "offsetof":
+            s, f = name.split(".")
+            assert getattr(structs[s], f).offset == int(val), name
+            checked += 1
+    assert checked == 36
+    # every field of the ctypes mirror was reported by the C side (reserved words aside)
+    for sname, st in structs.items():
+        for f, _ in st._fields_:
+            if not f.startswith("reserved") and not f.startswith("_"):
+                assert ("offsetof", f"{sname}.{f}") in seen, f"{sname}.{f}"
+    assert seen[("version", "jabas_sync")].startswith("0.")
+    assert seen[("status0", "ok")] == ""
+    assert seen[("encode", "0")] == ""
+    assert seen[("chunks", "8")] == ""                       # 5000 -> 3 chunks of 2 tiles, 9096 -> 5
+    assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * 96
+    assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
