@@ -179,3 +179,46 @@ def test_full_size_configuration(gpu, name):
     a.step(stats=False)
     torch.cuda.synchronize()
     assert torch.equal((agg1 * 4.0).view(torch.int32), a.agg.view(torch.int32))
+
+
+def test_gnmt_embedding_rows_with_independent_masks(gpu):
+    """The GNMT embedding bucket (32,317 x 1,024) at full size where every VSW saw its own 10 % of
+    the rows: a row of the aggregate is exactly +0 only where no VSW touched it, Adam's first
+    step leaves exactly those weights alone, and the whole aggregate is bit-exact."""
+    from jabas_amd import workloads as W, sync
+    cfg = W.config("gnmt")
+    rows, cols = W.GNMT_EMBEDDING_ROWS, W.GNMT_EMBEDDING_COLS
+    n, K = rows * cols, cfg.K
+    hg, keeps = [], []
+    for k in range(K):
+        gen = torch.Generator().manual_seed(4321 + k)
+        keep = torch.rand(rows, generator=gen) < 0.1
+        g = (torch.randn(rows, cols, generator=gen) * cfg.grad_std) * keep[:, None]
+        hg.append(torch.where(keep[:, None], g, torch.zeros(())).reshape(-1).contiguous())
+        keeps.append(keep)
+    touched = torch.stack(keeps).any(0)
+    assert 0.3 < touched.float().mean() < 0.4                               # 1 - 0.9^4 = 0.344
+    p_h = torch.randn(n, generator=torch.Generator().manual_seed(9)) * 0.05
+    p0 = p_h.clone()
+    m_h, v_h = torch.zeros(n), torch.zeros(n)
+    dg = [t.to(gpu) for t in hg]
+    p_d, m_d, v_d = p_h.to(gpu), torch.zeros(n, device=gpu), torch.zeros(n, device=gpu)
+    span = sync.SpanSpec(dg, agg_out=dg[0], param=p_d, state1=m_d, state2=v_d)
+    args = sync.make_step_args(cfg.batches, torch.float32, stats=True, opt=cfg.opt, step=1, first_step=True)
+    row = sync.sync_bucket(span, args)
+    torch.cuda.synchronize()
+    agg_h, rows_h = O.sync_step(hg, cfg.batches, [(0, n, ((0, 0),))], cfg.opt, p_h, m_h, v_h, step=1,
+                                first_step=True, want_stats=True)
+    agg_d = dg[0].cpu()
+    assert torch.equal(agg_d.view(torch.int32), agg_h.view(torch.int32))
+    a2 = agg_d.view(rows, cols)
+    assert torch.all(a2[~touched].view(torch.int32) == 0)                   # +0, not -0
+    assert torch.all((a2[touched] != 0).any(1))
+    p2 = p_d.cpu().view(rows, cols)
+    assert torch.equal(p2[~touched], p0.view(rows, cols)[~touched])
+    assert torch.equal(p_d.cpu().view(torch.int32), p_h.view(torch.int32))
+    assert torch.equal(m_d.cpu().view(torch.int32), m_h.view(torch.int32))
+    assert torch.equal(v_d.cpu().view(torch.int32), v_h.view(torch.int32))
+    assert torch.allclose(row.cpu()[:4 + K], rows_h[0][:4 + K], rtol=1e-6, atol=0.0)
+    for k in range(K):                                                      # per-worker norms: only that worker's rows count
+        assert row[4 + k].item() == pytest.approx((hg[k].double() ** 2).sum().item(), rel=1e-10)
