@@ -52,7 +52,7 @@ typedef enum JabasStatus {
     JABAS_ERR_PLAN = -8,        /* plan blob malformed or too small                    */
     JABAS_ERR_SIZE = -9,        /* numel / span count out of range                     */
     JABAS_ERR_LAUNCH = -10,     /* the HIP runtime refused the launch                  */
-    JABAS_ERR_ALIAS = -11       /* agg_out aliases a gradient buffer that is not fp32  */
+    JABAS_ERR_ALIAS = -11       /* a written buffer overlaps another buffer of the span */
 } JabasStatus;
 
 enum { JABAS_F32 = 0, JABAS_BF16 = 1 };
@@ -75,8 +75,10 @@ enum {
  * 16-byte line, and of every bf16 gradient buffer at the same position of an 8-byte line
  * ((address / element size) mod 4 equal for all buffers), which holds whenever they are
  * views at one element offset into 16-byte aligned arenas.
- * agg_out may alias grads[0] when the gradients are fp32 (in-place bucket update).
- * Unused pointers are NULL. */
+ * agg_out may be exactly one of the fp32 gradient buffers (in-place bucket update); apart
+ * from that every written buffer (agg_out, param, state1, state2, fanout) must be disjoint
+ * from every other buffer of the span, else JABAS_ERR_ALIAS. Overlap between different
+ * spans of one plan is the caller's responsibility. Unused pointers are NULL. */
 typedef struct JabasSpan {
     const void* grads[JABAS_MAX_K];     /* K gradient buffers (fp32 or bf16)           */
     float*      agg_out;                /* aggregated fp32 gradient, or NULL           */

@@ -114,6 +114,26 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDe
             if (grad_dtype != JABAS_F32 || static_cast<const void*>(in.agg_out) != in.grads[k]) return JABAS_ERR_ALIAS;
         }
     }
+    // Every buffer the launch writes must be disjoint from every other buffer of the span (the
+    // in-place aggregate above is the one exception): each element is read and written by a
+    // different thread at a different time, so any overlap would be a silent race.
+    const void* written[4 + JABAS_MAX_K - 1];
+    int nw = 0;
+    if (in.agg_out) written[nw++] = in.agg_out;
+    if (oc != 0) {
+        written[nw++] = in.param;
+        if (in.state1) written[nw++] = in.state1;
+        if (oc == 2) written[nw++] = in.state2;
+        for (uint32_t r = 0; r < in.n_fanout; ++r) written[nw++] = in.fanout[r];
+    }
+    const size_t fb = in.numel * 4;
+    for (int i = 0; i < nw; ++i) {
+        for (int j = i + 1; j < nw; ++j)
+            if (ranges_overlap(written[i], fb, written[j], fb)) return JABAS_ERR_ALIAS;
+        if (written[i] == static_cast<const void*>(in.agg_out)) continue;      // checked against the gradients above
+        for (int k = 0; k < K; ++k)
+            if (ranges_overlap(written[i], fb, in.grads[k], in.numel * gs)) return JABAS_ERR_ALIAS;
+    }
     out->lo = skew;
     out->hi = skew + in.numel;
     out->bound_begin = in.bound_begin;
@@ -320,7 +340,7 @@ JABAS_API const char* jabas_status_string(int status) {
         case JABAS_ERR_PLAN: return "plan blob malformed, too small or not matching the step arguments";
         case JABAS_ERR_SIZE: return "element, span or fan-out count out of range";
         case JABAS_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
-        case JABAS_ERR_ALIAS: return "agg_out overlaps a gradient buffer other than exactly in place (fp32)";
+        case JABAS_ERR_ALIAS: return "a written buffer overlaps another buffer of the span (only agg_out == grads[k], fp32, may alias)";
         default: return "unknown status";
     }
 }

@@ -258,7 +258,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
             const uint64_t rel = e - sp.lo;
             uint32_t jj = j;
             while (jj + 1 < sp.bound_count && bd[jj + 1].start <= rel) ++jj;
-            gid = bd[jj].group;
+            gid = bd[jj].group & (JABAS_MAX_GROUPS - 1);   // a bound table on the device cannot be checked by the host
         }
         const GroupDev G = a.groups[gid];
         float g[K][1], p[1] = {0.0f}, s1[1] = {0.0f}, s2[1] = {0.0f}, agg[1];
@@ -302,7 +302,7 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
         uint32_t gid = 0;
         if (nb) {
             while (j + 1 < nb && bd[j + 1].start <= rel) ++j;
-            gid = bd[j].group;
+            gid = bd[j].group & (JABAS_MAX_GROUPS - 1);
             if (j + 1 < nb) stretch_end = sp.lo + bd[j + 1].start;
         }
         uint32_t nfull = 0;

@@ -232,3 +232,36 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
     assert seen[("chunks", "8")] == ""                       # 5000 -> 3 chunks of 2 tiles, 9096 -> 5
     assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * 96
     assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
+
+
+def test_plan_encode_rejects_overlapping_written_buffers():
+    def span():
+        return _span(4096, opt=True)
+    s = span()
+    s.state1 = s.param + 4096 * 4 - 16                          # last four weights = first four momentum entries
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_ALIAS
+    s = span()
+    s.state1 = s.param + 4096 * 4                               # back to back: fine
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.OK
+    s = span()
+    s.state2 = s.state1
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIAS
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.OK               # SGD never touches state2
+    s = span()
+    s.param = s.grads[1]                                        # weights over a worker's gradients
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_ALIAS
+    s = span()
+    s.param = s.agg_out
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_ALIAS
+    s = span()
+    s.n_fanout = 2
+    s.fanout[0] = s.param + (1 << 30)
+    s.fanout[1] = s.fanout[0] + 16
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_ALIAS
+    s.fanout[1] = s.fanout[0] + 4096 * 4
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.OK
+    s.fanout[1] = s.param
+    assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_ALIAS
+    s = span()
+    s.param = s.grads[0]                                        # ignored without an optimizer
+    assert _encode([s], opt=L.OPT_NONE)[0] == L.OK
