@@ -6,8 +6,11 @@
 // Also: pure read, pure write, copy. Not part of libjabas_sync.so; a measurement aid.
 //
 //   ./stream_mix_probe [stagger_bytes]   prints one line per mix: ms, GB/s, fraction of 8 TB/s
+//   ./stream_mix_probe [stagger_bytes [lds_bytes]]
 //   stagger_bytes (default 0, multiple of 16): stream i starts i * stagger_bytes into its allocation,
 //   to see what the relative placement of the streams in memory is worth
+//   lds_bytes (default 0): unused dynamic LDS per workgroup, which caps the workgroups resident on a
+//   CU (160 KB of LDS each), to see what occupancy is worth: 40960 -> 3 workgroups = 3 waves per SIMD
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
@@ -90,10 +93,12 @@ static float time_ms(F launch, int iters = 20) {
     return ms / iters;
 }
 
+static unsigned g_lds_bytes = 0;
+
 template <int K, bool BF16, int S, bool OUT, int TILES, int U>
 static void run(const char* label, const Streams& P, size_t n) {
     const unsigned grid = static_cast<unsigned>(n / (1024u * TILES));      // n is a multiple of 4096
-    const float ms = time_ms([&] { hipLaunchKernelGGL((mix_kernel<K, BF16, S, OUT, TILES, U>), dim3(grid), dim3(256), 0, 0, P); });
+    const float ms = time_ms([&] { hipLaunchKernelGGL((mix_kernel<K, BF16, S, OUT, TILES, U>), dim3(grid), dim3(256), g_lds_bytes, 0, P); });
     const double bytes = static_cast<double>(n) * (K * (BF16 ? 2 : 4) + 8 * S + (OUT ? 4 : 0));
     const double gbs = bytes / ms / 1e6;
     std::printf("%-58s %8.3f ms %7.0f GB/s  %5.1f %% of 8 TB/s\n", label, ms, gbs, 100.0 * gbs / kPeakGBs);
@@ -102,6 +107,7 @@ static void run(const char* label, const Streams& P, size_t n) {
 
 int main(int argc, char** argv) {
     const size_t stagger = argc > 1 ? std::strtoull(argv[1], nullptr, 10) / 16 * 16 : 0;
+    g_lds_bytes = argc > 2 ? static_cast<unsigned>(std::strtoul(argv[2], nullptr, 10)) : 0;
     const size_t n = static_cast<size_t>(1) << 27;      // elements per stream: 512 MiB fp32, 256 MiB bf16
     Streams P{};
     for (int k = 0; k < kMaxK; ++k) {
@@ -124,7 +130,7 @@ int main(int argc, char** argv) {
     }
     CK(hipDeviceSynchronize());
 
-    std::printf("stream_mix_probe: %zu elements per stream, stagger %zu B, one 256-thread workgroup per chunk, nontemporal accesses\n", n, stagger);
+    std::printf("stream_mix_probe: %zu elements per stream, stagger %zu B, %u B of idle LDS per workgroup, one 256-thread workgroup per chunk, nontemporal accesses\n", n, stagger, g_lds_bytes);
     run<1, false, 0, false, 2, 2>("pure read, 1 stream", P, n);
     run<4, false, 0, false, 2, 2>("pure read, 4 streams", P, n);
     run<8, false, 0, false, 2, 2>("pure read, 8 streams", P, n);
