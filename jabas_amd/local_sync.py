@@ -23,7 +23,9 @@ from . import _lib as L
 
 class BucketStats:
     """Statistics row of one bucket on the device (what a stat step leaves in
-    ``GradientSimilarityState.grad_placeholder`` instead of a full gradient copy)."""
+    ``GradientSimilarityState.grad_placeholder`` instead of a full gradient copy). The row is
+    one of two buffers the bucket's launches alternate between: read it (``cpu()``) before the
+    second-next statistic step of that bucket."""
 
     def __init__(self, index, row):
         self.index, self.row = index, row
@@ -60,7 +62,8 @@ class LocalBucketSync:
         self._lock = threading.Lock()
         self._slots = {}
         self._main_stream = None
-        self._workspaces = {}
+        self._calls = {}                       # bucket index -> prepared sync.BucketCall
+        self._args_cache = {}
         self._done_events = []
         self._errors = []
         self.launched = 0                      # fused launches queued so far
@@ -99,13 +102,12 @@ class LocalBucketSync:
         main = self._main_stream
         try:
             if main is not None:
-                with torch.cuda.stream(main):
-                    for ev in slot.events[1:]:
-                        main.wait_event(ev)
-                    row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
-                    done = torch.cuda.Event()
-                    done.record(main)
-                    self._done_events.append(done)
+                for ev in slot.events[1:]:
+                    main.wait_event(ev)
+                row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
+                done = torch.cuda.Event()
+                done.record(main)
+                self._done_events.append(done)
             else:
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
         except Exception as exc:                       # reported by finish_step
@@ -118,27 +120,35 @@ class LocalBucketSync:
             self.launched += 1
 
     # ------------------------------------------------------------- the default launcher
+    def _step_args(self, dtype, want_stats, with_opt):
+        """JabasStepArgs of this step, built once per (step, kind of launch) and shared by its buckets."""
+        key = (self.step_count, self.lr_scale, dtype, bool(want_stats), bool(with_opt))
+        hit = self._args_cache.get(key)
+        if hit is None:
+            if len(self._args_cache) > 8:
+                self._args_cache.clear()
+            hit = self._args_cache[key] = sync.make_step_args(
+                self.batches, dtype, stats=want_stats, opt=self.opt if with_opt else None,
+                step=self.step_count + 1, first_step=self.step_count == 0, lr_scale=self.lr_scale)
+        return hit
+
     def _launch_fused(self, bucket_index, tensors, want_stats):
-        g0 = tensors[0]
-        pb = self.param_buckets.get(bucket_index)
-        opt = self.opt if pb is not None else None
-        span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
-                             param=pb and pb.get("param"), state1=pb and pb.get("state1"),
-                             state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
-                             bounds=(pb or {}).get("bounds", ()) if opt else ())
-        args = sync.make_step_args(self.batches, g0.dtype, stats=want_stats, opt=opt, step=self.step_count + 1,
-                                   first_step=self.step_count == 0, lr_scale=self.lr_scale)
-        ws = None
-        if want_stats:
-            key = (bucket_index, g0.numel())
-            ws = self._workspaces.get(key)
-            if ws is None:
-                ws = self._workspaces[key] = sync.Workspace.for_span(g0.numel(), g0.dtype, g0.device)
-        bd = None
-        if span.bounds:
-            bd = (pb or {}).get("_bounds_dev")
-        row = sync.sync_bucket(span, args, workspace=ws, bounds_dev=bd)
-        return row.clone() if row is not None else None
+        """Queues ``jabas_sync_bucket`` for one bucket on VSW 0's stream. DDP hands a hook the same
+        bucket buffers every step, so the prepared call (validated span, C struct, device bound table,
+        workspace) is kept per bucket and rebuilt only when the buffers change."""
+        call = self._calls.get(bucket_index)
+        if call is None or not call.matches(tensors):
+            g0 = tensors[0]
+            pb = self.param_buckets.get(bucket_index)
+            opt = self.opt if pb is not None else None
+            span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
+                                 param=pb and pb.get("param"), state1=pb and pb.get("state1"),
+                                 state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
+                                 bounds=(pb or {}).get("bounds", ()) if opt else ())
+            call = self._calls[bucket_index] = sync.BucketCall(span)
+            call.with_opt = opt is not None
+        args = self._step_args(tensors[0].dtype, want_stats, call.with_opt)
+        return call.run(args, stream=self._main_stream)
 
     # ------------------------------------------------------------------ trainer calls this
     def pending(self):

@@ -244,11 +244,7 @@ def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
     """One span by value (what a comm hook calls for the bucket it was handed)."""
     c_span = span.to_c()
     if span.bounds and bounds_dev is None:
-        host = np.zeros((len(span.bounds), 2), dtype=np.uint64)
-        for i, (start, group) in enumerate(span.bounds):
-            host[i, 0] = start
-            host[i, 1] = group                      # low 32 bits = group, high 32 = reserved
-        bounds_dev = torch.from_numpy(host.view(np.int64)).to(span.grads[0].device)
+        bounds_dev = bounds_to_device(span.bounds, span.grads[0].device)
     stats_ptr = ws_ptr = None
     ws_bytes = 0
     if args.stats:
@@ -261,6 +257,57 @@ def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
     if bounds_dev is not None:
         bounds_dev.record_stream(torch.cuda.current_stream() if stream is None else stream)
     return workspace.stats[0] if args.stats else None
+
+
+def bounds_to_device(bounds, device):
+    """Device copy of a span's bound table in JabasBound layout (for ``jabas_sync_bucket``)."""
+    host = np.zeros((len(bounds), 2), dtype=np.uint64)
+    for i, (start, group) in enumerate(bounds):
+        host[i, 0] = start
+        host[i, 1] = group                          # low 32 bits = group, high 32 = reserved
+    return torch.from_numpy(host.view(np.int64)).to(device)
+
+
+class BucketCall:
+    """One span prepared for repeated ``jabas_sync_bucket`` calls: the tensors are validated, the
+    C struct is filled, the bound table is on the device and the statistics workspace exists, so that
+    ``run`` is one foreign call. A comm hook sees the same bucket buffers every step; ``matches``
+    tells whether a prepared call still describes them."""
+
+    def __init__(self, span):
+        self.span = span
+        self.c_span = span.to_c()
+        g0 = span.grads[0]
+        self.key = self.key_of(span.grads)
+        self.bounds_dev = bounds_to_device(span.bounds, g0.device) if span.bounds else None
+        self.ws = None                              # created by the first statistics launch
+        self._fn = L.lib().jabas_sync_bucket
+
+    @staticmethod
+    def key_of(grads):
+        return tuple(g.data_ptr() for g in grads) + (grads[0].numel(),)
+
+    def matches(self, grads):
+        return self.key == self.key_of(grads)
+
+    def run(self, args, stream=None):
+        """Queues the step; returns the statistics row or None. Rows alternate between two device
+        buffers, so a returned row stays untouched by this call's next statistics launch and is
+        overwritten by the one after that."""
+        stats_ptr = ws_ptr = row = None
+        ws_bytes = 0
+        if args.stats:
+            if self.ws is None:
+                g0 = self.span.grads[0]
+                self.ws = Workspace.for_span(g0.numel(), g0.dtype, g0.device)
+                self._rows = torch.zeros(2, L.STATS_STRIDE, dtype=torch.float64, device=g0.device)
+                self._flip = 0
+            self._flip ^= 1
+            row = self._rows[self._flip]
+            stats_ptr, ws_ptr, ws_bytes = row.data_ptr(), self.ws.buf.data_ptr(), self.ws.nbytes
+        L.check(self._fn(C.byref(self.c_span), None if self.bounds_dev is None else self.bounds_dev.data_ptr(),
+                         C.byref(args), stats_ptr, ws_ptr, ws_bytes, _stream_ptr(stream)), "jabas_sync_bucket")
+        return row
 
 
 def _ptr_array(tensors):
