@@ -388,3 +388,114 @@ def test_special_values_denormals_infinities_nans(gpu):
     assert 0 < float(v_h[0]) < 1.2e-38                         # denormal second moment
     for a, b in ((p_d, p_h), (m_d, m_h), (v_d, v_h)):
         assert torch.equal(_bits(a), _bits(b))
+
+
+# ------------------------------------------------------------- randomized plans vs the oracle
+def _random_case(seed):
+    rng = np.random.RandomState(seed)
+    K = int(rng.randint(1, 9))
+    dtype = torch.bfloat16 if rng.rand() < 0.4 else torch.float32
+    opt = [None, SGD, ADAM, ADAMW][int(rng.randint(0, 4))]
+    if opt is SGD and rng.rand() < 0.3:
+        opt = dict(SGD, nesterov=True, momentum=0.8)
+    n_span = int(rng.randint(1, 25))
+    sizes = []
+    for _ in range(n_span):
+        kind = rng.rand()
+        if kind < 0.1:
+            sizes.append(0)
+        elif kind < 0.5:
+            sizes.append(int(rng.randint(1, 3000)))
+        elif kind < 0.8:
+            sizes.append(int(1024 * rng.randint(1, 9) + rng.choice([-1, 0, 1, 2])))
+        else:
+            sizes.append(int(rng.randint(20000, 120000)))
+    gaps = [int(rng.randint(0, 9)) for _ in sizes]
+    half_id = None
+    if K >= 2 and rng.rand() < 0.5:                      # arbitrary halves, both non-empty
+        while True:
+            half_id = [int(v) for v in rng.randint(0, 2, size=K)]
+            if 0 < sum(half_id) < K:
+                break
+    batches = tuple(int(v) for v in rng.randint(1, 65, size=K))
+    in_place = dtype == torch.float32 and rng.rand() < 0.5
+    n_fan = int(rng.randint(0, 3)) if opt else 0
+    bounds = []
+    for s in sizes:
+        if opt is None or s == 0:
+            bounds.append(())
+            continue
+        nb = int(rng.randint(0, 5))
+        starts = sorted(set([0] + [int(v) for v in rng.randint(1, max(2, s), size=nb) if v < s]))
+        bounds.append(tuple((st, int(rng.randint(0, 2))) for st in starts))
+    return K, dtype, opt, sizes, gaps, half_id, batches, in_place, n_fan, bounds
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_plans_match_the_oracle(gpu, seed):
+    """Random K, dtype, optimizer, span sizes (empty, sub-tile, tile-edge, large), line offsets, group
+    bounds, halves, fan-out and in-place aggregation: the planned launch against the oracle over 3 steps."""
+    from jabas_amd import sync, _lib as L
+    K, dtype, opt, sizes, gaps, half_id, batches, in_place, n_fan, bounds = _random_case(seed)
+    print(f"seed {seed}: K={K} {dtype} opt={opt and opt['kind']} spans={sizes} gaps={gaps} halves={half_id} "
+          f"in_place={in_place} fan={n_fan}", flush=True)
+    offs, off = [], 0
+    for s, gp in zip(sizes, gaps):
+        off += gp
+        offs.append(off)
+        off += s
+    total = max(off, 1)
+    hg = _host_grads(K, total, 300 + seed, std=5e-4, dtype=dtype)
+    p_h, s1_h, s2_h = _host_state(total, 40 + seed), torch.zeros(total), torch.zeros(total)
+    base_skew = seed % 4
+    dg = [_dev(t, gpu, base_skew) for t in hg]
+    agg_d = dg[0] if in_place else _dev(torch.zeros(total), gpu, base_skew)
+    p_d, s1_d, s2_d = _dev(p_h, gpu, base_skew), _dev(s1_h, gpu, base_skew), _dev(s2_h, gpu, base_skew)
+    fans = [_dev(torch.zeros(total), gpu, base_skew) for _ in range(n_fan)]
+    kind = sync.opt_kind(opt)
+    adam = kind in (L.OPT_ADAM, L.OPT_ADAMW)
+    spans_h, spans_d = [], []
+    for o, s, b in zip(offs, sizes, bounds):
+        sl = slice(o, o + s)
+        spans_h.append((o, s, b))
+        spans_d.append(sync.SpanSpec([g[sl] for g in dg], agg_out=agg_d[sl], param=p_d[sl] if opt else None,
+                                     state1=s1_d[sl] if opt else None, state2=s2_d[sl] if adam else None,
+                                     fanout=[f[sl] for f in fans], bounds=b))
+    plan = sync.SyncPlan(spans_d, kind)
+    hg_work = [t.clone() for t in hg]
+    for step in (1, 2, 3):
+        stats = step != 2
+        args = sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=step, first_step=(step == 1),
+                                   half_id=half_id)
+        rows = plan.run(args)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg_work, batches, spans_h, opt, p_h, s1_h, s2_h if adam else None, step=step,
+                                    first_step=(step == 1), want_stats=stats, half_id=half_id)
+        for i, (o, s, _) in enumerate(spans_h):
+            assert torch.equal(_bits(agg_d[o:o + s]), _bits(agg_h[o:o + s])), f"span {i} step {step}"
+        if stats:
+            rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+            got, want = rows.cpu()[:, :4 + K], rows_h[:, :4 + K]
+            scale = want[:, 1:3].abs().max(dim=1, keepdim=True).values.clamp_min(1e-300)   # dot may cancel: bound it by the norms
+            assert bool(((got - want).abs() <= rtol * want.abs() + 1e-9 * scale).all()), f"stats step {step}"
+        if opt:
+            for i, (o, s, _) in enumerate(spans_h):
+                assert torch.equal(_bits(p_d[o:o + s]), _bits(p_h[o:o + s])), f"weights span {i} step {step}"
+                assert torch.equal(_bits(s1_d[o:o + s]), _bits(s1_h[o:o + s])), f"state1 span {i} step {step}"
+                if adam:
+                    assert torch.equal(_bits(s2_d[o:o + s]), _bits(s2_h[o:o + s])), f"state2 span {i} step {step}"
+                for f in fans:
+                    assert torch.equal(_bits(f[o:o + s]), _bits(p_d[o:o + s]))
+        if in_place:
+            for (o, s, _) in spans_h:
+                hg_work[0][o:o + s] = agg_h[o:o + s]
+    # nothing outside the spans was written
+    covered = torch.zeros(total, dtype=torch.bool)
+    for o, s, _ in spans_h:
+        covered[o:o + s] = True
+    if opt and (~covered).any():
+        assert torch.equal(_bits(p_d)[~covered], _bits(_host_state(total, 40 + seed))[~covered])
+        for f in fans:
+            assert torch.count_nonzero(f.cpu()[~covered]) == 0
+    if not in_place and (~covered).any():
+        assert torch.count_nonzero(agg_d.cpu()[~covered]) == 0
