@@ -11,9 +11,10 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # JABAS_SYNC_LIB points at another build of the same library (kernel tuning experiments)
 LIB_PATH = os.environ.get("JABAS_SYNC_LIB") or os.path.join(_HERE, "csrc", "libjabas_sync.so")
 
-MAX_K = 8
+MAX_K = 16
 MAX_GROUPS = 16
-STATS_STRIDE = 12
+STATS_STRIDE = 20
+GRAM_MAX_K = 8
 GRAM_STRIDE = 64
 
 F32, BF16 = 0, 1

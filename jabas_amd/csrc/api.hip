@@ -17,7 +17,7 @@ namespace {
 
 constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 3;
+constexpr uint32_t kPlanVersion = 4;
 
 struct PlanHeader {
     uint32_t magic, version;
@@ -212,8 +212,10 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
 }
 
 typedef int (*LaunchFn)(int, int, int, const KArgs&, unsigned, hipStream_t);
-const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1, launch_fused_k2, launch_fused_k3, launch_fused_k4,
-                                       launch_fused_k5, launch_fused_k6, launch_fused_k7, launch_fused_k8};
+const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1,  launch_fused_k2,  launch_fused_k3,  launch_fused_k4,
+                                       launch_fused_k5,  launch_fused_k6,  launch_fused_k7,  launch_fused_k8,
+                                       launch_fused_k9,  launch_fused_k10, launch_fused_k11, launch_fused_k12,
+                                       launch_fused_k13, launch_fused_k14, launch_fused_k15, launch_fused_k16};
 
 // Second level of the statistics reduction: sums partial rows in a fixed order.
 //   stripes == 0  rows [s*in_stripes, (s+1)*in_stripes) of `in` -> row s of `out`
@@ -325,13 +327,13 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
 
 using namespace jabas;
 
-JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.1 (gfx950)"; }
+JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.2 (gfx950)"; }
 
 JABAS_API const char* jabas_status_string(int status) {
     switch (status) {
         case JABAS_OK: return "ok";
         case JABAS_ERR_NULL: return "a required pointer is NULL";
-        case JABAS_ERR_K: return "K outside 1..8 or half_id not 0/1";
+        case JABAS_ERR_K: return "K outside 1..16 (1..8 for jabas_gram) or half_id not 0/1";
         case JABAS_ERR_ALIGN: return "buffers of a span are not mutually congruent modulo 16 bytes";
         case JABAS_ERR_DTYPE: return "unsupported gradient dtype";
         case JABAS_ERR_OPT: return "unknown optimizer kind or inconsistent optimizer arguments";
@@ -561,7 +563,7 @@ JABAS_API int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtyp
 JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype, uint64_t numel,
                          double* gram_out, void* workspace, size_t workspace_bytes, jabas_stream_t stream) {
     if (!grads || !gram_out) return JABAS_ERR_NULL;
-    if (K < 1 || K > JABAS_MAX_K) return JABAS_ERR_K;
+    if (K < 1 || K > JABAS_GRAM_MAX_K) return JABAS_ERR_K;
     if (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(gram_out) % 8) return JABAS_ERR_ALIGN;

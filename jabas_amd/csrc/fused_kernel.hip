@@ -25,7 +25,7 @@
 #include "jabas_internal.h"
 
 #ifndef JABAS_K
-#error "compile with -DJABAS_K=<1..8>"
+#error "compile with -DJABAS_K=<1..16>"
 #endif
 // Most tiles whose loads are in flight together: a whole 4-tile chunk without statistics,
 // 2 tiles with (the fp64 accumulators need the registers).
@@ -289,7 +289,8 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     constexpr int EPT = GR::EPT;
     constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
     constexpr int UW = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
-    constexpr int U = UW < pick_chunk_tiles(K) ? UW : pick_chunk_tiles(K);   // never more than a chunk holds
+    constexpr int U0 = UW < pick_chunk_tiles(K) ? UW : pick_chunk_tiles(K);   // never more than a chunk holds
+    constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
     const uint32_t nb = sp.bound_count;
     const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
@@ -328,7 +329,7 @@ template <int K, int DT, int OPT, bool STATS>
 __device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const KArgs& a,
                                           double (&acc)[NStats<K, STATS>::value]) {
     if constexpr (STATS) {
-        constexpr uint32_t kDefaultMask = 0xAAu & ((1u << K) - 1u);
+        constexpr uint32_t kDefaultMask = 0xAAAAu & ((1u << K) - 1u);
         if (a.half_mask == kDefaultMask) span_range<K, DT, OPT, true, true>(sp, lt0, lt1, j0, a, acc);
         else span_range<K, DT, OPT, true, false>(sp, lt0, lt1, j0, a, acc);
     } else {
@@ -337,7 +338,7 @@ __device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint3
 }
 
 // Workgroup sum of NS per-thread accumulators -> one partial row. Through LDS rather than
-// wave shuffles: 12 stores + 16 loads per thread instead of ~18 DPP-and-add instructions per
+// wave shuffles: NS stores + 16 loads per thread instead of ~18 DPP-and-add instructions per
 // value, which matters because a workgroup only covers a few thousand elements.
 //   stage 1  thread (v, part) adds entries part, part+16, ..., part+240 of value v (in order);
 //   stage 2  the 16 parts of a value sit in one 16-lane row: DPP row reduction.
@@ -349,19 +350,21 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
 #pragma unroll
     for (int i = 0; i < NS; ++i) buf[i][tid] = acc[i];
     __syncthreads();
-    if (tid < NS * 16) {
-        const int v = tid >> 4, part = tid & 15;
-        double s = buf[v][part];
 #pragma unroll
-        for (int i = 1; i < 16; ++i) s += buf[v][i * 16 + part];
-        s += dpp_move<0xB1, 0xf>(s);     // quad_perm [1,0,3,2]
-        s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
-        s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
-        s += dpp_move<0x140, 0xf>(s);    // row_mirror
-        if (part == 0) row[v] = s;
-    } else if (tid >= kBlock - (kStatsStride - NS)) {
-        row[NS + (tid - (kBlock - (kStatsStride - NS)))] = 0.0;     // unused slots of the row
+    for (int v0 = 0; v0 < NS; v0 += 16) {          // 16 values per pass (K > 12 needs a second one)
+        if (tid < (NS - v0) * 16) {
+            const int v = v0 + (tid >> 4), part = tid & 15;
+            double s = buf[v][part];
+#pragma unroll
+            for (int i = 1; i < 16; ++i) s += buf[v][i * 16 + part];
+            s += dpp_move<0xB1, 0xf>(s);     // quad_perm [1,0,3,2]
+            s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
+            s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
+            s += dpp_move<0x140, 0xf>(s);    // row_mirror
+            if (part == 0) row[v] = s;
+        }
     }
+    if (tid >= kBlock - (kStatsStride - NS)) row[NS + (tid - (kBlock - (kStatsStride - NS)))] = 0.0;   // unused slots
 }
 
 template <int K, int DT, int OPT, bool STATS>

@@ -101,8 +101,8 @@ __global__ void __launch_bounds__(64) gram_finalize_kernel(int K, const double* 
     int a = 0;
     while ((a + 1) * (a + 2) / 2 <= t) ++a;  // packed index t = a*(a+1)/2 + b, b <= a
     const int b = t - a * (a + 1) / 2;
-    gram_out[a * JABAS_MAX_K + b] = s;
-    gram_out[b * JABAS_MAX_K + a] = s;
+    gram_out[a * JABAS_GRAM_MAX_K + b] = s;
+    gram_out[b * JABAS_GRAM_MAX_K + a] = s;
 }
 
 template <int K>

@@ -121,6 +121,8 @@ __device__ __forceinline__ double wave_sum_to_lane63(double v) {
                           unsigned grid, hipStream_t stream);
 JABAS_DECLARE_K(1) JABAS_DECLARE_K(2) JABAS_DECLARE_K(3) JABAS_DECLARE_K(4)
 JABAS_DECLARE_K(5) JABAS_DECLARE_K(6) JABAS_DECLARE_K(7) JABAS_DECLARE_K(8)
+JABAS_DECLARE_K(9) JABAS_DECLARE_K(10) JABAS_DECLARE_K(11) JABAS_DECLARE_K(12)
+JABAS_DECLARE_K(13) JABAS_DECLARE_K(14) JABAS_DECLARE_K(15) JABAS_DECLARE_K(16)
 #undef JABAS_DECLARE_K
 
 }  // namespace jabas

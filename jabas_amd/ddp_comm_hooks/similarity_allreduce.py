@@ -9,7 +9,7 @@ empties the list after reading it (jabas/train/trainer.py:184-195,480).
 What changed underneath: the reference clones the bucket, sums it over a sub-group and
 divides (a second copy of every gradient plus four passes); here the half-gradient
 statistics come out of the same fused kernel that aggregates the bucket, so the entry
-appended is a ``BucketStats`` (12 doubles on the device), not a gradient-sized tensor.
+appended is a ``BucketStats`` (4 + 16 doubles on the device), not a gradient-sized tensor.
 ``cosine_similarity_from_placeholder`` is the matching reader.
 """
 import torch

@@ -231,7 +231,7 @@ class SyncPlan:
 
     def run(self, args, stream=None):
         """Queues aggregate (+stats, +optimizer) over every span. Returns the stats tensor
-        (n_span x 12 doubles, device) when args.stats is set, else None."""
+        (n_span x STATS_STRIDE doubles, device) when args.stats is set, else None."""
         L.check(L.lib().jabas_sync_fused(self._host.ctypes.data, self._dev.data_ptr(), C.byref(args),
                                          self.ws.stats.data_ptr() if args.stats else None,
                                          self.ws.buf.data_ptr(), self.ws.nbytes, _stream_ptr(stream)),
@@ -334,7 +334,7 @@ def aggregate(grads, batches, out=None, stream=None):
 
 
 def gradient_stats(grads, batches, half_id=None, workspace=None, stream=None):
-    """Statistics row (12 doubles, device) of one span; writes nothing else."""
+    """Statistics row (STATS_STRIDE doubles, device) of one span; writes nothing else."""
     span = SpanSpec(grads)
     n, dev, gdt = span.validate()
     w, hid, hw = batch_weights(batches, half_id)
@@ -362,7 +362,7 @@ def gram(grads, stream=None):
     L.check(L.lib().jabas_gram(_ptr_array(grads), K, grad_dtype_code(gdt), n, out.data_ptr(), ws.data_ptr(),
                                ws.numel() * 8, _stream_ptr(stream)), "jabas_gram")
     ws.record_stream(torch.cuda.current_stream() if stream is None else stream)
-    return out.view(L.MAX_K, L.MAX_K)[:K, :K]
+    return out.view(L.GRAM_MAX_K, L.GRAM_MAX_K)[:K, :K]
 
 
 def sgd_step(grad, param, momentum_buf, lr, weight_decay=0.0, momentum=0.0, dampening=0.0, nesterov=False,

@@ -33,7 +33,7 @@ import math
 import numpy as np
 import torch
 
-STATS_STRIDE = 12
+STATS_STRIDE = 20
 DOT_AB, NORM_A, NORM_B, NORM_AGG, NORM_VSW0 = 0, 1, 2, 3, 4
 
 

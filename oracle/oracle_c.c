@@ -49,7 +49,7 @@ void oc_aggregate(const void* const* g, int K, int bf16, const float* w, float* 
 /* row[0]=dot(gA,gB) row[1]=|gA|^2 row[2]=|gB|^2 row[3]=|gbar|^2 row[4+k]=|g_k|^2; fp64 sums */
 void oc_stats(const void* const* g, int K, int bf16, const float* w, const uint8_t* half, const float* hw,
               size_t n, double* row) {
-    for (int i = 0; i < 12; ++i) row[i] = 0.0;
+    for (int i = 0; i < 4 + K; ++i) row[i] = 0.0;      /* the caller's row holds at least 4 + K entries */
     for (size_t i = 0; i < n; ++i) {
         float acc = 0.0f, ga = 0.0f, gb = 0.0f;
         int seen_a = 0, seen_b = 0;

@@ -32,10 +32,12 @@ def test_library_exports_every_declared_symbol():
 
 def test_struct_layouts_match_the_header():
     # sizes a C compiler gives the header's structs on x86-64 / amdgcn host ABI
-    assert C.sizeof(L.JabasSpan) == 8 * 8 + 4 * 8 + 7 * 8 + 8 + 4 * 4
+    K = L.MAX_K
+    assert K == 16 and L.STATS_STRIDE == 4 + K
+    assert C.sizeof(L.JabasSpan) == K * 8 + 4 * 8 + (K - 1) * 8 + 8 + 4 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
-    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 32 + 4 + 8 + 32 + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8
+    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 4 * K + 4 + K + 4 * K + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8
     assert L.JabasStepArgs.groups.offset % 8 == 0 and L.JabasStepArgs.momentum.offset % 8 == 0
 
 
@@ -52,11 +54,11 @@ def _span(numel, base=0x7f0000000000, K=2, gs=4, skew=0, opt=False, stride=1 << 
     s = L.JabasSpan()
     for k in range(K):
         s.grads[k] = base + k * stride + skew * gs
-    s.agg_out = base + 8 * stride + skew * 4
+    s.agg_out = base + 16 * stride + skew * 4
     if opt:
-        s.param = base + 9 * stride + skew * 4
-        s.state1 = base + 10 * stride + skew * 4
-        s.state2 = base + 11 * stride + skew * 4
+        s.param = base + 17 * stride + skew * 4
+        s.state1 = base + 18 * stride + skew * 4
+        s.state2 = base + 19 * stride + skew * 4
     s.numel = numel
     return s
 
@@ -81,10 +83,11 @@ def test_plan_encode_counts_chunks():
     rc, blob, _ = _encode([_span(n) for n in sizes])
     assert rc == L.OK
     assert lib.jabas_plan_chunks(blob.ctypes.data) == 2 + 3 + 1 + 0 + 21
-    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (27 + 5) * 12 * 8     # a row per chunk and per span, at least
-    rc, blob, _ = _encode([_span(n, K=8) for n in sizes], K=8)
-    assert rc == L.OK
-    assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
+    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (27 + 5) * L.STATS_STRIDE * 8     # a row per chunk and per span, at least
+    for K in (8, 16):
+        rc, blob, _ = _encode([_span(n, K=K) for n in sizes], K=K)
+        assert rc == L.OK
+        assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
     # a span that starts 3 elements into a 16-byte line needs one more tile when it is exactly full
     rc, blob, _ = _encode([_span(4096, skew=3)])
     assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data) == 3
@@ -107,7 +110,7 @@ def test_plan_encode_rejects_bad_spans():
     s = _span(4096)
     s.grads[1] = 0
     assert _encode([s])[0] == L.ERR_NULL
-    assert _encode([_span(4096)], K=9)[0] == L.ERR_K
+    assert _encode([_span(4096)], K=17)[0] == L.ERR_K
     assert _encode([_span(4096)], dtype=7)[0] == L.ERR_DTYPE
     assert _encode([_span(4096)], opt=9)[0] == L.ERR_OPT
     assert _encode([_span(4096)], opt=L.OPT_SGD)[0] == L.ERR_NULL    # optimizer without weights
@@ -125,7 +128,7 @@ def test_plan_encode_rejects_bad_spans():
     s.agg_out = s.grads[0]
     assert _encode([s], dtype=L.BF16)[0] == L.ERR_ALIAS          # fp32 output over bf16 input
     s = _span(4096, opt=True)
-    s.n_fanout = 8
+    s.n_fanout = 16
     assert _encode([s], opt=L.OPT_SGD)[0] == L.ERR_SIZE
 
 
@@ -159,9 +162,10 @@ def test_plan_blob_too_small_and_garbage_header():
 
 def test_workspace_bytes_cover_any_line_position():
     lib = L.lib()
-    assert lib.jabas_sync_workspace_bytes(0, L.F32) >= 96
-    assert lib.jabas_sync_workspace_bytes(4096, L.F32) >= 3 * 96      # a shifted start adds a chunk
-    assert lib.jabas_sync_workspace_bytes(1 << 30, L.BF16) >= ((1 << 30) // 2048) * 96
+    row = L.STATS_STRIDE * 8
+    assert lib.jabas_sync_workspace_bytes(0, L.F32) >= row
+    assert lib.jabas_sync_workspace_bytes(4096, L.F32) >= 3 * row      # a shifted start adds a chunk
+    assert lib.jabas_sync_workspace_bytes(1 << 30, L.BF16) >= ((1 << 30) // 2048) * row
 
 
 def test_entry_points_validate_before_launching():
@@ -230,7 +234,7 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
     assert seen[("status0", "ok")] == ""
     assert seen[("encode", "0")] == ""
     assert seen[("chunks", "8")] == ""                       # 5000 -> 3 chunks of 2 tiles, 9096 -> 5
-    assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * 96
+    assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * L.STATS_STRIDE * 8
     assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
 
 

@@ -15,7 +15,9 @@ from oracle import oracle as O
 pytestmark = pytest.mark.gpu
 
 BATCHES = {1: (32,), 2: (32, 32), 3: (4, 2, 2), 4: (48, 32, 32, 16), 5: (5, 4, 3, 2, 1),
-           6: (7, 7, 5, 3, 2, 1), 7: (64, 56, 48, 40, 32, 24, 16), 8: tuple(range(64, 0, -8))}
+           6: (7, 7, 5, 3, 2, 1), 7: (64, 56, 48, 40, 32, 24, 16), 8: tuple(range(64, 0, -8)),
+           9: (9, 8, 7, 6, 5, 4, 3, 2, 1), 10: (16,) * 10, 11: tuple(range(11, 0, -1)), 12: (32, 16, 8) * 4,
+           13: tuple(range(1, 14)), 14: (3, 5) * 7, 15: tuple(range(30, 0, -2)), 16: tuple(range(64, 0, -4))}
 
 SGD = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
            groups=[dict(lr=0.1, weight_decay=0.0), dict(lr=0.1, weight_decay=1e-4)])
@@ -63,7 +65,7 @@ def _same_bits(a, b):
 
 
 # ---------------------------------------------------------------------------- aggregate
-@pytest.mark.parametrize("K", range(1, 9))
+@pytest.mark.parametrize("K", range(1, 17))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_aggregate_bit_exact(gpu, K, dtype):
     from jabas_amd import sync
@@ -104,7 +106,7 @@ def test_aggregate_keeps_zero_rows_exactly_zero(gpu):
 
 
 # --------------------------------------------------------------------------- statistics
-@pytest.mark.parametrize("K", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 5, 8, 9, 12, 13, 16])
 @pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-6), (torch.bfloat16, 1e-2)])
 def test_stats_row(gpu, K, dtype, rtol):
     from jabas_amd import sync
@@ -151,6 +153,14 @@ def test_gram(gpu, K, dtype):
         want = O.gram(hg)
         assert _close(G, want, 1e-11, 1e-30)[0], f"K={K} n={n}"
         assert torch.equal(G, G.t())
+
+
+def test_gram_is_limited_to_eight_workers(gpu):
+    from jabas_amd import sync, _lib as L
+    g = [torch.zeros(4096, device=gpu) for _ in range(9)]
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.gram(g)
+    assert e.value.status == L.ERR_K
 
 
 # ---------------------------------------------------------------------------- optimizer
@@ -206,7 +216,10 @@ def test_adam_steps(gpu, hp):
 # ------------------------------------------------------------------ fused, single bucket
 @pytest.mark.parametrize("K,dtype,opt", [(2, torch.float32, SGD), (4, torch.float32, ADAMW),
                                          (3, torch.float32, ADAM), (8, torch.bfloat16, ADAMW),
-                                         (5, torch.bfloat16, SGD), (1, torch.float32, ADAM)])
+                                         (5, torch.bfloat16, SGD), (1, torch.float32, ADAM),
+                                         (9, torch.float32, ADAM), (12, torch.float32, SGD),
+                                         (13, torch.bfloat16, ADAM), (16, torch.bfloat16, ADAMW),
+                                         (16, torch.float32, ADAMW)])
 def test_sync_bucket_fused(gpu, K, dtype, opt):
     from jabas_amd import sync
     n = 200003
@@ -246,7 +259,8 @@ def test_sync_bucket_fused(gpu, K, dtype, opt):
 @pytest.mark.parametrize("K,dtype,opt,in_place", [
     (2, torch.float32, SGD, True), (4, torch.float32, ADAMW, True), (3, torch.float32, SGD, False),
     (4, torch.float32, ADAM, False), (8, torch.bfloat16, ADAMW, False), (6, torch.float32, None, True),
-    (7, torch.bfloat16, None, False)])
+    (7, torch.bfloat16, None, False), (10, torch.float32, ADAMW, True), (16, torch.bfloat16, SGD, False),
+    (15, torch.float32, None, False)])
 def test_sync_fused_plan_ragged_spans(gpu, K, dtype, opt, in_place):
     from jabas_amd import sync, _lib as L
     # span sizes: tiny, exactly one tile, ragged, empty, large; offsets chosen so that some
@@ -321,7 +335,7 @@ def test_fused_rejects_bad_arguments(gpu):
         sync.aggregate([g[0][:n], g[1][:n]], (1, 1), out=g[0][4:n + 4])      # partial overlap
     assert e.value.status == L.ERR_ALIAS
     with pytest.raises(ValueError):
-        sync.aggregate([g[0][:n]] * 9, (1,) * 9)
+        sync.aggregate([g[0][:n]] * 17, (1,) * 17)
     span = sync.SpanSpec([g[0][:n], g[1][:n]], param=None)
     args = sync.make_step_args((1, 1), torch.float32, opt=SGD)
     with pytest.raises(L.JabasSyncError) as e:
@@ -393,7 +407,7 @@ def test_special_values_denormals_infinities_nans(gpu):
 # ------------------------------------------------------------- randomized plans vs the oracle
 def _random_case(seed):
     rng = np.random.RandomState(seed)
-    K = int(rng.randint(1, 9))
+    K = int(rng.randint(1, 9)) if seed < 16 else int(rng.randint(9, 17))
     dtype = torch.bfloat16 if rng.rand() < 0.4 else torch.float32
     opt = [None, SGD, ADAM, ADAMW][int(rng.randint(0, 4))]
     if opt is SGD and rng.rand() < 0.3:
@@ -431,7 +445,7 @@ def _random_case(seed):
     return K, dtype, opt, sizes, gaps, half_id, batches, in_place, n_fan, bounds
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_plans_match_the_oracle(gpu, seed):
     """Random K, dtype, optimizer, span sizes (empty, sub-tile, tile-edge, large), line offsets, group
     bounds, halves, fan-out and in-place aggregation: the planned launch against the oracle over 3 steps."""
