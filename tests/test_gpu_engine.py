@@ -107,8 +107,8 @@ def test_reconfigure_changes_k_and_keeps_weights_and_state(gpu):
     O.sync_step(host["g"], batches, spans, ADAM, host["p"], host["s1"], host["s2"], step=1, first_step=True)
     torch.cuda.synchronize()
     p_before, m_before = eng.param.clone(), eng.state1.clone()
-    # grow to 3 workers, then shrink to 1
-    for new_batches, step in (((4, 4, 4), 2), ((4,), 3)):
+    # grow to 3 workers, shrink to 1, grow past 8, to the maximum, and back
+    for new_batches, step in (((4, 4, 4), 2), ((4,), 3), ((2,) * 11, 4), (tuple(range(16, 0, -1)), 5), ((8, 8), 6)):
         eng.reconfigure(new_batches)
         assert eng.K == len(new_batches) and len(eng.grads) == eng.K and len(eng.fanout) == eng.K - 1
         assert torch.equal(eng.param, p_before) and torch.equal(eng.state1, m_before)
