@@ -29,7 +29,9 @@ def _bits(t):
 
 
 BATCHES = {1: (32,), 2: (32, 32), 3: (4, 2, 2), 4: (48, 32, 32, 16), 5: (5, 4, 3, 2, 1),
-           6: (7, 7, 5, 3, 2, 1), 7: (64, 56, 48, 40, 32, 24, 16), 8: tuple(range(64, 0, -8))}
+           6: (7, 7, 5, 3, 2, 1), 7: (64, 56, 48, 40, 32, 24, 16), 8: tuple(range(64, 0, -8)),
+           9: (9, 8, 7, 6, 5, 4, 3, 2, 1), 12: (32, 16, 8) * 4, 13: tuple(range(1, 14)),
+           16: tuple(range(64, 0, -4))}
 
 
 # ------------------------------------------------------------------------------ weights
@@ -44,7 +46,7 @@ def test_batch_weights_are_double_quotients_rounded_once():
 
 
 # ---------------------------------------------------------------------------- aggregate
-@pytest.mark.parametrize("K", range(1, 9))
+@pytest.mark.parametrize("K", list(range(1, 9)) + [9, 12, 13, 16])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_aggregate_matches_c_restatement_bitwise(K, dtype):
     g = _grads(K, 4099, K, dtype=dtype)
@@ -71,7 +73,7 @@ def test_aggregate_k1_is_identity():
     assert torch.equal(_bits(O.aggregate(g, (32,))), _bits(g[0]))
 
 
-@pytest.mark.parametrize("K", [2, 4, 8])
+@pytest.mark.parametrize("K", [2, 4, 8, 16])
 def test_aggregate_equal_batches_power_of_two_is_sum_then_divide(K):
     # the reference's own pattern: sum over workers, then one division by the count
     # (similarity_allreduce.py:32); exact for power-of-two counts
@@ -116,7 +118,7 @@ def test_bf16_widening_is_exact():
 
 
 # --------------------------------------------------------------------------- statistics
-@pytest.mark.parametrize("K", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 8, 9, 13, 16])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_stats_match_c_restatement(K, dtype):
     g = _grads(K, 10007, 20 + K, dtype=dtype)
