@@ -17,7 +17,7 @@ namespace {
 
 constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 4;
+constexpr uint32_t kPlanVersion = 5;
 
 struct PlanHeader {
     uint32_t magic, version;
@@ -27,10 +27,13 @@ struct PlanHeader {
     uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
     uint32_t chunk_tiles;     // tiles per workgroup the chunk table was cut for
     uint32_t max_span_chunks; // chunks of the largest span (sizes the striped finalize)
+    uint32_t block;           // threads per workgroup the chunk table was cut for
+    uint32_t pad;
     uint64_t off_spans, off_prefix, off_chunks, off_bounds, total_bytes;
 };
-static_assert(sizeof(PlanHeader) == 88, "plan header layout");
+static_assert(sizeof(PlanHeader) == 96, "plan header layout");
 constexpr size_t kHeaderBytes = 96;
+static_assert(kHeaderBytes >= sizeof(PlanHeader) && kHeaderBytes % 16 == 0, "plan header slot");
 
 inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
 
@@ -50,17 +53,17 @@ inline bool ranges_overlap(const void* a, size_t na, const void* b, size_t nb) {
 }
 
 // Tiles a span occupies, counted from the 16-byte line its first element falls in.
-inline uint64_t span_tiles(const JabasSpan& in, int grad_dtype) {
+inline uint64_t span_tiles(const JabasSpan& in, int grad_dtype, int block) {
     if (in.numel == 0) return 0;
     const int gs = grad_dtype == JABAS_BF16 ? 2 : 4;
     const uint64_t skew = (reinterpret_cast<uintptr_t>(in.grads[0]) / gs) % ept_of(grad_dtype);
-    const uint64_t te = tile_elems(grad_dtype);
+    const uint64_t te = tile_elems_of(block);
     return (skew + in.numel + te - 1) / te;
 }
 inline uint64_t chunks_of_tiles(uint64_t tiles, uint64_t ct) { return (tiles + ct - 1) / ct; }
 
 // Validates one span and produces the rebased device view. Host-only logic.
-int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDev* out, uint32_t* tiles) {
+int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int block, SpanDev* out, uint32_t* tiles) {
     const int gs = grad_dtype == JABAS_BF16 ? 2 : 4;
     const int ept = ept_of(grad_dtype);
     if (in.numel > (static_cast<uint64_t>(1) << 40)) return JABAS_ERR_SIZE;
@@ -138,7 +141,7 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, SpanDe
     out->hi = skew + in.numel;
     out->bound_begin = in.bound_begin;
     out->bound_count = in.bound_count;
-    const uint64_t te = tile_elems(grad_dtype);
+    const uint64_t te = tile_elems_of(block);
     const uint64_t nt = in.numel ? (out->hi + te - 1) / te : 0;
     if (nt > 0x7fffffffull) return JABAS_ERR_SIZE;
     *tiles = static_cast<uint32_t>(nt);
@@ -349,16 +352,16 @@ JABAS_API const char* jabas_status_string(int status) {
 
 JABAS_API size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype) {
     // chunks of a single span whose first element may sit anywhere in a 16-byte line
+    // under the launch shape with the smallest chunks
     const int dt = grad_dtype == JABAS_BF16 ? JABAS_BF16 : JABAS_F32;
-    const uint64_t te = tile_elems(dt);
-    const uint64_t tiles = (numel + ept_of(dt) - 1 + te - 1) / te;
-    return workspace_rows(chunks_of_tiles(tiles, kMinChunkTiles), 1) * kStatsStride * sizeof(double);
+    const uint64_t chunks = (numel + ept_of(dt) - 1 + kMinChunkElems - 1) / kMinChunkElems;
+    return workspace_rows(chunks, 1) * kStatsStride * sizeof(double);
 }
 
 namespace {
-uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype, uint64_t ct) {
+uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype, int block, uint64_t ct) {
     uint64_t n = 0;
-    for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype), ct);
+    for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype, block), ct);
     return n;
 }
 size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
@@ -371,7 +374,8 @@ size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
 
 JABAS_API size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds, int32_t grad_dtype) {
     if (!spans || (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16)) return 0;
-    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype, kMinChunkTiles));
+    // K and the optimizer are not known here: size for the launch shape with the smallest chunks
+    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype, kMinChunkElems / 4, 1));
 }
 
 JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
@@ -386,8 +390,9 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     if (opt_class_of(opt_kind) < 0) return JABAS_ERR_OPT;
     for (uint32_t i = 0; i < n_span; ++i)
         if (spans[i].numel && !spans[i].grads[0]) return JABAS_ERR_NULL;
-    const uint32_t ct = pick_chunk_tiles(K);
-    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype, ct);
+    const int block = launch_block(K, grad_dtype, opt_class_of(opt_kind));
+    const uint32_t ct = launch_chunk_tiles(K, grad_dtype, opt_class_of(opt_kind));
+    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype, block, ct);
     if (n_chunks > 0x7fffffffull) return JABAS_ERR_SIZE;
     const size_t need = plan_bytes_for(n_span, n_bounds, n_chunks);
     if (blob_bytes < need) return JABAS_ERR_PLAN;
@@ -406,6 +411,7 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     h.grad_dtype = grad_dtype;
     h.opt_kind = opt_kind;
     h.chunk_tiles = ct;
+    h.block = static_cast<uint32_t>(block);
     h.off_spans = kHeaderBytes;
     h.off_prefix = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
     h.off_chunks = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
@@ -416,11 +422,11 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     SpanDev* sd = reinterpret_cast<SpanDev*>(base + h.off_spans);
     uint32_t* prefix = reinterpret_cast<uint32_t*>(base + h.off_prefix);
     ChunkDesc* cd = reinterpret_cast<ChunkDesc*>(base + h.off_chunks);
-    const uint64_t te = tile_elems(grad_dtype);
+    const uint64_t te = tile_elems_of(block);
     uint32_t c = 0;
     for (uint32_t i = 0; i < n_span; ++i) {
         uint32_t tiles = 0;
-        int rc = encode_span(spans[i], K, grad_dtype, opt_kind, &sd[i], &tiles);
+        int rc = encode_span(spans[i], K, grad_dtype, opt_kind, block, &sd[i], &tiles);
         if (rc != JABAS_OK) return rc;
         rc = check_bounds_host(spans[i], bounds, n_bounds, &h.max_group);
         if (rc != JABAS_OK) return rc;
@@ -477,8 +483,13 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     if (rc != JABAS_OK) return rc;
     if (args->K != h.K || args->grad_dtype != h.grad_dtype) return JABAS_ERR_PLAN;
     const int oc = opt_class_of(args->opt_kind);
+    // the chunk table is cut for the launch shape of (K, dtype, optimizer class), and the state pointers
+    // were validated for that class only
+    if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;
+    if (h.block != static_cast<uint32_t>(launch_block(h.K, h.grad_dtype, oc)) ||
+        h.chunk_tiles != static_cast<uint32_t>(launch_chunk_tiles(h.K, h.grad_dtype, oc)))
+        return JABAS_ERR_PLAN;
     if (oc != 0) {
-        if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;       // state pointers were not validated
         if (h.max_group >= static_cast<uint32_t>(args->n_groups)) return JABAS_ERR_GROUP;
         if (oc == 1 && args->momentum != 0.0 && !h.all_have_s1) return JABAS_ERR_NULL;
     }
@@ -502,9 +513,10 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     int rc = fill_kargs(args, &a);
     if (rc != JABAS_OK) return rc;
     uint32_t tiles = 0;
-    rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind, &a.span0, &tiles);
-    if (rc != JABAS_OK) return rc;
     const int oc = opt_class_of(args->opt_kind);
+    rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind, launch_block(args->K, args->grad_dtype, oc),
+                     &a.span0, &tiles);
+    if (rc != JABAS_OK) return rc;
     if (oc == 1 && args->momentum != 0.0 && !span->state1) return JABAS_ERR_NULL;
     if (span->bound_count && !bounds_dev) return JABAS_ERR_NULL;
     // bounds_dev is indexed from its own start: the span's entries begin at element 0 of it
@@ -514,7 +526,7 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.chunks = nullptr;
     a.chunk_prefix = nullptr;
     a.n_span = 1;
-    a.chunk_tiles = pick_chunk_tiles(args->K);
+    a.chunk_tiles = launch_chunk_tiles(args->K, args->grad_dtype, oc);
     a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, a.chunk_tiles));
     a.use_inline = 1;
     return run_fused(a, args, a.n_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
@@ -573,7 +585,7 @@ JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype
     sp.numel = numel;
     SpanDev sd;
     uint32_t tiles = 0;
-    const int rc = encode_span(sp, K, grad_dtype, JABAS_OPT_NONE, &sd, &tiles);
+    const int rc = encode_span(sp, K, grad_dtype, JABAS_OPT_NONE, kBlock, &sd, &tiles);
     if (rc != JABAS_OK) return rc;
     uint64_t g = kGramGrid;
     if (g > tiles) g = tiles;

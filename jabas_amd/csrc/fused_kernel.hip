@@ -173,7 +173,7 @@ template <int K, int DT, int OPT, int U>
 __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
-    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
@@ -194,7 +194,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
                                         double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
-    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
@@ -226,7 +226,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
                                          const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
-    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * Grad<DT>::EPT;
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     uint32_t i = 0;
@@ -287,9 +287,10 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
-    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
     constexpr int UW = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
-    constexpr int U0 = UW < pick_chunk_tiles(K) ? UW : pick_chunk_tiles(K);   // never more than a chunk holds
+    constexpr int CT = launch_chunk_tiles(K, DT, OPT);
+    constexpr int U0 = UW < CT ? UW : CT;     // never more than a chunk holds
     constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
     const uint32_t nb = sp.bound_count;
@@ -343,20 +344,23 @@ __device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint3
 //   stage 1  thread (v, part) adds entries part, part+16, ..., part+240 of value v (in order);
 //   stage 2  the 16 parts of a value sit in one 16-lane row: DPP row reduction.
 // The order is fixed, so the row is bit-identical from run to run.
-template <int NS>
+template <int NS, int BS>
 __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
-    __shared__ double buf[NS][kBlock];
+    constexpr int kParts = 16;                       // lanes of one DPP row
+    constexpr int kPerPass = BS / kParts;            // values reduced per pass (16 with 256 threads)
+    __shared__ double buf[NS][BS];
     const int tid = threadIdx.x;
 #pragma unroll
     for (int i = 0; i < NS; ++i) buf[i][tid] = acc[i];
     __syncthreads();
+    static_assert(kStatsStride - NS <= BS, "one thread per unused slot");
 #pragma unroll
-    for (int v0 = 0; v0 < NS; v0 += 16) {          // 16 values per pass (K > 12 needs a second one)
-        if (tid < (NS - v0) * 16) {
+    for (int v0 = 0; v0 < NS; v0 += kPerPass) {      // K > 12 needs a second pass at 256 threads
+        if (tid < (NS - v0) * kParts) {
             const int v = v0 + (tid >> 4), part = tid & 15;
             double s = buf[v][part];
 #pragma unroll
-            for (int i = 1; i < 16; ++i) s += buf[v][i * 16 + part];
+            for (int i = 1; i < BS / kParts; ++i) s += buf[v][i * kParts + part];
             s += dpp_move<0xB1, 0xf>(s);     // quad_perm [1,0,3,2]
             s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
             s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
@@ -364,13 +368,15 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
             if (part == 0) row[v] = s;
         }
     }
-    if (tid >= kBlock - (kStatsStride - NS)) row[NS + (tid - (kBlock - (kStatsStride - NS)))] = 0.0;   // unused slots
+    if (tid < kStatsStride - NS) row[NS + tid] = 0.0;          // unused slots of the row
 }
 
 template <int K, int DT, int OPT, bool STATS>
-__global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
+__global__ void __launch_bounds__(launch_block(K, DT, OPT)) fused_kernel(const KArgs a) {
     constexpr int NS = NStats<K, STATS>::value;
-    constexpr uint64_t TE = static_cast<uint64_t>(kBlock) * Grad<DT>::EPT;
+    constexpr int BS = launch_block(K, DT, OPT);
+    constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT);     // the host cuts the chunk table for the same shape
+    constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
     const uint32_t b = blockIdx.x;
     double acc[NS];
 #pragma unroll
@@ -379,8 +385,8 @@ __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
     if (a.use_inline) {
         const SpanDev& sp = a.span0;
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
-        const uint32_t lt0 = b * a.chunk_tiles;
-        const uint32_t lt1 = lt0 + a.chunk_tiles < tiles ? lt0 + a.chunk_tiles : tiles;
+        const uint32_t lt0 = b * CT;
+        const uint32_t lt1 = lt0 + CT < tiles ? lt0 + CT : tiles;
         uint32_t j0 = 0;
         if (sp.bound_count) {                  // largest j with bounds[j].start <= first live element
             const BoundDev* bd = a.bounds + sp.bound_begin;
@@ -398,10 +404,10 @@ __global__ void __launch_bounds__(kBlock) fused_kernel(const KArgs a) {
         const ChunkDesc c = a.chunks[b];
         const SpanDev& sp = a.spans[c.span];
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
-        const uint32_t lt1 = c.tile0 + a.chunk_tiles < tiles ? c.tile0 + a.chunk_tiles : tiles;
+        const uint32_t lt1 = c.tile0 + CT < tiles ? c.tile0 + CT : tiles;
         run_chunk<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
-    if constexpr (STATS) flush_stats<NS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);
+    if constexpr (STATS) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);
 }
 
 template <int K, int DT, int OPT, bool STATS>
@@ -411,8 +417,11 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
     // mixes as long as the kernel does not need the waves to hide its own arithmetic. Measured (A/B in
     // one process): Adam/AdamW without statistics at K <= 4, fp32 gradients, gains 1-4 % at 5 workgroups
     // per CU instead of the 6 its registers allow; SGD kernels and every statistics kernel lose.
-    constexpr unsigned idle = (OPT == OPT_ADAM && !STATS && K <= 4 && DT == JABAS_F32) ? 32768u : 0u;
-    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(kBlock), idle, stream, a);
+#ifndef JABAS_IDLE_LDS_BYTES
+#define JABAS_IDLE_LDS_BYTES 32768u
+#endif
+    constexpr unsigned idle = (OPT == OPT_ADAM && !STATS && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
+    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(launch_block(K, DT, OPT)), idle, stream, a);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -8,21 +8,50 @@
 
 namespace jabas {
 
-constexpr int kBlock = 256;                 // threads per workgroup = 4 wave64
+// Launch shape: threads per workgroup and tiles per workgroup (a tile = one 16-byte fp32 vector per
+// thread; a chunk = the tiles one workgroup processes). Small chunks keep the streamed window of every
+// buffer compact (higher HBM rate) and cut the ramp-up / drain of a launch; kernels with many gradient
+// streams have low occupancy and a long prologue, and do better with twice the work per workgroup.
+// Measured per kernel family (A/B builds of the whole library):
+//   SGD, fp32 gradients, K <= 4   128 threads x 2 tiles (1024 elements): +2-5 % over 256 x 2
+//   Adam/AdamW and every other    256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
+//   case                          1024 threads were all slower with statistics on
+// The macros let a tuning build try other shapes without touching the sources.
+#ifndef JABAS_BLOCK
+#define JABAS_BLOCK 256
+#endif
+#ifndef JABAS_BLOCK_SGD
+#define JABAS_BLOCK_SGD 128
+#endif
+#ifndef JABAS_CHUNK_TILES_LO
+#define JABAS_CHUNK_TILES_LO 2
+#endif
+#ifndef JABAS_CHUNK_TILES_HI
+#define JABAS_CHUNK_TILES_HI 4
+#endif
+constexpr int kBlock = JABAS_BLOCK;         // default threads per workgroup (256 = 4 wave64)
+static_assert(kBlock % 64 == 0 && kBlock >= 64 && kBlock <= 1024, "whole waves");
+static_assert(JABAS_BLOCK_SGD % 64 == 0 && JABAS_BLOCK_SGD >= 64 && JABAS_BLOCK_SGD <= 1024, "whole waves");
 constexpr int kWaves = kBlock / 64;
-constexpr int kMinChunkTiles = 2;           // a chunk = the tiles one workgroup processes: 2 or 4
-constexpr int kMaxChunkTiles = 4;
-// Small chunks keep the streamed window of every buffer compact (higher HBM rate) and cut
-// the ramp-up / drain of a launch; kernels with many gradient streams and statistics have
-// low occupancy and a long prologue, and do better with twice the work per workgroup.
-__host__ __device__ constexpr int pick_chunk_tiles(int K) { return K > 4 ? kMaxChunkTiles : kMinChunkTiles; }
+constexpr int kMinChunkTiles = JABAS_CHUNK_TILES_LO;
+constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW. The shape depends on what a plan is encoded for (K, gradient
+// dtype, optimizer class), never on per-step flags, so one chunk table serves every step.
+__host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class) {
+    return (opt_class == 1 && K <= 4 && grad_dtype == JABAS_F32) ? JABAS_BLOCK_SGD : kBlock;
+}
+__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int /*opt_class*/) {
+    return K > 4 ? kMaxChunkTiles : kMinChunkTiles;
+}
+// Fewest elements any chunk covers, over all shapes: sizes workspaces that must fit every launch.
+constexpr int kMinChunkElems = (JABAS_BLOCK_SGD < JABAS_BLOCK ? JABAS_BLOCK_SGD : JABAS_BLOCK) * 4 * JABAS_CHUNK_TILES_LO;
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
 // Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer
 // (bf16 gradients are then read as 8-byte vectors, which keeps every access of a wave
 // contiguous).
 __host__ __device__ constexpr int ept_of(int /*grad_dtype*/) { return 4; }
-__host__ __device__ constexpr int tile_elems(int grad_dtype) { return kBlock * ept_of(grad_dtype); }
+__host__ __device__ constexpr int tile_elems_of(int block) { return block * 4; }
 
 // A span as the kernels see it. Pointers are rebased downwards by `lo` elements so that
 // element index 0 of every buffer is 16-byte aligned; [lo, hi) is the live range.
@@ -80,7 +109,7 @@ struct KArgs {
     const float* grad_scale;                 // device scalar or NULL (clipping)
     uint32_t n_span;
     uint32_t n_chunks;
-    uint32_t chunk_tiles;                    // tiles per workgroup
+    uint32_t chunk_tiles;                    // tiles per workgroup (the kernel's own shape; checked on the host)
     uint32_t use_inline;                     // 1: the only span is `span0`, chunk b starts at tile b*chunk_tiles
     uint32_t half_mask;                      // bit k set: VSW k belongs to half B
     uint32_t pad0;

@@ -150,7 +150,9 @@ def test_plan_blob_too_small_and_garbage_header():
     spans = (L.JabasSpan * 1)(_span(4096))
     nbytes = lib.jabas_plan_bytes(spans, 1, 0, L.F32)
     blob = np.zeros(nbytes // 8 + 1, dtype=np.uint64)
-    assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, nbytes - 8) == L.ERR_PLAN
+    # jabas_plan_bytes is an upper bound over the launch shapes; the header and one span do not fit 128 bytes
+    assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, 128) == L.ERR_PLAN
+    assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, nbytes) == L.OK
     junk = np.zeros(64, dtype=np.uint64)
     assert lib.jabas_plan_chunks(junk.ctypes.data) == L.ERR_PLAN
     assert lib.jabas_plan_workspace_bytes(junk.ctypes.data) == 0
@@ -233,8 +235,8 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
     assert seen[("version", "jabas_sync")].startswith("0.")
     assert seen[("status0", "ok")] == ""
     assert seen[("encode", "0")] == ""
-    assert seen[("chunks", "8")] == ""                       # 5000 -> 3 chunks of 2 tiles, 9096 -> 5
-    assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * L.STATS_STRIDE * 8
+    assert seen[("chunks", "14")] == ""                      # SGD, K = 2, fp32: 1024 elements per chunk -> 5 + 9
+    assert int(next(n for (k, n) in seen if k == "workspace")) >= (14 + 2) * L.STATS_STRIDE * 8
     assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
 
 
@@ -269,3 +271,28 @@ def test_plan_encode_rejects_overlapping_written_buffers():
     s = span()
     s.param = s.grads[0]                                        # ignored without an optimizer
     assert _encode([s], opt=L.OPT_NONE)[0] == L.OK
+
+
+def test_launch_shape_follows_what_the_plan_is_encoded_for():
+    """SGD with fp32 gradients and K <= 4 runs 128-thread workgroups (1024 elements per chunk); every other
+    kernel family 256 threads x 2 tiles (K <= 4) or 4 tiles. A plan serves launches of its own optimizer
+    class only."""
+    lib = L.lib()
+    n = 10 * 4096
+    def chunks(K, dtype, opt, gs=4):
+        rc, blob, _ = _encode([_span(n, K=K, gs=gs, opt=True)], K=K, dtype=dtype, opt=opt)
+        assert rc == L.OK
+        return lib.jabas_plan_chunks(blob.ctypes.data), blob
+    assert chunks(2, L.F32, L.OPT_SGD)[0] == n // 1024
+    assert chunks(4, L.F32, L.OPT_SGD)[0] == n // 1024
+    assert chunks(5, L.F32, L.OPT_SGD)[0] == n // 4096
+    assert chunks(2, L.BF16, L.OPT_SGD, gs=2)[0] == n // 2048
+    assert chunks(2, L.F32, L.OPT_ADAM)[0] == n // 2048
+    assert chunks(2, L.F32, L.OPT_NONE)[0] == n // 2048
+    _, blob = chunks(2, L.F32, L.OPT_SGD)
+    args = L.JabasStepArgs()
+    args.K, args.grad_dtype, args.opt_kind = 2, L.F32, L.OPT_NONE
+    assert lib.jabas_sync_fused(blob.ctypes.data, 0x1000, C.byref(args), None, None, 0, None) == L.ERR_PLAN
+    args.opt_kind, args.n_groups = L.OPT_ADAM, 1
+    args.groups[0].step = 1
+    assert lib.jabas_sync_fused(blob.ctypes.data, 0x1000, C.byref(args), None, None, 0, None) == L.ERR_PLAN
