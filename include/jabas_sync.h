@@ -143,7 +143,11 @@ size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype);
  * chunk table, group bounds). jabas_plan_encode validates the spans and writes the
  * blob into host memory; the caller copies the same bytes to the device once and
  * passes both copies to jabas_sync_fused at every step. Pure host code: runs without
- * a GPU.
+ * a GPU. The chunk table is cut for the launch shape of (K, grad_dtype, optimizer
+ * class of opt_kind: none / SGD / Adam+AdamW), so a plan serves launches of exactly
+ * that K, dtype and class (statistics on or off, any step, any learning rate);
+ * anything else is JABAS_ERR_PLAN. jabas_plan_bytes is an upper bound over all
+ * launch shapes; the blob (device copy 16-byte aligned) may be larger than used.
  * Stands in for the per-tensor Python loops that walk buckets and parameters at every
  * step in the reference: jabas/train/trainer.py:327-337 (hook registration per local
  * model), examples/gnmt/seq2seq/train/shard_optimizer.py:40-73 (per-parameter loop
