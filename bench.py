@@ -32,10 +32,8 @@ ROTATE_TARGET_BYTES = 1.5e9   # minimum total working set per configuration
 
 # HBM bytes per launch of the fused kernel measured with rocprofv3 --pmc (FETCH_SIZE and
 # WRITE_SIZE runs, scaled by a copy kernel of known size; profiles/fused_kernel_hbm_traffic_pmc.md).
-MEASURED_TRAFFIC_BYTES = {
-    "vit_b16": 3818.2e6, "resnet50": 717.3e6, "faster_rcnn_r50_fpn": 1342.9e6, "gnmt": 7086.1e6,
-    "vit_l16": 13405.5e6,
-}
+MEASURED_TRAFFIC_BYTES = {"vit_b16": 3816.9e6, "resnet50": 718.9e6, "faster_rcnn_r50_fpn": 1345.5e6,
+                          "gnmt": 7083.6e6, "vit_l16": 13405.5e6}
 
 
 def algorithmic_bytes_per_elem(cfg):

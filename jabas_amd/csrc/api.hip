@@ -232,11 +232,13 @@ constexpr int kFinalizeBlock = 256;
 constexpr uint32_t kStripeRows = 512;        // chunk rows one workgroup sums in the striped launch
 constexpr uint32_t kMaxStripes = 32;
 constexpr uint32_t kSingleLaunchRows = 2560; // up to here one workgroup per span finishes in about 6 us
+template <int NS>
 __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
                                                                         uint32_t use_inline, uint32_t stripes,
-                                                                        uint32_t in_stripes, int ns, const double* in,
-                                                                        double* out) {
-    __shared__ double red[kFinalizeBlock / 64][kStatsStride];
+                                                                        uint32_t in_stripes, uint32_t out_stride,
+                                                                        const double* in, double* out) {
+    // input rows are compact (NS = 4 + K doubles each); output rows have out_stride slots, the unused ones 0
+    __shared__ double red[kFinalizeBlock / 64][NS];
     const uint32_t s = blockIdx.y, j = blockIdx.x, t = threadIdx.x;
     uint32_t c0, c1, o;
     if (stripes == 0) {
@@ -251,27 +253,48 @@ __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const ui
         c1 = c0 + per < b1 ? c0 + per : b1;
         o = s * stripes + j;
     }
-    double acc[kStatsStride];
+    double acc[NS];
 #pragma unroll
-    for (int i = 0; i < kStatsStride; ++i) acc[i] = 0.0;
+    for (int i = 0; i < NS; ++i) acc[i] = 0.0;
 #pragma unroll 2
     for (uint32_t c = c0 + t; c < c1; c += kFinalizeBlock) {
-        const double* row = in + static_cast<uint64_t>(c) * kStatsStride;
+        const double* row = in + static_cast<uint64_t>(c) * NS;
 #pragma unroll
-        for (int i = 0; i < kStatsStride; ++i) acc[i] += row[i];
+        for (int i = 0; i < NS; ++i) acc[i] += row[i];
     }
     const int lane = t & 63, wave = t >> 6;
 #pragma unroll
-    for (int i = 0; i < kStatsStride; ++i) {
+    for (int i = 0; i < NS; ++i) {
         const double v = wave_sum_to_lane63(acc[i]);
         if (lane == 63) red[wave][i] = v;
     }
     __syncthreads();
-    if (t < kStatsStride) {
-        double sum = red[0][t];
+    if (t < out_stride) {
+        double sum = 0.0;
+        if (t < NS) {
+            sum = red[0][t];
 #pragma unroll
-        for (int w = 1; w < kFinalizeBlock / 64; ++w) sum += red[w][t];
-        out[static_cast<uint64_t>(o) * kStatsStride + t] = t < static_cast<uint32_t>(ns) ? sum : 0.0;
+            for (int w = 1; w < kFinalizeBlock / 64; ++w) sum += red[w][t];
+        }
+        out[static_cast<uint64_t>(o) * out_stride + t] = sum;
+    }
+}
+
+template <int NS>
+void launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
+                     uint32_t out_stride, const double* in, double* out) {
+    hipLaunchKernelGGL(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
+                       a.use_inline, stripes, in_stripes, out_stride, in, out);
+}
+// One instantiation per row width 4 + K, K = 1..16.
+void finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
+              uint32_t out_stride, const double* in, double* out) {
+    switch (ns) {
+#define JABAS_FIN(n) case n: launch_finalize<n>(grid, stream, a, stripes, in_stripes, out_stride, in, out); break;
+        JABAS_FIN(5) JABAS_FIN(6) JABAS_FIN(7) JABAS_FIN(8) JABAS_FIN(9) JABAS_FIN(10) JABAS_FIN(11) JABAS_FIN(12)
+        JABAS_FIN(13) JABAS_FIN(14) JABAS_FIN(15) JABAS_FIN(16) JABAS_FIN(17) JABAS_FIN(18) JABAS_FIN(19) JABAS_FIN(20)
+#undef JABAS_FIN
+        default: break;
     }
 }
 
@@ -311,14 +334,11 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
         const uint32_t st = stripes_for(max_span_chunks);
         const int ns = 4 + s->K;
         if (st == 1) {
-            hipLaunchKernelGGL(finalize_stats_kernel, dim3(1, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
-                               a.n_chunks, a.use_inline, 1u, 0u, ns, a.partials, stats_out);
+            finalize(ns, dim3(1, a.n_span), stream, a, 1u, 0u, kStatsStride, a.partials, stats_out);
         } else {
-            double* level2 = a.partials + static_cast<uint64_t>(a.n_chunks) * kStatsStride;
-            hipLaunchKernelGGL(finalize_stats_kernel, dim3(st, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
-                               a.n_chunks, a.use_inline, st, 0u, ns, a.partials, level2);
-            hipLaunchKernelGGL(finalize_stats_kernel, dim3(1, a.n_span), dim3(kFinalizeBlock), 0, stream, a.chunk_prefix,
-                               a.n_chunks, a.use_inline, 0u, st, ns, level2, stats_out);
+            double* level2 = a.partials + static_cast<uint64_t>(a.n_chunks) * ns;
+            finalize(ns, dim3(st, a.n_span), stream, a, st, 0u, static_cast<uint32_t>(ns), a.partials, level2);
+            finalize(ns, dim3(1, a.n_span), stream, a, 0u, st, kStatsStride, level2, stats_out);
         }
         if (hipGetLastError() != hipSuccess) return JABAS_ERR_LAUNCH;
     }

@@ -353,7 +353,6 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
 #pragma unroll
     for (int i = 0; i < NS; ++i) buf[i][tid] = acc[i];
     __syncthreads();
-    static_assert(kStatsStride - NS <= BS, "one thread per unused slot");
 #pragma unroll
     for (int v0 = 0; v0 < NS; v0 += kPerPass) {      // K > 12 needs a second pass at 256 threads
         if (tid < (NS - v0) * kParts) {
@@ -368,7 +367,6 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
             if (part == 0) row[v] = s;
         }
     }
-    if (tid < kStatsStride - NS) row[NS + tid] = 0.0;          // unused slots of the row
 }
 
 template <int K, int DT, int OPT, bool STATS>
@@ -407,7 +405,7 @@ __global__ void __launch_bounds__(launch_block(K, DT, OPT)) fused_kernel(const K
         const uint32_t lt1 = c.tile0 + CT < tiles ? c.tile0 + CT : tiles;
         run_chunk<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
-    if constexpr (STATS) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * kStatsStride);
+    if constexpr (STATS) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * NS);   // compact rows of 4 + K
 }
 
 template <int K, int DT, int OPT, bool STATS>
