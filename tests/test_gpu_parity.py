@@ -513,3 +513,47 @@ def test_random_plans_match_the_oracle(gpu, seed):
             assert torch.count_nonzero(f.cpu()[~covered]) == 0
     if not in_place and (~covered).any():
         assert torch.count_nonzero(agg_d.cpu()[~covered]) == 0
+
+
+@pytest.mark.parametrize("seed", range(100, 112))
+def test_random_buckets_through_the_inline_path(gpu, seed):
+    """The same random cases, one jabas_sync_bucket call per span (span by value, bound table on the
+    device, first bound of each workgroup found by binary search)."""
+    from jabas_amd import sync, _lib as L
+    K, dtype, opt, sizes, gaps, half_id, batches, in_place, n_fan, bounds = _random_case(seed - 100 if seed % 2 else seed)
+    rng = np.random.RandomState(seed)
+    sizes = [s for s in sizes if s > 0][:8] or [777]
+    bounds = [b for s, b in zip(sizes, [b for b in bounds if b] + [()] * len(sizes))]
+    print(f"seed {seed}: K={K} {dtype} opt={opt and opt['kind']} sizes={sizes} halves={half_id}", flush=True)
+    kind = sync.opt_kind(opt)
+    adam = kind in (L.OPT_ADAM, L.OPT_ADAMW)
+    for si, n in enumerate(sizes):
+        skew = int(rng.randint(0, 4))
+        b = tuple((st, g) for st, g in bounds[si] if st < n) if opt else ()
+        if opt and (not b or b[0][0] != 0):
+            b = ((0, 1),) + tuple(x for x in b if x[0] > 0)
+        hg = _host_grads(K, n, 500 + 13 * seed + si, std=5e-4, dtype=dtype)
+        p_h, s1_h, s2_h = _host_state(n, 60 + seed + si), torch.zeros(n), torch.zeros(n)
+        dg = [_dev(t, gpu, skew) for t in hg]
+        agg_d = _dev(torch.zeros(n), gpu, skew)
+        p_d, s1_d, s2_d = _dev(p_h, gpu, skew), _dev(s1_h, gpu, skew), _dev(s2_h, gpu, skew)
+        span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d if opt else None, state1=s1_d if opt else None,
+                             state2=s2_d if adam else None, bounds=b)
+        call = sync.BucketCall(span)
+        for step in (1, 2):
+            args = sync.make_step_args(batches, dtype, stats=True, opt=opt, step=step, first_step=(step == 1),
+                                       half_id=half_id)
+            row = call.run(args)
+            torch.cuda.synchronize()
+            agg_h, rows_h = O.sync_step(hg, batches, [(0, n, b)], opt, p_h, s1_h, s2_h if adam else None, step=step,
+                                        first_step=(step == 1), want_stats=True, half_id=half_id)
+            assert torch.equal(_bits(agg_d), _bits(agg_h)), (si, step)
+            rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+            got, want = row.cpu()[:4 + K], rows_h[0][:4 + K]
+            scale = want[1:3].abs().max().clamp_min(1e-300)
+            assert bool(((got - want).abs() <= rtol * want.abs() + 1e-9 * scale).all()), (si, step)
+            if opt:
+                assert torch.equal(_bits(p_d), _bits(p_h)), (si, step)
+                assert torch.equal(_bits(s1_d), _bits(s1_h)), (si, step)
+                if adam:
+                    assert torch.equal(_bits(s2_d), _bits(s2_h)), (si, step)
