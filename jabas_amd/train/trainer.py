@@ -4,8 +4,14 @@
 reaches the path (jabas/train/trainer.py: ``prepare_stream_parallel`` :82-86,
 ``prepare_weight_sync_method`` :88-98, ``compute`` :171-174, ``step`` :176-197,
 ``_compute_cosine_similarity`` :470-483, ``_adjust_adaptive_lr`` :693-700; attributes
-``local_models``, ``main_model``, ``model_streams``, ``num_models``, ``similarity_state``,
-``cos_placeholder``): K model replicas on K HIP streams, one sync step per iteration.
+``local_models``, ``main_model``, ``local_optimizers``, ``main_optimizer``, ``local_schedulers``,
+``model_streams``, ``num_models``, ``sync_step``, ``similarity_state``, ``cos_placeholder``):
+K model replicas on K HIP streams, one sync step per iteration. The optimizer object the
+caller hands to ``prepare_weight_sync_method`` stays the place where hyperparameters live
+(``main_optimizer.param_groups[i]['lr']`` is read at every step, so the reference's learning-rate
+policies and torch LR schedulers work unchanged) and where the state is visible
+(``main_optimizer.state[p]`` holds views of the state arenas, so ``state_dict()`` checkpoints it);
+its own ``step()`` is never called: the fused launch does the update.
 It is not the reference's trainer: data loading, the configuration solver, elastic
 restarts and the cross-GPU all-reduce are outside this build.
 
@@ -57,9 +63,45 @@ def tag_parameter_indices(model):
     return model
 
 
+def opt_from_torch_optimizer(optimizer):
+    """Hyperparameter dictionary (the form ``sync.make_step_args`` takes) of a torch.optim.SGD / Adam /
+    AdamW or a jabas_amd.optim.Shard* object. One momentum / betas / eps for all groups, as the
+    kernel takes them per launch; learning rate and weight decay per group."""
+    from ..optim import ShardSGD, ShardAdam, ShardAdamW
+    groups = optimizer.param_groups
+    if not groups:
+        raise ValueError("optimizer has no parameter groups")
+    g0 = groups[0]
+
+    def same(key):
+        vals = [g[key] for g in groups]
+        if any(v != vals[0] for v in vals[1:]):
+            raise ValueError(f"parameter groups differ in {key!r}: one value per launch is supported")
+        return vals[0]
+
+    if isinstance(optimizer, (torch.optim.SGD, ShardSGD)):
+        opt = dict(kind="sgd", momentum=float(same("momentum")), dampening=float(same("dampening")),
+                   nesterov=bool(same("nesterov")))
+        if g0.get("maximize", False):
+            raise ValueError("maximize=True is not supported")
+    elif isinstance(optimizer, (torch.optim.AdamW, ShardAdamW, torch.optim.Adam, ShardAdam)):
+        adamw = isinstance(optimizer, (torch.optim.AdamW, ShardAdamW))
+        if g0.get("amsgrad", False) or g0.get("maximize", False):
+            raise ValueError("amsgrad / maximize are not supported")
+        b1, b2 = same("betas")
+        opt = dict(kind="adamw" if adamw else "adam", betas=(float(b1), float(b2)), eps=float(same("eps")))
+    else:
+        raise TypeError(f"unsupported optimizer type {type(optimizer).__name__}: SGD, Adam, AdamW or their "
+                        "Shard counterparts")
+    opt["groups"] = [dict(lr=float(g["lr"]), weight_decay=float(g.get("weight_decay", 0.0))) for g in groups]
+    return opt
+
+
 class VSWSyncTrainer:
-    def __init__(self, gpu, local_batch_sizes, opt, interval=100, grad_dtype=torch.float32,
+    def __init__(self, gpu, local_batch_sizes, opt=None, interval=100, grad_dtype=torch.float32,
                  param_groups_func=None, similarity_target=None, controller=None, clip_norm=None):
+        """opt: hyperparameter dictionary, or None when an optimizer object follows through
+        ``prepare_weight_sync_method`` (the reference's order of calls)."""
         self.gpu = torch.device("cuda", gpu) if isinstance(gpu, int) else torch.device(gpu)
         self.local_batch_sizes = tuple(local_batch_sizes)
         self.num_models = len(self.local_batch_sizes)
@@ -72,20 +114,61 @@ class VSWSyncTrainer:
         self.clip_norm = clip_norm
         self.global_lr_modifier = 1.0
         self.local_models, self.model_streams = [], []
-        self.main_model = None
+        self.local_optimizers, self.local_schedulers = [], []
+        self.main_model = self.main_optimizer = None
+        self.sync_step = 0
         self.engine = None
+        self._step_tensor = torch.zeros((), dtype=torch.float32)       # Adam's state['step'], shared by all parameters
         self.cos_placeholder = None
         self.grad_placeholders = [[], []]
         workers = self.num_models if self.num_models % 2 == 0 else self.num_models + 1
         self.similarity_state = GradientSimilarityState(None, workers, None, self.grad_placeholders[0], interval)
 
     # ---------------------------------------------------------------------- set-up
-    def prepare_stream_parallel(self, model, criterion):
-        model = model.to(self.gpu)
+    def prepare_stream_parallel(self, model, criterion, **kwargs):
+        """Counterpart of jabas/train/trainer.py:82-86. With a hyperparameter dictionary given to the
+        constructor the arenas are built here; otherwise by ``prepare_weight_sync_method``."""
+        self._model0 = model.to(self.gpu)
+        self.main_model = self._model0
+        self.criterion = criterion
+        if self.opt is not None:
+            self._build(None)
+
+    def prepare_weight_sync_method(self, optimizer, scheduler=None, param_groups_func=None):
+        """Counterpart of jabas/train/trainer.py:88-98: takes the optimizer the caller built over
+        ``main_model``'s parameters (torch.optim.SGD / Adam / AdamW or ShardSGD / ShardAdam / ShardAdamW,
+        examples/resnet50/main.py:351-363) and an optional LR scheduler that is stepped once per sync
+        step. Parameter groups of the optimizer become the kernel's parameter groups."""
+        if self.main_model is None:
+            raise RuntimeError("call prepare_stream_parallel(model, criterion) first")
+        if self.engine is not None:
+            raise RuntimeError("the weight-sync method is already prepared")
+        if param_groups_func is not None:
+            self.param_groups_func = param_groups_func
+        self.opt = opt_from_torch_optimizer(optimizer)
+        self.main_optimizer = optimizer
+        self.local_optimizers = [optimizer]          # replicas hold no optimizer state of their own here
+        self.local_schedulers = [scheduler] if scheduler is not None else []
+        try:
+            self._build(optimizer)
+        except Exception:                            # leave the trainer as it was: the caller may try again
+            self.opt = self.main_optimizer = self.engine = None
+            self.local_optimizers, self.local_schedulers = [], []
+            raise
+
+    def _build(self, optimizer):
+        model = self._model0
         names = [n for n, _ in model.named_parameters()]
         params = [p for _, p in model.named_parameters()]
         group_of = {}
-        if self.param_groups_func is not None:
+        if optimizer is not None:
+            for gi, group in enumerate(optimizer.param_groups):
+                for p in group["params"]:
+                    group_of[id(p)] = gi
+            missing = [n for n, p in zip(names, params) if p.requires_grad and id(p) not in group_of]
+            if missing:
+                raise ValueError(f"parameters without an optimizer group: {missing[:4]}")
+        elif self.param_groups_func is not None:
             for gi, group in enumerate(self.param_groups_func(model)):
                 for p in group["params"]:
                     group_of[id(p)] = gi
@@ -94,13 +177,37 @@ class VSWSyncTrainer:
                                   device=self.gpu, n_fanout=max(1, self.num_models - 1))
         if self.num_models == 1:
             self.engine.reconfigure(self.local_batch_sizes)       # keeps the fan-out slot for later replicas
-        self.criterion = criterion
         self.local_models = [model] + [copy.deepcopy(model) for _ in range(self.num_models - 1)]
         self.main_model = self.local_models[0]
         self.model_streams = [torch.cuda.Stream(self.gpu) for _ in range(self.num_models)]
         for k, m in enumerate(self.local_models):
             self._bind_model(k, m, copy_weights=True)
+        if optimizer is not None:
+            self._expose_state(optimizer)
         torch.cuda.synchronize(self.gpu)
+
+    def _expose_state(self, optimizer):
+        """optimizer.state[p] = views of the state arenas under the names torch's optimizers use, so that
+        ``state_dict()`` of the caller's optimizer checkpoints what the fused launch maintains."""
+        eng = self.engine
+        sgd = self.opt["kind"] == "sgd"
+        for i, p in enumerate(self.main_model.parameters()):
+            st = optimizer.state[p]
+            if sgd:
+                if eng.state1 is not None:
+                    st["momentum_buffer"] = eng._view(eng.state1, i).view(p.shape)
+            else:
+                st["step"] = self._step_tensor
+                st["exp_avg"] = eng._view(eng.state1, i).view(p.shape)
+                st["exp_avg_sq"] = eng._view(eng.state2, i).view(p.shape)
+
+    def _refresh_hyperparameters(self):
+        """Learning rate and weight decay as the caller's optimizer object holds them now."""
+        if self.main_optimizer is None:
+            return
+        for mine, theirs in zip(self.opt["groups"], self.main_optimizer.param_groups):
+            mine["lr"] = float(theirs["lr"])
+            mine["weight_decay"] = float(theirs.get("weight_decay", 0.0))
 
     def _bind_model(self, k, m, copy_weights):
         """Points replica k's parameters and gradients at its arenas."""
@@ -160,7 +267,14 @@ class VSWSyncTrainer:
             cur.wait_stream(s)
         st = self.similarity_state
         want = st.step % st.interval == 0
+        self._refresh_hyperparameters()
         rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm)
+        self.sync_step += 1
+        self._step_tensor.fill_(float(self.engine.step_count))
+        if self.local_schedulers:
+            self.main_optimizer._opt_called = True      # what torch's schedulers look at to see that an update preceded them
+            for sched in self.local_schedulers:
+                sched.step()
         if want:
             self._compute_cosine_similarity(rows)
         for k in range(self.num_models):

@@ -233,3 +233,85 @@ def test_trainer_adds_and_removes_workers_from_the_similarity(gpu):
         trainer.compute(data)
         trainer.step()
     assert trainer.num_models == 4 and len(trainer.model_streams) == 4 and trainer.engine.K == 4
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw", "shard_adam"])
+def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
+    """The reference's order of calls (examples/resnet50/main.py:351-366, examples/vit/main.py:425-478):
+    prepare_stream_parallel, an optimizer built over trainer.main_model, prepare_weight_sync_method
+    (optimizer, scheduler), then learning rates driven through trainer.main_optimizer.param_groups."""
+    from jabas_amd.train import VSWSyncTrainer
+    from jabas_amd import optim
+    batches = (5, 3)
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, interval=2)
+    trainer.prepare_stream_parallel(_mlp(11), crit)
+    ref_model = _mlp(11).to(gpu)
+
+    def build(model, shard):
+        groups = _groups(model)
+        if kind == "sgd":
+            return torch.optim.SGD(groups, lr=0.05, momentum=0.9, foreach=False)
+        if kind == "adamw":
+            return torch.optim.AdamW(groups, lr=1e-3, foreach=False)
+        return (optim.ShardAdam if shard else torch.optim.Adam)(groups, lr=2e-3, **({} if shard else {"foreach": False}))
+
+    mine, ref_opt = build(trainer.main_model, True), build(ref_model, False)
+    lam = lambda it: 1.0 / (1.0 + 0.5 * it)
+    sched = torch.optim.lr_scheduler.LambdaLR(mine, lam) if kind != "sgd" else None
+    ref_sched = torch.optim.lr_scheduler.LambdaLR(ref_opt, lam) if kind != "sgd" else None
+    trainer.prepare_weight_sync_method(mine, sched, _groups)
+    assert trainer.main_optimizer is mine and trainer.local_optimizers == [mine]
+    w, _, _ = O.batch_weights(batches)
+    for step in range(1, 6):
+        if kind == "sgd":                                   # the reference's lr policy writes param_groups directly
+            for opt_ in (trainer.main_optimizer, ref_opt):
+                for g in opt_.param_groups:
+                    g["lr"] = 0.05 * (0.8 ** step)
+        gen = torch.Generator().manual_seed(70 + step)
+        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        trainer.compute(data)
+        per_vsw = []
+        for x, y in data:
+            ref_model.zero_grad(set_to_none=True)
+            crit(ref_model(x), y).backward()
+            per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(per_vsw[0][i], w[0]), torch.mul(per_vsw[1][i], w[1]))
+        ref_opt.step()
+        if ref_sched is not None:
+            ref_sched.step()
+        trainer.step()
+        torch.cuda.synchronize()
+        assert trainer.sync_step == step
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), f"{kind} step {step}"
+        if ref_sched is not None:
+            assert mine.param_groups[0]["lr"] == pytest.approx(ref_opt.param_groups[0]["lr"], rel=1e-12)
+    # the caller's optimizer object shows the state the fused launch maintains
+    sd = mine.state_dict()
+    assert len(sd["state"]) == len(list(trainer.main_model.parameters()))
+    key = "momentum_buffer" if kind == "sgd" else "exp_avg"
+    for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+        assert _close(mine.state[p][key], ref_opt.state[rp][key], 1e-6, 1e-8)
+        if kind != "sgd":
+            assert float(mine.state[p]["step"]) == 5.0
+            assert _close(mine.state[p]["exp_avg_sq"], ref_opt.state[rp]["exp_avg_sq"], 1e-6, 1e-12)
+
+
+def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
+    from jabas_amd.train import VSWSyncTrainer
+    trainer = VSWSyncTrainer(gpu, (2, 2))
+    with pytest.raises(RuntimeError):
+        trainer.prepare_weight_sync_method(None)
+    trainer.prepare_stream_parallel(_mlp(1), torch.nn.MSELoss())
+    with pytest.raises(TypeError):
+        trainer.prepare_weight_sync_method(torch.optim.RMSprop(trainer.main_model.parameters(), lr=0.1))
+    with pytest.raises(ValueError):
+        trainer.prepare_weight_sync_method(torch.optim.Adam(trainer.main_model.parameters(), lr=0.1, amsgrad=True))
+    groups = _groups(trainer.main_model)
+    groups[0]["momentum"] = 0.5
+    with pytest.raises(ValueError):
+        trainer.prepare_weight_sync_method(torch.optim.SGD(groups, lr=0.1, momentum=0.9))
+    with pytest.raises(ValueError):                         # a parameter outside every group
+        trainer.prepare_weight_sync_method(torch.optim.SGD(list(trainer.main_model.parameters())[:2], lr=0.1))
