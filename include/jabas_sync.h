@@ -143,7 +143,7 @@ size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype);
  * chunk table, group bounds). jabas_plan_encode validates the spans and writes the
  * blob into host memory; the caller copies the same bytes to the device once and
  * passes both copies to jabas_sync_fused at every step. Pure host code: runs without
- * a GPU. The chunk table is cut for the launch shape of (K, grad_dtype, optimizer
+ * a GPU. The chunk tables are cut for the launch shapes of (K, grad_dtype, optimizer
  * class of opt_kind: none / SGD / Adam+AdamW), so a plan serves launches of exactly
  * that K, dtype and class (statistics on or off, any step, any learning rate);
  * anything else is JABAS_ERR_PLAN. jabas_plan_bytes is an upper bound over all
@@ -158,9 +158,10 @@ int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span,
                       const JabasBound* bounds, uint32_t n_bounds,
                       int32_t K, int32_t grad_dtype, int32_t opt_kind,
                       void* host_blob, size_t blob_bytes);
-/* Number of workgroups (chunks) one launch of the plan uses; negative JabasStatus on a
- * malformed blob. */
-int64_t jabas_plan_chunks(const void* host_blob);
+/* Number of workgroups (chunks) one launch of the plan uses, without (stats == 0) or with
+ * statistics: the two kinds of launch may run different workgroup shapes, the plan holds a
+ * chunk table for each. Negative JabasStatus on a malformed blob. */
+int64_t jabas_plan_chunks(const void* host_blob, int32_t stats);
 /* Bytes of device workspace jabas_sync_fused needs for this plan when statistics are
  * requested (0 on a malformed blob). */
 size_t jabas_plan_workspace_bytes(const void* host_blob);

@@ -81,7 +81,7 @@ SIGNATURES = {
     "jabas_plan_bytes": (C.c_size_t, [C.POINTER(JabasSpan), C.c_uint32, C.c_uint32, C.c_int32]),
     "jabas_plan_encode": (C.c_int, [C.POINTER(JabasSpan), C.c_uint32, C.POINTER(JabasBound), C.c_uint32,
                                     C.c_int32, C.c_int32, C.c_int32, C.c_void_p, C.c_size_t]),
-    "jabas_plan_chunks": (C.c_int64, [C.c_void_p]),
+    "jabas_plan_chunks": (C.c_int64, [C.c_void_p, C.c_int32]),
     "jabas_plan_workspace_bytes": (C.c_size_t, [C.c_void_p]),
     "jabas_sync_fused": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(JabasStepArgs), C.c_void_p,
                                    C.c_void_p, C.c_size_t, C.c_void_p]),

@@ -17,22 +17,29 @@ namespace {
 
 constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 5;
+constexpr uint32_t kPlanVersion = 6;
 
+// A plan holds one chunk table per launch shape: index 0 for launches without statistics, 1 with.
+// When both shapes are the same the two entries describe the same table.
+struct PlanShape {
+    uint32_t block;           // threads per workgroup the chunk table was cut for
+    uint32_t chunk_tiles;     // tiles per workgroup
+    uint32_t n_chunks;        // workgroups of one launch
+    uint32_t max_span_chunks; // chunks of the largest span (sizes the striped finalize)
+    uint64_t off_prefix, off_chunks;
+};
 struct PlanHeader {
     uint32_t magic, version;
-    uint32_t n_span, n_bounds, n_chunks;
+    uint32_t n_span, n_bounds;
     int32_t K, grad_dtype, opt_kind;
     uint32_t max_group;       // largest group index any bound names
     uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
-    uint32_t chunk_tiles;     // tiles per workgroup the chunk table was cut for
-    uint32_t max_span_chunks; // chunks of the largest span (sizes the striped finalize)
-    uint32_t block;           // threads per workgroup the chunk table was cut for
     uint32_t pad;
-    uint64_t off_spans, off_prefix, off_chunks, off_bounds, total_bytes;
+    PlanShape shape[2];
+    uint64_t off_spans, off_bounds, total_bytes;
 };
-static_assert(sizeof(PlanHeader) == 96, "plan header layout");
-constexpr size_t kHeaderBytes = 96;
+static_assert(sizeof(PlanShape) == 32 && sizeof(PlanHeader) == 128, "plan header layout");
+constexpr size_t kHeaderBytes = 128;
 static_assert(kHeaderBytes >= sizeof(PlanHeader) && kHeaderBytes % 16 == 0, "plan header slot");
 
 inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
@@ -384,18 +391,20 @@ uint64_t plan_chunks(const JabasSpan* spans, uint32_t n_span, int grad_dtype, in
     for (uint32_t i = 0; i < n_span; ++i) n += chunks_of_tiles(span_tiles(spans[i], grad_dtype, block), ct);
     return n;
 }
-size_t plan_bytes_for(uint32_t n_span, uint32_t n_bounds, uint64_t n_chunks) {
+size_t table_bytes(uint32_t n_span, uint64_t n_chunks) {
+    return align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t)) + align16(static_cast<size_t>(n_chunks) * sizeof(ChunkDesc));
+}
+size_t plan_fixed_bytes(uint32_t n_span, uint32_t n_bounds) {
     return kHeaderBytes + align16(static_cast<size_t>(n_span) * sizeof(SpanDev)) +
-           align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t)) +
-           align16(static_cast<size_t>(n_chunks) * sizeof(ChunkDesc)) +
            align16(static_cast<size_t>(n_bounds) * sizeof(BoundDev));
 }
 }  // namespace
 
 JABAS_API size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds, int32_t grad_dtype) {
     if (!spans || (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16)) return 0;
-    // K and the optimizer are not known here: size for the launch shape with the smallest chunks
-    return plan_bytes_for(n_span, n_bounds, plan_chunks(spans, n_span, grad_dtype, kMinChunkElems / 4, 1));
+    // K and the optimizer are not known here: two chunk tables of the launch shape with the smallest chunks
+    return plan_fixed_bytes(n_span, n_bounds) +
+           2 * table_bytes(n_span, plan_chunks(spans, n_span, grad_dtype, kMinChunkElems / 4, 1));
 }
 
 JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
@@ -410,84 +419,109 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     if (opt_class_of(opt_kind) < 0) return JABAS_ERR_OPT;
     for (uint32_t i = 0; i < n_span; ++i)
         if (spans[i].numel && !spans[i].grads[0]) return JABAS_ERR_NULL;
-    const int block = launch_block(K, grad_dtype, opt_class_of(opt_kind));
-    const uint32_t ct = launch_chunk_tiles(K, grad_dtype, opt_class_of(opt_kind));
-    const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype, block, ct);
-    if (n_chunks > 0x7fffffffull) return JABAS_ERR_SIZE;
-    const size_t need = plan_bytes_for(n_span, n_bounds, n_chunks);
+    const int oc = opt_class_of(opt_kind);
+    PlanHeader h;
+    memset(&h, 0, sizeof(h));
+    size_t need = plan_fixed_bytes(n_span, n_bounds);
+    h.off_spans = kHeaderBytes;
+    h.off_bounds = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
+    size_t cursor = need;
+    for (int v = 0; v < 2; ++v) {
+        PlanShape& ps = h.shape[v];
+        ps.block = static_cast<uint32_t>(launch_block(K, grad_dtype, oc, v != 0));
+        ps.chunk_tiles = static_cast<uint32_t>(launch_chunk_tiles(K, grad_dtype, oc, v != 0));
+        if (v == 1 && ps.block == h.shape[0].block && ps.chunk_tiles == h.shape[0].chunk_tiles) {
+            ps = h.shape[0];                     // same shape: one table serves both kinds of launch
+            break;
+        }
+        const uint64_t n_chunks = plan_chunks(spans, n_span, grad_dtype, static_cast<int>(ps.block), ps.chunk_tiles);
+        if (n_chunks > 0x7fffffffull) return JABAS_ERR_SIZE;
+        ps.n_chunks = static_cast<uint32_t>(n_chunks);
+        ps.off_prefix = cursor;
+        ps.off_chunks = cursor + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
+        cursor += table_bytes(n_span, n_chunks);
+    }
+    need = cursor;
     if (blob_bytes < need) return JABAS_ERR_PLAN;
     if (reinterpret_cast<uintptr_t>(host_blob) % 8) return JABAS_ERR_ALIGN;
 
     char* base = static_cast<char*>(host_blob);
     memset(base, 0, need);
-    PlanHeader h;
-    memset(&h, 0, sizeof(h));
     h.magic = kPlanMagic;
     h.version = kPlanVersion;
     h.n_span = n_span;
     h.n_bounds = n_bounds;
-    h.n_chunks = static_cast<uint32_t>(n_chunks);
     h.K = K;
     h.grad_dtype = grad_dtype;
     h.opt_kind = opt_kind;
-    h.chunk_tiles = ct;
-    h.block = static_cast<uint32_t>(block);
-    h.off_spans = kHeaderBytes;
-    h.off_prefix = h.off_spans + align16(static_cast<size_t>(n_span) * sizeof(SpanDev));
-    h.off_chunks = h.off_prefix + align16((static_cast<size_t>(n_span) + 1) * sizeof(uint32_t));
-    h.off_bounds = h.off_chunks + align16(static_cast<size_t>(n_chunks) * sizeof(ChunkDesc));
     h.total_bytes = need;
     h.all_have_s1 = 1;
 
     SpanDev* sd = reinterpret_cast<SpanDev*>(base + h.off_spans);
-    uint32_t* prefix = reinterpret_cast<uint32_t*>(base + h.off_prefix);
-    ChunkDesc* cd = reinterpret_cast<ChunkDesc*>(base + h.off_chunks);
-    const uint64_t te = tile_elems_of(block);
-    uint32_t c = 0;
     for (uint32_t i = 0; i < n_span; ++i) {
         uint32_t tiles = 0;
-        int rc = encode_span(spans[i], K, grad_dtype, opt_kind, block, &sd[i], &tiles);
+        int rc = encode_span(spans[i], K, grad_dtype, opt_kind, static_cast<int>(h.shape[0].block), &sd[i], &tiles);
         if (rc != JABAS_OK) return rc;
         rc = check_bounds_host(spans[i], bounds, n_bounds, &h.max_group);
         if (rc != JABAS_OK) return rc;
         if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
-        prefix[i] = c;
-        const uint32_t span_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, ct));
-        if (span_chunks > h.max_span_chunks) h.max_span_chunks = span_chunks;
-        uint32_t j = 0;
-        for (uint32_t t0 = 0; t0 < tiles; t0 += ct, ++c) {
-            cd[c].span = i;
-            cd[c].tile0 = t0;
-            if (spans[i].bound_count) {       // bound entry covering the chunk's first live element
-                const uint64_t e0 = static_cast<uint64_t>(t0) * te;
-                const uint64_t rel = (e0 > sd[i].lo ? e0 : sd[i].lo) - sd[i].lo;
-                const JabasBound* b = bounds + spans[i].bound_begin;
-                while (j + 1 < spans[i].bound_count && b[j + 1].start <= rel) ++j;
-            }
-            cd[c].bound0 = j;
-        }
     }
-    prefix[n_span] = c;
-    if (c != h.n_chunks) return JABAS_ERR_PLAN;
+    const int n_tables = (h.shape[1].off_prefix == h.shape[0].off_prefix) ? 1 : 2;
+    for (int v = 0; v < n_tables; ++v) {
+        PlanShape& ps = h.shape[v];
+        uint32_t* prefix = reinterpret_cast<uint32_t*>(base + ps.off_prefix);
+        ChunkDesc* cd = reinterpret_cast<ChunkDesc*>(base + ps.off_chunks);
+        const uint64_t te = tile_elems_of(static_cast<int>(ps.block));
+        const uint32_t ct = ps.chunk_tiles;
+        uint32_t c = 0;
+        for (uint32_t i = 0; i < n_span; ++i) {
+            const uint64_t tiles64 = spans[i].numel ? (sd[i].hi + te - 1) / te : 0;
+            if (tiles64 > 0x7fffffffull) return JABAS_ERR_SIZE;
+            const uint32_t tiles = static_cast<uint32_t>(tiles64);
+            prefix[i] = c;
+            const uint32_t span_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, ct));
+            if (span_chunks > ps.max_span_chunks) ps.max_span_chunks = span_chunks;
+            uint32_t j = 0;
+            for (uint32_t t0 = 0; t0 < tiles; t0 += ct, ++c) {
+                cd[c].span = i;
+                cd[c].tile0 = t0;
+                if (spans[i].bound_count) {       // bound entry covering the chunk's first live element
+                    const uint64_t e0 = static_cast<uint64_t>(t0) * te;
+                    const uint64_t rel = (e0 > sd[i].lo ? e0 : sd[i].lo) - sd[i].lo;
+                    const JabasBound* b = bounds + spans[i].bound_begin;
+                    while (j + 1 < spans[i].bound_count && b[j + 1].start <= rel) ++j;
+                }
+                cd[c].bound0 = j;
+            }
+        }
+        prefix[n_span] = c;
+        if (c != ps.n_chunks) return JABAS_ERR_PLAN;
+    }
+    if (n_tables == 1) h.shape[1] = h.shape[0];
     if (n_bounds) memcpy(base + h.off_bounds, bounds, static_cast<size_t>(n_bounds) * sizeof(JabasBound));
     memcpy(base, &h, sizeof(h));
     return JABAS_OK;
 }
 
-JABAS_API int64_t jabas_plan_chunks(const void* host_blob) {
+namespace {
+bool read_plan_header(const void* host_blob, PlanHeader* h) {
+    memcpy(h, host_blob, sizeof(*h));
+    return h->magic == kPlanMagic && h->version == kPlanVersion;
+}
+}  // namespace
+
+JABAS_API int64_t jabas_plan_chunks(const void* host_blob, int32_t stats) {
     if (!host_blob) return JABAS_ERR_NULL;
     PlanHeader h;
-    memcpy(&h, host_blob, sizeof(h));
-    if (h.magic != kPlanMagic || h.version != kPlanVersion) return JABAS_ERR_PLAN;
-    return h.n_chunks;
+    if (!read_plan_header(host_blob, &h)) return JABAS_ERR_PLAN;
+    return h.shape[stats ? 1 : 0].n_chunks;
 }
 
 JABAS_API size_t jabas_plan_workspace_bytes(const void* host_blob) {
-    const int64_t n = jabas_plan_chunks(host_blob);
-    if (n < 0) return 0;
+    if (!host_blob) return 0;
     PlanHeader h;
-    memcpy(&h, host_blob, sizeof(h));
-    return workspace_rows(static_cast<uint64_t>(n), h.n_span) * kStatsStride * sizeof(double);
+    if (!read_plan_header(host_blob, &h)) return 0;
+    return workspace_rows(h.shape[1].n_chunks, h.n_span) * kStatsStride * sizeof(double);
 }
 
 JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, const JabasStepArgs* args,
@@ -503,11 +537,13 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     if (rc != JABAS_OK) return rc;
     if (args->K != h.K || args->grad_dtype != h.grad_dtype) return JABAS_ERR_PLAN;
     const int oc = opt_class_of(args->opt_kind);
-    // the chunk table is cut for the launch shape of (K, dtype, optimizer class), and the state pointers
+    // the chunk tables are cut for the launch shapes of (K, dtype, optimizer class), and the state pointers
     // were validated for that class only
     if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;
-    if (h.block != static_cast<uint32_t>(launch_block(h.K, h.grad_dtype, oc)) ||
-        h.chunk_tiles != static_cast<uint32_t>(launch_chunk_tiles(h.K, h.grad_dtype, oc)))
+    const bool stats = args->stats != 0;
+    const PlanShape& ps = h.shape[stats ? 1 : 0];
+    if (ps.block != static_cast<uint32_t>(launch_block(h.K, h.grad_dtype, oc, stats)) ||
+        ps.chunk_tiles != static_cast<uint32_t>(launch_chunk_tiles(h.K, h.grad_dtype, oc, stats)))
         return JABAS_ERR_PLAN;
     if (oc != 0) {
         if (h.max_group >= static_cast<uint32_t>(args->n_groups)) return JABAS_ERR_GROUP;
@@ -515,14 +551,14 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     }
     const char* dev = static_cast<const char*>(plan_dev);
     a.spans = reinterpret_cast<const SpanDev*>(dev + h.off_spans);
-    a.chunk_prefix = reinterpret_cast<const uint32_t*>(dev + h.off_prefix);
-    a.chunks = reinterpret_cast<const ChunkDesc*>(dev + h.off_chunks);
+    a.chunk_prefix = reinterpret_cast<const uint32_t*>(dev + ps.off_prefix);
+    a.chunks = reinterpret_cast<const ChunkDesc*>(dev + ps.off_chunks);
     a.bounds = h.n_bounds ? reinterpret_cast<const BoundDev*>(dev + h.off_bounds) : nullptr;
     a.n_span = h.n_span;
-    a.n_chunks = h.n_chunks;
-    a.chunk_tiles = h.chunk_tiles;
+    a.n_chunks = ps.n_chunks;
+    a.chunk_tiles = ps.chunk_tiles;
     a.use_inline = 0;
-    return run_fused(a, args, h.max_span_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+    return run_fused(a, args, ps.max_span_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev, const JabasStepArgs* args,
@@ -534,8 +570,9 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     if (rc != JABAS_OK) return rc;
     uint32_t tiles = 0;
     const int oc = opt_class_of(args->opt_kind);
-    rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind, launch_block(args->K, args->grad_dtype, oc),
-                     &a.span0, &tiles);
+    const bool stats = args->stats != 0;
+    rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind,
+                     launch_block(args->K, args->grad_dtype, oc, stats), &a.span0, &tiles);
     if (rc != JABAS_OK) return rc;
     if (oc == 1 && args->momentum != 0.0 && !span->state1) return JABAS_ERR_NULL;
     if (span->bound_count && !bounds_dev) return JABAS_ERR_NULL;
@@ -546,7 +583,7 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.chunks = nullptr;
     a.chunk_prefix = nullptr;
     a.n_span = 1;
-    a.chunk_tiles = launch_chunk_tiles(args->K, args->grad_dtype, oc);
+    a.chunk_tiles = launch_chunk_tiles(args->K, args->grad_dtype, oc, stats);
     a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, a.chunk_tiles));
     a.use_inline = 1;
     return run_fused(a, args, a.n_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));

@@ -169,11 +169,11 @@ template <int K, int DT, int U> struct TileRegs {
 
 // Issues every load of U consecutive full tiles. e is the (rebased) index of this
 // thread's first element in the first tile.
-template <int K, int DT, int OPT, int U>
+template <int K, int DT, int OPT, int U, int BS>
 __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(BS) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
@@ -194,7 +194,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
                                         double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, STATS)) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
@@ -226,13 +226,14 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 template <int K, int DT, int OPT, bool STATS, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
                                          const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * Grad<DT>::EPT;
+    constexpr int BS = launch_block(K, DT, OPT, STATS);
+    constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     uint32_t i = 0;
     for (; i + U <= nfull; i += U, e += U * TE) {
         TileRegs<K, DT, U> r;
-        issue_loads<K, DT, OPT, U>(r, sp, e, load_s1);
+        issue_loads<K, DT, OPT, U, BS>(r, sp, e, load_s1);
         consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, clip, use_s1, load_s1, acc);
     }
     if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, clip, acc);
@@ -287,9 +288,9 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT)) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, STATS)) * EPT;
     constexpr int UW = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
-    constexpr int CT = launch_chunk_tiles(K, DT, OPT);
+    constexpr int CT = launch_chunk_tiles(K, DT, OPT, STATS);
     constexpr int U0 = UW < CT ? UW : CT;     // never more than a chunk holds
     constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
@@ -370,10 +371,10 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
 }
 
 template <int K, int DT, int OPT, bool STATS>
-__global__ void __launch_bounds__(launch_block(K, DT, OPT)) fused_kernel(const KArgs a) {
+__global__ void __launch_bounds__(launch_block(K, DT, OPT, STATS)) fused_kernel(const KArgs a) {
     constexpr int NS = NStats<K, STATS>::value;
-    constexpr int BS = launch_block(K, DT, OPT);
-    constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT);     // the host cuts the chunk table for the same shape
+    constexpr int BS = launch_block(K, DT, OPT, STATS);
+    constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT, STATS);     // the host cuts the chunk table for the same shape
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
     const uint32_t b = blockIdx.x;
     double acc[NS];
@@ -419,7 +420,7 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
 #define JABAS_IDLE_LDS_BYTES 32768u
 #endif
     constexpr unsigned idle = (OPT == OPT_ADAM && !STATS && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
-    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(launch_block(K, DT, OPT)), idle, stream, a);
+    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(launch_block(K, DT, OPT, STATS)), idle, stream, a);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -10,12 +10,14 @@ namespace jabas {
 
 // Launch shape: threads per workgroup and tiles per workgroup (a tile = one 16-byte fp32 vector per
 // thread; a chunk = the tiles one workgroup processes). Small chunks keep the streamed window of every
-// buffer compact (higher HBM rate) and cut the ramp-up / drain of a launch; kernels with many gradient
-// streams have low occupancy and a long prologue, and do better with twice the work per workgroup.
-// Measured per kernel family (A/B builds of the whole library):
-//   SGD, fp32 gradients, K <= 4   128 threads x 2 tiles (1024 elements): +2-5 % over 256 x 2
-//   Adam/AdamW and every other    256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
-//   case                          1024 threads were all slower with statistics on
+// buffer compact (higher HBM rate) and cut the ramp-up / drain of a launch; kernels that carry fp64
+// statistics have low occupancy and a long epilogue, and do better with more work per workgroup.
+// Measured per kernel family (A/B builds of the whole library, every shape passes the parity suite):
+//   with statistics               256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
+//                                 1024 threads were all slower (-2 ... -15 %)
+//   plain, K > 4                  512 threads x 1 tile: +3 ... +8 % over 256 x 4 (bf16 and fp32, SGD and Adam)
+//   plain, SGD, fp32, K <= 4      128 threads x 2 tiles: +2 ... +5 % over 256 x 2
+//   plain, everything else        256 threads x 2 tiles
 // The macros let a tuning build try other shapes without touching the sources.
 #ifndef JABAS_BLOCK
 #define JABAS_BLOCK 256
@@ -23,28 +25,40 @@ namespace jabas {
 #ifndef JABAS_BLOCK_SGD
 #define JABAS_BLOCK_SGD 128
 #endif
+#ifndef JABAS_BLOCK_MANYK
+#define JABAS_BLOCK_MANYK 512
+#endif
 #ifndef JABAS_CHUNK_TILES_LO
 #define JABAS_CHUNK_TILES_LO 2
 #endif
 #ifndef JABAS_CHUNK_TILES_HI
 #define JABAS_CHUNK_TILES_HI 4
 #endif
+#ifndef JABAS_CHUNK_TILES_MANYK
+#define JABAS_CHUNK_TILES_MANYK 1
+#endif
 constexpr int kBlock = JABAS_BLOCK;         // default threads per workgroup (256 = 4 wave64)
-static_assert(kBlock % 64 == 0 && kBlock >= 64 && kBlock <= 1024, "whole waves");
-static_assert(JABAS_BLOCK_SGD % 64 == 0 && JABAS_BLOCK_SGD >= 64 && JABAS_BLOCK_SGD <= 1024, "whole waves");
 constexpr int kWaves = kBlock / 64;
+constexpr bool block_ok(int b) { return b % 64 == 0 && b >= 64 && b <= 1024; }
+static_assert(block_ok(JABAS_BLOCK) && block_ok(JABAS_BLOCK_SGD) && block_ok(JABAS_BLOCK_MANYK), "whole waves");
 constexpr int kMinChunkTiles = JABAS_CHUNK_TILES_LO;
 constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
 // opt_class: 0 none, 1 SGD, 2 Adam/AdamW. The shape depends on what a plan is encoded for (K, gradient
-// dtype, optimizer class), never on per-step flags, so one chunk table serves every step.
-__host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class) {
-    return (opt_class == 1 && K <= 4 && grad_dtype == JABAS_F32) ? JABAS_BLOCK_SGD : kBlock;
+// dtype, optimizer class) and on whether the launch carries statistics; a plan holds one chunk table
+// per shape, so it serves every step.
+__host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, bool stats) {
+    if (stats) return kBlock;
+    if (K > 4) return JABAS_BLOCK_MANYK;
+    return (opt_class == 1 && grad_dtype == JABAS_F32) ? JABAS_BLOCK_SGD : kBlock;
 }
-__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int /*opt_class*/) {
-    return K > 4 ? kMaxChunkTiles : kMinChunkTiles;
+__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int /*opt_class*/, bool stats) {
+    if (K > 4) return stats ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
+    return kMinChunkTiles;
 }
-// Fewest elements any chunk covers, over all shapes: sizes workspaces that must fit every launch.
-constexpr int kMinChunkElems = (JABAS_BLOCK_SGD < JABAS_BLOCK ? JABAS_BLOCK_SGD : JABAS_BLOCK) * 4 * JABAS_CHUNK_TILES_LO;
+constexpr int imin(int a, int b) { return a < b ? a : b; }
+// Fewest elements any chunk covers, over all shapes: sizes workspaces and blobs that must fit every launch.
+constexpr int kMinChunkElems = 4 * imin(imin(JABAS_BLOCK_SGD * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
+                                        imin(JABAS_BLOCK_MANYK * JABAS_CHUNK_TILES_MANYK, JABAS_BLOCK * JABAS_CHUNK_TILES_HI));
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
 // Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer

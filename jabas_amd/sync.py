@@ -224,7 +224,8 @@ class SyncPlan:
         L.check(lib.jabas_plan_encode(c_spans, n_span, c_bounds if all_bounds else None, len(all_bounds),
                                       self.K, grad_dtype_code(gdt), opt_kind_code,
                                       self._host.ctypes.data, nbytes), "jabas_plan_encode")
-        self.n_chunks = int(lib.jabas_plan_chunks(self._host.ctypes.data))
+        self.n_chunks = int(lib.jabas_plan_chunks(self._host.ctypes.data, 0))            # workgroups of a plain launch
+        self.n_chunks_stats = int(lib.jabas_plan_chunks(self._host.ctypes.data, 1))      # of a launch with statistics
         self._dev = torch.from_numpy(self._host.view(np.int64)).to(dev)
         self.ws = Workspace(lib.jabas_plan_workspace_bytes(self._host.ctypes.data), n_span, dev)
         self.n_span = n_span

@@ -77,7 +77,8 @@ int main(void) {
     if (!blob) return 2;
     int rc = jabas_plan_encode(spans, 2, bounds, 2, 2, JABAS_F32, JABAS_OPT_SGD, blob, nbytes);
     printf("encode %d\n", rc);
-    printf("chunks %lld\n", (long long)jabas_plan_chunks(blob));
+    printf("chunks %lld\n", (long long)jabas_plan_chunks(blob, 0));
+    printf("chunks_stats %lld\n", (long long)jabas_plan_chunks(blob, 1));
     printf("workspace %zu\n", jabas_plan_workspace_bytes(blob));
     spans[1].grads[1] = (char*)spans[1].grads[1] + 4; /* breaks the 16-byte congruence rule */
     rc = jabas_plan_encode(spans, 2, bounds, 2, 2, JABAS_F32, JABAS_OPT_SGD, blob, nbytes);

@@ -82,15 +82,17 @@ def test_plan_encode_counts_chunks():
     sizes = [4096, 4097, 1, 0, 10 * 4096 + 5]
     rc, blob, _ = _encode([_span(n) for n in sizes])
     assert rc == L.OK
-    assert lib.jabas_plan_chunks(blob.ctypes.data) == 2 + 3 + 1 + 0 + 21
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == 2 + 3 + 1 + 0 + 21
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == 2 + 3 + 1 + 0 + 21      # K <= 4 without optimizer: one shape
     assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (27 + 5) * L.STATS_STRIDE * 8     # a row per chunk and per span, at least
-    for K in (8, 16):
+    for K in (8, 16):                  # K > 4: 4 tiles of 1024 with statistics, one tile of 2048 without
         rc, blob, _ = _encode([_span(n, K=K) for n in sizes], K=K)
         assert rc == L.OK
-        assert lib.jabas_plan_chunks(blob.ctypes.data) == 1 + 2 + 1 + 0 + 11
+        assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == 1 + 2 + 1 + 0 + 11
+        assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == 2 + 3 + 1 + 0 + 21
     # a span that starts 3 elements into a 16-byte line needs one more tile when it is exactly full
     rc, blob, _ = _encode([_span(4096, skew=3)])
-    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data) == 3
+    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == 3
 
 
 def test_plan_encode_bf16_positions_are_counted_in_elements():
@@ -154,7 +156,7 @@ def test_plan_blob_too_small_and_garbage_header():
     assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, 128) == L.ERR_PLAN
     assert lib.jabas_plan_encode(spans, 1, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, nbytes) == L.OK
     junk = np.zeros(64, dtype=np.uint64)
-    assert lib.jabas_plan_chunks(junk.ctypes.data) == L.ERR_PLAN
+    assert lib.jabas_plan_chunks(junk.ctypes.data, 0) == L.ERR_PLAN
     assert lib.jabas_plan_workspace_bytes(junk.ctypes.data) == 0
     args = L.JabasStepArgs()
     args.K = 2
@@ -235,8 +237,9 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
     assert seen[("version", "jabas_sync")].startswith("0.")
     assert seen[("status0", "ok")] == ""
     assert seen[("encode", "0")] == ""
-    assert seen[("chunks", "14")] == ""                      # SGD, K = 2, fp32: 1024 elements per chunk -> 5 + 9
-    assert int(next(n for (k, n) in seen if k == "workspace")) >= (14 + 2) * L.STATS_STRIDE * 8
+    assert seen[("chunks", "14")] == ""                      # SGD, K = 2, fp32, plain: 1024 elements per chunk -> 5 + 9
+    assert seen[("chunks_stats", "8")] == ""                 # with statistics: 2048 per chunk -> 3 + 5
+    assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * L.STATS_STRIDE * 8
     assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
 
 
@@ -274,22 +277,24 @@ def test_plan_encode_rejects_overlapping_written_buffers():
 
 
 def test_launch_shape_follows_what_the_plan_is_encoded_for():
-    """SGD with fp32 gradients and K <= 4 runs 128-thread workgroups (1024 elements per chunk); every other
-    kernel family 256 threads x 2 tiles (K <= 4) or 4 tiles. A plan serves launches of its own optimizer
-    class only."""
+    """Launches with statistics run 256-thread workgroups of 2 tiles (K <= 4) or 4 tiles; plain launches
+    512 threads x 1 tile for K > 4, 128 threads x 2 tiles for SGD with fp32 gradients and K <= 4, else
+    256 x 2. A plan holds a chunk table per shape and serves launches of its own optimizer class only."""
     lib = L.lib()
     n = 10 * 4096
     def chunks(K, dtype, opt, gs=4):
         rc, blob, _ = _encode([_span(n, K=K, gs=gs, opt=True)], K=K, dtype=dtype, opt=opt)
         assert rc == L.OK
-        return lib.jabas_plan_chunks(blob.ctypes.data), blob
-    assert chunks(2, L.F32, L.OPT_SGD)[0] == n // 1024
-    assert chunks(4, L.F32, L.OPT_SGD)[0] == n // 1024
-    assert chunks(5, L.F32, L.OPT_SGD)[0] == n // 4096
-    assert chunks(2, L.BF16, L.OPT_SGD, gs=2)[0] == n // 2048
-    assert chunks(2, L.F32, L.OPT_ADAM)[0] == n // 2048
-    assert chunks(2, L.F32, L.OPT_NONE)[0] == n // 2048
+        return (lib.jabas_plan_chunks(blob.ctypes.data, 0), lib.jabas_plan_chunks(blob.ctypes.data, 1)), blob
+    assert chunks(2, L.F32, L.OPT_SGD)[0] == (n // 1024, n // 2048)
+    assert chunks(4, L.F32, L.OPT_SGD)[0] == (n // 1024, n // 2048)
+    assert chunks(5, L.F32, L.OPT_SGD)[0] == (n // 2048, n // 4096)
+    assert chunks(2, L.BF16, L.OPT_SGD, gs=2)[0] == (n // 2048, n // 2048)
+    assert chunks(2, L.F32, L.OPT_ADAM)[0] == (n // 2048, n // 2048)
+    assert chunks(8, L.BF16, L.OPT_ADAMW, gs=2)[0] == (n // 2048, n // 4096)
+    assert chunks(2, L.F32, L.OPT_NONE)[0] == (n // 2048, n // 2048)
     _, blob = chunks(2, L.F32, L.OPT_SGD)
+    assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (n // 2048 + 1) * L.STATS_STRIDE * 8
     args = L.JabasStepArgs()
     args.K, args.grad_dtype, args.opt_kind = 2, L.F32, L.OPT_NONE
     assert lib.jabas_sync_fused(blob.ctypes.data, 0x1000, C.byref(args), None, None, 0, None) == L.ERR_PLAN
