@@ -97,6 +97,21 @@ def time_config(cfg, device, steps, warmup, torch):
     torch.cuda.synchronize()
     launch_ms = sorted(a.elapsed_time(b) for a, b in evs)
     mean_launch_ms = sum(launch_ms) / len(launch_ms)
+    # the step between statistic steps (statistics run every `interval` steps in training): same
+    # bytes, no fp64 sums, the launch shape of the plain kernels
+    plain = None
+    if cfg.stats:
+        for i in range(warmup):
+            engines[i % n].step(stats=False)
+        p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        p0.record()
+        for i in range(steps):
+            engines[i % n].step(stats=False)
+        p1.record()
+        torch.cuda.synchronize()
+        plain_ms = max(p0.elapsed_time(p1), 1e-6) / steps
+        plain = dict(ms_per_step=plain_ms, GBps=bytes_per_step / 1e9 / (plain_ms / 1e3),
+                     pct_hbm_peak=100.0 * bytes_per_step / 1e9 / (plain_ms / 1e3) / HBM_PEAK_GBPS)
     stats_rows = engines[0].step(stats=True) if cfg.stats else None
     cos = engines[0].cosine(stats_rows) if stats_rows is not None else None
     finite = bool(torch.isfinite(engines[0].param).all())
@@ -108,7 +123,7 @@ def time_config(cfg, device, steps, warmup, torch):
         launch_ms_mean=mean_launch_ms, launch_ms_median=launch_ms[len(launch_ms) // 2], launch_ms_min=launch_ms[0],
         GBps_launch=bytes_per_step / 1e9 / (mean_launch_ms / 1e3),
         pct_hbm_peak=100.0 * bytes_per_step / 1e9 / (mean_launch_ms / 1e3) / HBM_PEAK_GBPS,
-        buffer_copies=copies, cosine=cos, finite=finite)
+        buffer_copies=copies, cosine=cos, finite=finite, step_without_statistics=plain)
     del engines
     torch.cuda.empty_cache()
     return res
@@ -235,9 +250,13 @@ def main():
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
     for cfg in order:
         results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch)
-        print(f"# {cfg.name}: {results[cfg.name]['ms_per_step']:.4f} ms/step, "
-              f"{results[cfg.name]['GBps']:.0f} GB/s, {results[cfg.name]['pct_hbm_peak']:.1f} % of HBM peak",
-              file=sys.stderr, flush=True)
+        r = results[cfg.name]
+        extra = ""
+        if r["step_without_statistics"]:
+            extra = (f"; without statistics {r['step_without_statistics']['ms_per_step']:.4f} ms/step, "
+                     f"{r['step_without_statistics']['pct_hbm_peak']:.1f} %")
+        print(f"# {cfg.name}: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s, "
+              f"{r['pct_hbm_peak']:.1f} % of HBM peak{extra}", file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
                                                                       args.steps, torch)
