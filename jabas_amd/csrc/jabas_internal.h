@@ -15,7 +15,8 @@ namespace jabas {
 // Measured per kernel family (A/B builds of the whole library, every shape passes the parity suite):
 //   with statistics               256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
 //                                 1024 threads were all slower (-2 ... -15 %)
-//   plain, K > 4                  512 threads x 1 tile: +3 ... +8 % over 256 x 4 (bf16 and fp32, SGD and Adam)
+//   plain with optimizer, K > 4   512 threads x 1 tile: +3 ... +8 % over 256 x 4 (bf16 and fp32, SGD and Adam);
+//                                 aggregate-only launches lose 20 % there and stay at 256 x 4
 //   plain, SGD, fp32, K <= 4      128 threads x 2 tiles: +2 ... +5 % over 256 x 2
 //   plain, everything else        256 threads x 2 tiles
 // The macros let a tuning build try other shapes without touching the sources.
@@ -47,12 +48,12 @@ constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
 // dtype, optimizer class) and on whether the launch carries statistics; a plan holds one chunk table
 // per shape, so it serves every step.
 __host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, bool stats) {
-    if (stats) return kBlock;
+    if (stats || opt_class == 0) return kBlock;
     if (K > 4) return JABAS_BLOCK_MANYK;
     return (opt_class == 1 && grad_dtype == JABAS_F32) ? JABAS_BLOCK_SGD : kBlock;
 }
-__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int /*opt_class*/, bool stats) {
-    if (K > 4) return stats ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
+__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int opt_class, bool stats) {
+    if (K > 4) return (stats || opt_class == 0) ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
     return kMinChunkTiles;
 }
 constexpr int imin(int a, int b) { return a < b ? a : b; }

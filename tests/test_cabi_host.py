@@ -85,11 +85,11 @@ def test_plan_encode_counts_chunks():
     assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == 2 + 3 + 1 + 0 + 21
     assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == 2 + 3 + 1 + 0 + 21      # K <= 4 without optimizer: one shape
     assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (27 + 5) * L.STATS_STRIDE * 8     # a row per chunk and per span, at least
-    for K in (8, 16):                  # K > 4: 4 tiles of 1024 with statistics, one tile of 2048 without
+    for K in (8, 16):                  # K > 4 without optimizer: 4 tiles of 1024 for both kinds of launch
         rc, blob, _ = _encode([_span(n, K=K) for n in sizes], K=K)
         assert rc == L.OK
         assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == 1 + 2 + 1 + 0 + 11
-        assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == 2 + 3 + 1 + 0 + 21
+        assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == 1 + 2 + 1 + 0 + 11
     # a span that starts 3 elements into a 16-byte line needs one more tile when it is exactly full
     rc, blob, _ = _encode([_span(4096, skew=3)])
     assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == 3
@@ -293,6 +293,7 @@ def test_launch_shape_follows_what_the_plan_is_encoded_for():
     assert chunks(2, L.F32, L.OPT_ADAM)[0] == (n // 2048, n // 2048)
     assert chunks(8, L.BF16, L.OPT_ADAMW, gs=2)[0] == (n // 2048, n // 4096)
     assert chunks(2, L.F32, L.OPT_NONE)[0] == (n // 2048, n // 2048)
+    assert chunks(8, L.F32, L.OPT_NONE)[0] == (n // 4096, n // 4096)
     _, blob = chunks(2, L.F32, L.OPT_SGD)
     assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (n // 2048 + 1) * L.STATS_STRIDE * 8
     args = L.JabasStepArgs()
