@@ -3,19 +3,21 @@
 // streams are fully unrolled into independent 128-bit loads.
 //
 // Execution shape
-//   - one 256-thread workgroup (4 wave64) per chunk of 2 or 4 consecutive tiles of
-//     one span; a tile is 256 threads x 4 elements (one 16-byte vector of every fp32
-//     buffer, one 8-byte vector of a bf16 gradient buffer). Small, short-lived workgroups dispatched in order keep the part of every
-//     buffer that is being streamed at any moment compact, which on MI355X sustains a
-//     markedly higher HBM rate than a persistent grid that spreads over the whole buffers;
-//   - every global access is a 128-bit vector access with the nontemporal hint (each byte
-//     is touched exactly once per step);
+//   - one workgroup per chunk of consecutive tiles of one span; a tile is one 16-byte vector of
+//     every fp32 buffer (one 8-byte vector of a bf16 gradient buffer) per thread. Threads per
+//     workgroup and tiles per chunk depend on the kernel family (launch_block / launch_chunk_tiles):
+//     256 threads x 2 or 4 tiles with statistics, 128 x 2, 256 x 2 or 512 x 1 without. Small,
+//     short-lived workgroups dispatched in order keep the part of every buffer that is being
+//     streamed at any moment compact, which on MI355X sustains a markedly higher HBM rate than a
+//     persistent grid that spreads over the whole buffers;
+//   - every global access is a vector access with the nontemporal hint (each byte is touched
+//     exactly once per step);
 //   - tiles that lie wholly inside the live range of a span and inside one parameter
 //     group take the vector path (all loads of U tiles issued before any arithmetic);
 //     the few tiles that straddle a span end or a group change take a scalar path;
-//   - statistics: per-thread fp64 accumulators -> wave64 DPP tree -> LDS across the
-//     4 waves -> one partial row per workgroup in the workspace, summed in fixed order by
-//     the finalize kernel. The tree is fixed, so results are bit-identical run to run.
+//   - statistics: per-thread fp64 accumulators -> LDS -> 16-way sums in fixed order -> DPP row
+//     reduction -> one partial row of 4 + K doubles per workgroup in the workspace, summed in
+//     fixed order by the finalize kernel. The order is fixed, so results are bit-identical run to run.
 //
 // Arithmetic is compiled with -ffp-contract=off: every fp32 product and sum of the
 // aggregate and of the optimizer formulas is rounded on its own, so results can be
