@@ -113,28 +113,30 @@ class VSWFlatSync:
         return slice(bk.offset, bk.offset + bk.numel)
 
     # ---- the step ----------------------------------------------------------------
-    def step_args(self, stats=False, lr_scale=1.0, with_opt=True):
+    def step_args(self, stats=False, lr_scale=1.0, with_opt=True, accumulations=1):
         opt = self.opt if with_opt else None
         first = self.step_count == 0
         return make_step_args(self.batches, self.grad_dtype, stats=stats, opt=opt, step=self.step_count + 1,
-                              first_step=first, lr_scale=lr_scale)
+                              first_step=first, lr_scale=lr_scale, accumulations=accumulations)
 
-    def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None):
+    def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None, accumulations=1):
         """One sync step over the whole gradient set. Returns the per-span stats tensor
         when ``stats`` is set.
 
         Without ``clip_norm``: one fused launch. With it (global-norm clipping as
         examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
         clipping coefficient on the device, then the optimizer launch over the aggregate
-        scaled by it -- the norm has to be known before any weight moves."""
+        scaled by it -- the norm has to be known before any weight moves.
+
+        ``accumulations``: micro-batches every VSW summed into its buckets since the last step."""
         if clip_norm is None or self.opt is None:
-            args = self.step_args(stats=stats, lr_scale=lr_scale)
+            args = self.step_args(stats=stats, lr_scale=lr_scale, accumulations=accumulations)
             out = self.plan.run(args, stream=stream)
             self.step_count += 1
             return out
         if self._plan_agg is None:
             self._build_clip_plans()
-        rows = self._plan_agg.run(self.step_args(stats=True, with_opt=False), stream=stream)
+        rows = self._plan_agg.run(self.step_args(stats=True, with_opt=False, accumulations=accumulations), stream=stream)
         coef = clip_coef(rows, clip_norm, out=self._coef, stream=stream)
         args = make_step_args((1,), torch.float32, stats=False, opt=self.opt, step=self.step_count + 1,
                               first_step=self.step_count == 0, lr_scale=lr_scale, grad_scale=coef)

@@ -16,21 +16,30 @@ from . import _lib as L
 
 
 # ----------------------------------------------------------------------------- weights
-def batch_weights(batches, half_id=None):
+def batch_weights(batches, half_id=None, accumulations=1):
     """Per-VSW fp32 weights of the batch-weighted aggregate and of the two halves.
 
     w_k = fp32(b_k / B): the quotient is formed in double and rounded once, which is what
     a Python float becomes when ATen applies it to an fp32 tensor. Halves follow the
     reference's rank-parity split (jabas/train/trainer.py:427-432) mapped onto the VSW
     index: even k -> half A (0), odd k -> half B (1).
+
+    ``accumulations``: micro-batches each VSW accumulated into its bucket before this sync step
+    (IIDP's accum_step + 1). The bucket then holds a sum of that many mean gradients, and the
+    reference's divisor, the number of decoupled workers, counts them
+    (jabas/train/trainer.py:594-599: global batch = local batch x decoupled workers), so
+    w_k = fp32(b_k / (B * accumulations)).
     """
+    if int(accumulations) < 1:
+        raise ValueError("accumulations must be a positive integer")
     b = [float(x) for x in batches]
     K = len(b)
     if not 1 <= K <= L.MAX_K:
         raise ValueError(f"number of VSWs must be in 1..{L.MAX_K}, got {K}")
     if any(x <= 0 for x in b):
         raise ValueError(f"local batch sizes must be positive: {batches}")
-    total = sum(b)
+    acc = float(int(accumulations))
+    total = sum(b) * acc
     w = np.array([x / total for x in b], dtype=np.float64).astype(np.float32)
     if half_id is None:
         half_id = [k % 2 for k in range(K)]
@@ -39,7 +48,7 @@ def batch_weights(batches, half_id=None):
         raise ValueError("half_id must hold K entries of 0 or 1")
     hw = np.zeros(K, dtype=np.float32)
     for h in (0, 1):
-        tot = sum(x for x, hid in zip(b, half_id) if hid == h)
+        tot = sum(x for x, hid in zip(b, half_id) if hid == h) * acc
         for k in range(K):
             if half_id[k] == h:
                 hw[k] = np.float32(b[k] / tot)
@@ -65,14 +74,14 @@ def grad_dtype_code(dtype):
 
 
 def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_step=False, half_id=None,
-                   lr_scale=1.0, grad_scale=None):
+                   lr_scale=1.0, grad_scale=None, accumulations=1):
     """Builds the JabasStepArgs of one call.
 
     ``opt``: None or dict(kind='sgd'|'adam'|'adamw', groups=[dict(lr=, weight_decay=)], plus
     momentum/dampening/nesterov or betas/eps). ``step`` is the 1-based Adam step count,
     ``lr_scale`` the adaptive-batching LR modifier (jabas/train/trainer.py:693-700).
     """
-    w, hid, hw = batch_weights(batches, half_id)
+    w, hid, hw = batch_weights(batches, half_id, accumulations)
     a = L.JabasStepArgs()
     a.K = len(w)
     a.grad_dtype = grad_dtype_code(grad_dtype)

@@ -117,6 +117,7 @@ class VSWSyncTrainer:
         self.local_optimizers, self.local_schedulers = [], []
         self.main_model = self.main_optimizer = None
         self.sync_step = 0
+        self.accumulated = 0                      # compute() calls since the last step (IIDP's accum_step + 1 at step time)
         self.engine = None
         self._step_tensor = torch.zeros((), dtype=torch.float32)       # Adam's state['step'], shared by all parameters
         self.cos_placeholder = None
@@ -244,7 +245,9 @@ class VSWSyncTrainer:
 
     # ------------------------------------------------------------------- one iteration
     def compute(self, data):
-        """data: one (input, target) pair per VSW, already on the GPU."""
+        """data: one (input, target) pair per VSW, already on the GPU. May be called several times
+        before ``step`` (gradient accumulation, IIDP's accum_step): every call adds one micro-batch
+        gradient per VSW to its buckets, and the step divides by the number of calls."""
         if len(data) != self.num_models:
             raise ValueError(f"expected {self.num_models} local batches, got {len(data)}")
         cur = torch.cuda.current_stream(self.gpu)
@@ -256,9 +259,14 @@ class VSWSyncTrainer:
                 loss.backward()
                 if self.grad_dtype != torch.float32:
                     for i, p in enumerate(m.parameters()):
-                        self.engine.grad_view(k, i).copy_(p.grad.reshape(-1))
+                        view = self.engine.grad_view(k, i)
+                        if self.accumulated == 0:
+                            view.copy_(p.grad.reshape(-1))
+                        else:
+                            view.add_(p.grad.reshape(-1).to(view.dtype))
                         p.grad = None
                 losses.append(loss.detach())
+        self.accumulated += 1
         return losses
 
     def step(self):
@@ -268,7 +276,9 @@ class VSWSyncTrainer:
         st = self.similarity_state
         want = st.step % st.interval == 0
         self._refresh_hyperparameters()
-        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm)
+        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm,
+                                accumulations=max(1, self.accumulated))
+        self.accumulated = 0
         self.sync_step += 1
         self._step_tensor.fill_(float(self.engine.step_count))
         if self.local_schedulers:

@@ -38,16 +38,19 @@ DOT_AB, NORM_A, NORM_B, NORM_AGG, NORM_VSW0 = 0, 1, 2, 3, 4
 
 
 # ------------------------------------------------------------------------------ weights
-def batch_weights(batches, half_id=None):
-    """w_k = fp32(b_k / B) with the quotient formed in double; half weights likewise over
-    each half's own batch total. Default halves: even VSW index -> A, odd -> B."""
+def batch_weights(batches, half_id=None, accumulations=1):
+    """w_k = fp32(b_k / (B * accumulations)) with the quotient formed in double; half weights likewise
+    over each half's own batch total. Default halves: even VSW index -> A, odd -> B. accumulations =
+    micro-batches summed into each bucket before the step (every one of them a decoupled worker in the
+    reference's count, jabas/train/trainer.py:594-599)."""
     b = [float(x) for x in batches]
     K = len(b)
-    total = math.fsum(b)
+    total = math.fsum(b) * float(int(accumulations))
     w = [float(np.float32(x / total)) for x in b]
     if half_id is None:
         half_id = [k % 2 for k in range(K)]
-    tot = [math.fsum(x for x, h in zip(b, half_id) if h == 0), math.fsum(x for x, h in zip(b, half_id) if h == 1)]
+    acc = float(int(accumulations))
+    tot = [math.fsum(x for x, h in zip(b, half_id) if h == 0) * acc, math.fsum(x for x, h in zip(b, half_id) if h == 1) * acc]
     hw = [float(np.float32(b[k] / tot[half_id[k]])) for k in range(K)]
     return w, list(half_id), hw
 

@@ -315,3 +315,40 @@ def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
         trainer.prepare_weight_sync_method(torch.optim.SGD(groups, lr=0.1, momentum=0.9))
     with pytest.raises(ValueError):                         # a parameter outside every group
         trainer.prepare_weight_sync_method(torch.optim.SGD(list(trainer.main_model.parameters())[:2], lr=0.1))
+
+
+def test_trainer_accumulates_micro_batches_between_steps(gpu):
+    """compute() twice, then step(): every VSW's bucket holds the sum of two micro-batch gradients, the
+    step divides by the number of accumulated micro-batches (IIDP's accum_step + 1)."""
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (4, 2)
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, interval=1)
+    trainer.prepare_stream_parallel(_mlp(21), crit)
+    mine = torch.optim.SGD(_groups(trainer.main_model), lr=0.05, momentum=0.9, foreach=False)
+    trainer.prepare_weight_sync_method(mine, None, _groups)
+    ref_model = _mlp(21).to(gpu)
+    ref_opt = torch.optim.SGD(_groups(ref_model), lr=0.05, momentum=0.9, foreach=False)
+    w, _, _ = O.batch_weights(batches, accumulations=2)
+    for step in range(1, 4):
+        sums = None
+        for micro in range(2):
+            gen = torch.Generator().manual_seed(1000 * step + micro)
+            data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu))
+                    for b in batches]
+            trainer.compute(data)
+            per_vsw = []
+            for x, y in data:
+                ref_model.zero_grad(set_to_none=True)
+                crit(ref_model(x), y).backward()
+                per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+            sums = per_vsw if sums is None else [[a + b for a, b in zip(s, g)] for s, g in zip(sums, per_vsw)]
+        assert trainer.accumulated == 2
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(sums[0][i], w[0]), torch.mul(sums[1][i], w[1]))
+        ref_opt.step()
+        trainer.step()
+        torch.cuda.synchronize()
+        assert trainer.accumulated == 0
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), step

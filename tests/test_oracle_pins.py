@@ -331,3 +331,23 @@ def test_clip_matches_torch_clip_grad_norm(max_norm):
         assert c > 1.0 and torch.equal(got, flat)              # above the norm: untouched, bit for bit
     else:
         assert c < 1.0 and float(torch.linalg.vector_norm(got.double())) == pytest.approx(max_norm, rel=1e-4)
+
+
+def test_accumulated_micro_batches_count_as_decoupled_workers():
+    """With A micro-batches summed into every bucket the divisor grows by A (the reference's
+    global batch = local batch x decoupled workers, jabas/train/trainer.py:594-599)."""
+    w, hid, hw = O.batch_weights((4, 2, 2), accumulations=2)
+    assert w == [0.25, 0.125, 0.125] and hid == [0, 1, 0]
+    assert hw == [float(np.float32(4 / 12)), 0.5, float(np.float32(2 / 12))]
+    from jabas_amd import sync
+    w2, hid2, hw2 = sync.batch_weights((4, 2, 2), accumulations=2)
+    assert [float(x) for x in w2] == w and [float(x) for x in hw2] == hw
+    with pytest.raises(ValueError):
+        sync.batch_weights((4, 2), accumulations=0)
+    # equal batches, power-of-two count: accumulating twice equals one worker set of twice the size
+    g = _grads(2, 1000, 77)
+    summed = [torch.add(g[0], g[1]), torch.add(g[1], g[0])]                 # two micro-batches per worker
+    w4, _, _ = O.batch_weights((8, 8), accumulations=2)
+    got = torch.add(torch.mul(summed[0], w4[0]), torch.mul(summed[1], w4[1]))
+    want = O.aggregate([g[0], g[1], g[1], g[0]], (8, 8, 8, 8))
+    assert torch.allclose(got, want, rtol=0, atol=float(torch.finfo(torch.float32).eps) * float(want.abs().max()) * 4)
