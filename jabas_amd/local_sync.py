@@ -58,6 +58,7 @@ class LocalBucketSync:
         self.param_buckets = param_buckets or {}     # bucket index -> dict(param=, state1=, state2=, bounds=, fanout=)
         self.step_count = 0
         self.lr_scale = 1.0
+        self.accumulations = 1                 # micro-batches each VSW summed into its buckets (no_sync() steps + 1)
         self._launcher = launcher or self._launch_fused
         self._lock = threading.Lock()
         self._slots = {}
@@ -122,14 +123,15 @@ class LocalBucketSync:
     # ------------------------------------------------------------- the default launcher
     def _step_args(self, dtype, want_stats, with_opt):
         """JabasStepArgs of this step, built once per (step, kind of launch) and shared by its buckets."""
-        key = (self.step_count, self.lr_scale, dtype, bool(want_stats), bool(with_opt))
+        key = (self.step_count, self.lr_scale, self.accumulations, dtype, bool(want_stats), bool(with_opt))
         hit = self._args_cache.get(key)
         if hit is None:
             if len(self._args_cache) > 8:
                 self._args_cache.clear()
             hit = self._args_cache[key] = sync.make_step_args(
                 self.batches, dtype, stats=want_stats, opt=self.opt if with_opt else None,
-                step=self.step_count + 1, first_step=self.step_count == 0, lr_scale=self.lr_scale)
+                step=self.step_count + 1, first_step=self.step_count == 0, lr_scale=self.lr_scale,
+                accumulations=self.accumulations)
         return hit
 
     def _launch_fused(self, bucket_index, tensors, want_stats):
