@@ -561,3 +561,19 @@ def test_random_buckets_through_the_inline_path(gpu, seed):
                 assert torch.equal(_bits(s1_d), _bits(s1_h)), (si, step)
                 if adam:
                     assert torch.equal(_bits(s2_d), _bits(s2_h)), (si, step)
+
+
+def test_plan_with_nothing_but_empty_spans(gpu):
+    """No workgroup to launch: the statistics rows still come back, all zero, and nothing is touched."""
+    from jabas_amd import sync, _lib as L
+    g = [torch.zeros(16, device=gpu) for _ in range(2)]
+    p, m = torch.ones(16, device=gpu), torch.zeros(16, device=gpu)
+    spans = [sync.SpanSpec([t[4:4] for t in g], agg_out=g[0][4:4], param=p[4:4], state1=m[4:4]) for _ in range(3)]
+    plan = sync.SyncPlan(spans, L.OPT_SGD)
+    assert plan.n_chunks == 0 and plan.n_chunks_stats == 0
+    rows = plan.run(sync.make_step_args((1, 1), torch.float32, stats=True, opt=SGD, step=1, first_step=True))
+    torch.cuda.synchronize()
+    assert rows.shape == (3, L.STATS_STRIDE) and torch.count_nonzero(rows) == 0
+    assert plan.run(sync.make_step_args((1, 1), torch.float32, stats=False, opt=SGD, step=2)) is None
+    torch.cuda.synchronize()
+    assert torch.equal(p, torch.ones(16, device=gpu)) and torch.count_nonzero(m) == 0
