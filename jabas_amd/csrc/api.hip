@@ -288,20 +288,20 @@ __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const ui
 }
 
 template <int NS>
-void launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
-                     uint32_t out_stride, const double* in, double* out) {
-    hipLaunchKernelGGL(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
-                       a.use_inline, stripes, in_stripes, out_stride, in, out);
+hipError_t launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
+                           uint32_t out_stride, const double* in, double* out) {
+    return launch_kernel(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
+                         a.use_inline, stripes, in_stripes, out_stride, in, out);
 }
 // One instantiation per row width 4 + K, K = 1..16.
-void finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
-              uint32_t out_stride, const double* in, double* out) {
+hipError_t finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
+                    uint32_t out_stride, const double* in, double* out) {
     switch (ns) {
-#define JABAS_FIN(n) case n: launch_finalize<n>(grid, stream, a, stripes, in_stripes, out_stride, in, out); break;
+#define JABAS_FIN(n) case n: return launch_finalize<n>(grid, stream, a, stripes, in_stripes, out_stride, in, out);
         JABAS_FIN(5) JABAS_FIN(6) JABAS_FIN(7) JABAS_FIN(8) JABAS_FIN(9) JABAS_FIN(10) JABAS_FIN(11) JABAS_FIN(12)
         JABAS_FIN(13) JABAS_FIN(14) JABAS_FIN(15) JABAS_FIN(16) JABAS_FIN(17) JABAS_FIN(18) JABAS_FIN(19) JABAS_FIN(20)
 #undef JABAS_FIN
-        default: break;
+        default: return hipErrorInvalidValue;
     }
 }
 
@@ -340,14 +340,16 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
     if (stats) {
         const uint32_t st = stripes_for(max_span_chunks);
         const int ns = 4 + s->K;
+        hipError_t err;
         if (st == 1) {
-            finalize(ns, dim3(1, a.n_span), stream, a, 1u, 0u, kStatsStride, a.partials, stats_out);
+            err = finalize(ns, dim3(1, a.n_span), stream, a, 1u, 0u, kStatsStride, a.partials, stats_out);
         } else {
             double* level2 = a.partials + static_cast<uint64_t>(a.n_chunks) * ns;
-            finalize(ns, dim3(st, a.n_span), stream, a, st, 0u, static_cast<uint32_t>(ns), a.partials, level2);
-            finalize(ns, dim3(1, a.n_span), stream, a, 0u, st, kStatsStride, level2, stats_out);
+            err = finalize(ns, dim3(st, a.n_span), stream, a, st, 0u, static_cast<uint32_t>(ns), a.partials, level2);
+            if (err == hipSuccess)
+                err = finalize(ns, dim3(1, a.n_span), stream, a, 0u, st, kStatsStride, level2, stats_out);
         }
-        if (hipGetLastError() != hipSuccess) return JABAS_ERR_LAUNCH;
+        if (err != hipSuccess) return JABAS_ERR_LAUNCH;
     }
     return JABAS_OK;
 }
@@ -662,9 +664,9 @@ JABAS_API int jabas_clip_coef(const double* stats_rows, uint32_t n_rows, double 
     if (n_rows < 1) return JABAS_ERR_SIZE;
     if (!(max_norm > 0.0) || eps < 0.0) return JABAS_ERR_OPT;
     if (reinterpret_cast<uintptr_t>(stats_rows) % 8 || reinterpret_cast<uintptr_t>(coef_out) % 4) return JABAS_ERR_ALIGN;
-    hipLaunchKernelGGL(clip_coef_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), stats_rows, n_rows,
-                       max_norm, eps, coef_out);
-    return hipGetLastError() == hipSuccess ? JABAS_OK : JABAS_ERR_LAUNCH;
+    const hipError_t err = launch_kernel(clip_coef_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                                         stats_rows, n_rows, max_norm, eps, coef_out);
+    return err == hipSuccess ? JABAS_OK : JABAS_ERR_LAUNCH;
 }
 
 JABAS_API int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t numel, double lr,

@@ -422,8 +422,8 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
 #define JABAS_IDLE_LDS_BYTES 32768u
 #endif
     constexpr unsigned idle = (OPT == OPT_ADAM && !STATS && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
-    hipLaunchKernelGGL((fused_kernel<K, DT, OPT, STATS>), dim3(grid), dim3(launch_block(K, DT, OPT, STATS)), idle, stream, a);
-    return static_cast<int>(hipGetLastError());
+    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, STATS>, dim3(grid), dim3(launch_block(K, DT, OPT, STATS)),
+                                          idle, stream, a));
 }
 
 }  // namespace

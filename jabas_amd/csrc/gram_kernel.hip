@@ -108,10 +108,8 @@ __global__ void __launch_bounds__(64) gram_finalize_kernel(int K, const double* 
 template <int K>
 int launch_gram_k(int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
     if (grad_dtype == JABAS_BF16)
-        hipLaunchKernelGGL((gram_kernel<K, JABAS_BF16>), dim3(grid), dim3(kBlock), 0, stream, sp, partials);
-    else
-        hipLaunchKernelGGL((gram_kernel<K, JABAS_F32>), dim3(grid), dim3(kBlock), 0, stream, sp, partials);
-    return static_cast<int>(hipGetLastError());
+        return static_cast<int>(launch_kernel(gram_kernel<K, JABAS_BF16>, dim3(grid), dim3(kBlock), 0, stream, sp, partials));
+    return static_cast<int>(launch_kernel(gram_kernel<K, JABAS_F32>, dim3(grid), dim3(kBlock), 0, stream, sp, partials));
 }
 
 }  // namespace
@@ -131,8 +129,7 @@ int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsi
 }
 
 int launch_gram_finalize(int K, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
-    hipLaunchKernelGGL(gram_finalize_kernel, dim3(1), dim3(64), 0, stream, K, partials, grid, gram_out);
-    return static_cast<int>(hipGetLastError());
+    return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(64), 0, stream, K, partials, grid, gram_out));
 }
 
 }  // namespace jabas

@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <tuple>
 #include "jabas_sync.h"
 
 namespace jabas {
@@ -136,6 +138,18 @@ struct KArgs {
 };
 
 #if defined(__HIPCC__)
+// Launch through hipLaunchKernel so that the status is the one of THIS launch: hipGetLastError() would
+// also hand back (and clear) whatever an earlier, unrelated HIP call of the calling thread left behind.
+template <typename... Params, typename... Given>
+inline hipError_t launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t stream,
+                                Given&&... given) {
+    static_assert(sizeof...(Params) == sizeof...(Given), "one argument per kernel parameter");
+    std::tuple<Params...> values(static_cast<Params>(given)...);
+    void* ptrs[sizeof...(Params) > 0 ? sizeof...(Params) : 1];
+    std::apply([&](auto&... v) { size_t i = 0; ((ptrs[i++] = static_cast<void*>(&v)), ...); }, values);
+    return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds_bytes, stream);
+}
+
 // Sum over the 64 lanes of a wave with DPP moves (no LDS traffic); the total lands in
 // lane 63. Pairing order is fixed: lane^1, lane^2, mirror within 8, mirror within 16,
 // row 0->1 and 2->3, rows 0..1 -> 2..3.
