@@ -161,3 +161,30 @@ def test_fused_step_replays_in_a_hip_graph(gpu):
         torch.cuda.synchronize()
         assert torch.isfinite(scratch)
         check(r, step, plan.ws.stats)
+
+
+def test_a_stale_hip_error_of_the_calling_thread_is_not_reported_as_ours(gpu):
+    """An earlier, unrelated HIP call of the thread failed and nobody read its status. The library's
+    launch must report its own status (OK), and leave that stale status where it was."""
+    import ctypes as C
+    from jabas_amd import _lib as L
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipFree.argtypes, hip.hipFree.restype = [C.c_void_p], C.c_int
+    hip.hipGetLastError.restype = C.c_int
+    n = 100000
+    g = [torch.randn(n, device=gpu) for _ in range(2)]
+    out = torch.empty(n, device=gpu)
+    want = O.aggregate([t.cpu() for t in g], (3, 1))
+    ptrs = (C.c_void_p * 2)(g[0].data_ptr(), g[1].data_ptr())
+    w = (C.c_float * 2)(*[float(x) for x in O.batch_weights((3, 1))[0]])
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    lib = L.lib()
+    assert hip.hipFree(C.c_void_p(0x10)) != 0                    # fails, leaves its status in the thread's last-error slot
+    rc = lib.jabas_aggregate(ptrs, 2, L.F32, w, out.data_ptr(), n, stream)
+    stale = hip.hipGetLastError()                                # read (and clear) it before torch sees it
+    assert rc == L.OK
+    assert stale != 0, "the library swallowed the caller's pending HIP status"
+    assert hip.hipGetLastError() == 0
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu().view(torch.int32), want.view(torch.int32))
