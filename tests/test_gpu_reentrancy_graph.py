@@ -1,4 +1,4 @@
-"""Two properties of the C ABI that its callers rely on:
+"""Three properties of the C ABI that its callers rely on:
 
   * it is re-entrant: comm hooks of several replicas call it from different host threads on
     different streams at the same time (reference: one thread and one stream per VSW,
@@ -6,7 +6,9 @@
     the oracle's bits;
   * it only launches kernels (no allocation, no memset, no synchronisation), so a step can be
     captured in a HIP graph and replayed. Each replay is checked against the oracle, with eager work
-    and synchronisations between the replays.
+    and synchronisations between the replays;
+  * a status it returns is the status of its own launch: a HIP error an earlier call of the thread
+    left unread is neither reported as a launch failure nor cleared.
 """
 import threading
 
