@@ -14,11 +14,13 @@
  *   - plain C types only; every buffer is caller-owned device memory;
  *   - no entry point allocates, frees or synchronises the device; all work is queued
  *     on the stream passed in (jabas_stream_t is a hipStream_t);
- *   - the library keeps no mutable global state besides cached device attributes, so
+ *   - the library keeps no mutable global state, so
  *     calls from different threads on different streams do not interfere as long as
  *     they use different workspaces;
  *   - return value: JABAS_OK (0) or a negative JabasStatus; nothing is launched when a
  *     negative status is returned (except JABAS_ERR_LAUNCH, reported after the fact).
+ *     JABAS_ERR_LAUNCH is the return value of this call's own hipLaunchKernel: a HIP
+ *     error an earlier call of the thread left unread is neither reported nor cleared;
  *
  * What each entry point stands in for in the reference is cited beside it
  * (paths relative to the JABAS repository).
@@ -113,7 +115,8 @@ typedef struct JabasGroup {
 typedef struct JabasStepArgs {
     int32_t K;
     int32_t grad_dtype;                 /* JABAS_F32 / JABAS_BF16                      */
-    float   weight[JABAS_MAX_K];        /* w_k = fp32(b_k / B)                         */
+    float   weight[JABAS_MAX_K];        /* w_k = fp32(b_k / B); with A micro-batches summed
+                                           into every bucket, fp32(b_k / (B*A))         */
     int32_t stats;                      /* 0: none, 1: write a stats_out row per span  */
     uint8_t half_id[JABAS_MAX_K];       /* 0 = half A, 1 = half B                      */
     float   half_weight[JABAS_MAX_K];   /* fp32(b_k / sum of b over k's half)          */
