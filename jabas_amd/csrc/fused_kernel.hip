@@ -241,18 +241,40 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
     if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, clip, acc);
 }
 
-// Scalar path for one tile that touches a span edge or a group change. tile_e0 is the
-// (rebased) index of the first element of the tile, j the bound entry covering the
-// first live element of the tile.
+// One tile that touches a span edge or a group change. tile_e0 is the (rebased) index of the first
+// element of the tile, j the bound entry covering the first live element of the tile. Each thread
+// looks at its own four elements: all live and in one parameter group -> the vector path with that
+// group's constants (held per thread); otherwise -> element by element. Only the few threads whose
+// vector straddles the span's first or last element or a bound take the slow way, so such a tile costs
+// little more than a full one (ResNet-50's batch-norm tensors and ViT's biases put a group change
+// into roughly every hundredth tile; one span per tensor puts an edge into every tensor).
 template <int K, int DT, int OPT, bool STATS>
 __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const KArgs& a, uint32_t j,
                                              float clip, double (&acc)[NStats<K, STATS>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
+    constexpr int BS = launch_block(K, DT, OPT, STATS);
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     const BoundDev* bd = sp.bound_count ? a.bounds + sp.bound_begin : nullptr;
     const uint64_t e_first = tile_e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
+    const bool all_live = e_first >= sp.lo && e_first + EPT <= sp.hi;
+    bool one_group = true;
+    uint32_t gid_first = 0;
+    if (bd && all_live) {
+        const uint64_t rel = e_first - sp.lo;
+        uint32_t jj = j;
+        while (jj + 1 < sp.bound_count && bd[jj + 1].start <= rel) ++jj;
+        gid_first = bd[jj].group & (JABAS_MAX_GROUPS - 1);
+        one_group = jj + 1 >= sp.bound_count || bd[jj + 1].start >= rel + EPT;
+    }
+    if (all_live && one_group) {
+        const GroupDev G = a.groups[gid_first];
+        TileRegs<K, DT, 1> r;
+        issue_loads<K, DT, OPT, 1, BS>(r, sp, e_first, load_s1);
+        consume<K, DT, OPT, STATS, false, 1>(r, sp, e_first, a, G, clip, use_s1, load_s1, acc);   // halves from the mask: always right
+        return;
+    }
     for (int i = 0; i < EPT; ++i) {
         const uint64_t e = e_first + i;
         if (e < sp.lo || e >= sp.hi) continue;
