@@ -77,7 +77,12 @@ enum {
  * indexed alike. Element e of every fp32 buffer must fall at the same position of a
  * 16-byte line, and of every bf16 gradient buffer at the same position of an 8-byte line
  * ((address / element size) mod 4 equal for all buffers), which holds whenever they are
- * views at one element offset into 16-byte aligned arenas.
+ * views at one element offset into 16-byte aligned arenas. That much is required
+ * (JABAS_ERR_ALIGN otherwise). Spans run fastest when the same holds within 64 elements
+ * ((address / element size) mod 64 equal for all buffers: views at one element offset into
+ * 256-byte aligned arenas, which allocators of device memory give): the launch then starts its
+ * element grid at that 256-byte line and moves whole cache lines; spans that start at arbitrary
+ * elements lose 8-17 % of the rate without it.
  * agg_out may be exactly one of the fp32 gradient buffers (in-place bucket update); apart
  * from that every written buffer (agg_out, param, state1, state2, fanout) must be disjoint
  * from every other buffer of the span, else JABAS_ERR_ALIAS. Overlap between different

@@ -71,7 +71,8 @@ __host__ __device__ constexpr int ept_of(int /*grad_dtype*/) { return 4; }
 __host__ __device__ constexpr int tile_elems_of(int block) { return block * 4; }
 
 // A span as the kernels see it. Pointers are rebased downwards by `lo` elements so that
-// element index 0 of every buffer is 16-byte aligned; [lo, hi) is the live range.
+// element index 0 of every buffer is 16-byte aligned (256-byte aligned when the buffers allow
+// it, lo < 64 then, else lo < 4); [lo, hi) is the live range. Nothing below `lo` is accessed.
 struct SpanDev {
     const void* g[JABAS_MAX_K];
     float* out;

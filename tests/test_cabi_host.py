@@ -95,6 +95,26 @@ def test_plan_encode_counts_chunks():
     assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == 3
 
 
+def test_plan_encode_starts_the_element_grid_at_a_256_byte_line_when_all_buffers_allow_it():
+    """2048 elements per workgroup here (K = 2, no optimizer). With every buffer 61 elements into a
+    256-byte line the grid starts at that line: 61 + 4036 elements still fit two workgroups, one
+    more element does not. With one buffer elsewhere in its 256-byte line (but at the same place of
+    its 16-byte line) the grid starts at the first element's 16-byte line, 1 element in."""
+    lib = L.lib()
+    for numel, want in ((4096 - 61, 2), (4096 - 60, 3)):
+        rc, blob, _ = _encode([_span(numel, skew=61)])
+        assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == want
+    for numel, want in ((4096 - 60, 2), (4095, 2), (4096, 3)):
+        s = _span(numel, skew=61)
+        s.agg_out -= 16 * 4                  # 45 elements in: congruent mod 4, not mod 64
+        rc, blob, _ = _encode([s])
+        assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == want
+    # the bound jabas_plan_bytes and jabas_sync_workspace_bytes are sized by holds in either case
+    rc, blob, nbytes = _encode([_span(1, skew=63), _span(2048 - 63, skew=63), _span(2048 - 62, skew=63)])
+    assert rc == L.OK and lib.jabas_plan_chunks(blob.ctypes.data, 0) == 1 + 1 + 2
+    assert lib.jabas_sync_workspace_bytes(2048 - 62, L.F32) >= 3 * L.STATS_STRIDE * 8
+
+
 def test_plan_encode_bf16_positions_are_counted_in_elements():
     # bf16 gradients 2 elements into an 8-byte line, fp32 buffers 2 elements into a 16-byte line: congruent
     rc, _, _ = _encode([_span(5000, gs=2, skew=2)], dtype=L.BF16)

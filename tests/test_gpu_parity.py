@@ -46,7 +46,7 @@ def _host_state(n, seed, scale=0.05):
 
 def _dev(t, gpu, skew=0):
     """Device copy of t placed `skew` elements into a 256-byte aligned allocation."""
-    buf = torch.zeros(t.numel() + 16, dtype=t.dtype, device=gpu)
+    buf = torch.zeros(t.numel() + 128, dtype=t.dtype, device=gpu)
     view = buf[skew:skew + t.numel()]
     view.copy_(t)
     return view
@@ -253,6 +253,47 @@ def test_sync_bucket_fused(gpu, K, dtype, opt):
     same, tot = _same_bits(p_d, p_h)
     print(f"fused bucket K={K} {dtype} {opt['kind']}: {same}/{tot} weights bit-identical")
     assert same == tot
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("skews", [
+    "37 for every buffer",                # one offset within 256 bytes: the launch's element grid starts at that line
+    "differs within 256 bytes",           # equal only within 16 bytes: the grid starts at the first element's 16-byte line
+    "63 for every buffer", "60 for every buffer"])
+def test_sync_bucket_buffer_offsets_within_a_256_byte_line(gpu, dtype, skews):
+    """Where the launch's element grid starts depends on how the buffers sit relative to 256-byte
+    lines; the results must not."""
+    from jabas_amd import sync
+    K, n = 3, 150001
+    bounds = ((0, 1), (3, 0), (61, 1), (1024, 0), (99999, 1))
+    if skews.endswith("for every buffer"):
+        sk = [int(skews.split()[0])] * 8
+    else:
+        sk = [5, 9, 61, 33, 1, 17, 49, 13]             # all 1 mod 4
+    hg = _host_grads(K, n, 300, std=5e-4, dtype=dtype)
+    p_h, s1_h, s2_h = _host_state(n, 6), torch.zeros(n), torch.zeros(n)
+    dg = [_dev(t, gpu, sk[k]) for k, t in enumerate(hg)]
+    agg_d = _dev(torch.zeros(n), gpu, sk[3])
+    p_d, s1_d, s2_d = _dev(p_h, gpu, sk[4]), _dev(s1_h, gpu, sk[5]), _dev(s2_h, gpu, sk[6])
+    fan = [_dev(torch.zeros(n), gpu, sk[7])]
+    guard = [t._base if t._base is not None else t for t in dg + [agg_d, p_d, s1_d, s2_d] + fan]
+    before = [(b[:sk_i].clone(), b[sk_i + n:].clone()) for b, sk_i in zip(guard, sk)]
+    span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d, state1=s1_d, state2=s2_d, fanout=fan, bounds=bounds)
+    ws = sync.Workspace.for_span(n, dtype, gpu)
+    for step in (1, 2):
+        args = sync.make_step_args(BATCHES[K], dtype, stats=True, opt=ADAMW, step=step, first_step=(step == 1))
+        row = sync.sync_bucket(span, args, workspace=ws)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg, BATCHES[K], [(0, n, bounds)], ADAMW, p_h, s1_h, s2_h, step=step,
+                                    first_step=(step == 1), want_stats=True)
+        assert torch.equal(_bits(agg_d), _bits(agg_h)), step
+        rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        assert _close(row.cpu()[:4 + K], rows_h[0][:4 + K], rtol, 1e-30)[0]
+        for got, want in ((p_d, p_h), (s1_d, s1_h), (s2_d, s2_h), (fan[0], p_h)):
+            assert torch.equal(_bits(got), _bits(want)), step
+    # nothing outside the live range was written
+    for b, sk_i, (head, tail) in zip(guard, sk, before):
+        assert torch.equal(b[:sk_i], head) and torch.equal(b[sk_i + n:], tail)
 
 
 # ---------------------------------------------------------------- fused, multi-span plan
