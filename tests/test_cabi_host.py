@@ -322,3 +322,32 @@ def test_launch_shape_follows_what_the_plan_is_encoded_for():
     args.opt_kind, args.n_groups = L.OPT_ADAM, 1
     args.groups[0].step = 1
     assert lib.jabas_sync_fused(blob.ctypes.data, 0x1000, C.byref(args), None, None, 0, None) == L.ERR_PLAN
+
+
+def test_product_paths_fail_when_the_library_is_missing(tmp_path):
+    """No CPU fallback: with no shared library the loader raises, and product entries given host
+    tensors refuse them or raise the loader's error; none computes anything (checked in a child
+    process so that this process keeps its loaded library)."""
+    import subprocess
+    import sys
+    code = """
+import torch
+from jabas_amd import _lib, sync
+from jabas_amd.local_sync import LocalBucketSync
+g = [torch.ones(8), torch.ones(8)]
+for name, call in (("lib", lambda: _lib.lib()),
+                   ("aggregate", lambda: sync.aggregate(g, (1, 1))),
+                   ("gradient_stats", lambda: sync.gradient_stats(g, (1, 1))),
+                   ("plan", lambda: sync.SyncPlan([sync.SpanSpec(g, agg_out=torch.zeros(8))], _lib.OPT_NONE))):
+    try:
+        call()
+    except (RuntimeError, ValueError) as exc:
+        assert "no CPU fallback" in str(exc) or (name != "lib" and "must live on the GPU" in str(exc)), (name, exc)
+    else:
+        raise SystemExit(name + " did not raise")
+print("all raised")
+"""
+    env = dict(os.environ, JABAS_SYNC_LIB=str(tmp_path / "absent.so"))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and "all raised" in res.stdout, res.stdout + res.stderr
