@@ -69,7 +69,8 @@ def _same_bits(a, b):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_aggregate_bit_exact(gpu, K, dtype):
     from jabas_amd import sync
-    for n, skew in ((1, 0), (3, 1), (1023, 0), (1024, 2), (1025, 3), (4099, 0), (262144 + 77, 0), (1 << 20, 3)):
+    for n, skew in ((1, 0), (3, 1), (1023, 0), (1024, 2), (1025, 3), (4099, 0), (262144 + 77, 0), (1 << 20, 3),
+                    (4099, 37), (70001, 63), (5, 61)):
         print(f"aggregate K={K} {dtype} n={n} skew={skew}", flush=True)
         hg = _host_grads(K, n, K + n % 7, dtype=dtype)
         dg = [_dev(t, gpu, skew) for t in hg]
@@ -110,7 +111,7 @@ def test_aggregate_keeps_zero_rows_exactly_zero(gpu):
 @pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-6), (torch.bfloat16, 1e-2)])
 def test_stats_row(gpu, K, dtype, rtol):
     from jabas_amd import sync
-    for n, skew in ((5, 0), (4099, 1), (300007, 0), (1 << 21, 2)):
+    for n, skew in ((5, 0), (4099, 1), (300007, 0), (1 << 21, 2), (4099, 45), (3, 63)):
         print(f"stats K={K} {dtype} n={n} skew={skew}", flush=True)
         hg = _host_grads(K, n, 20 + K, std=5e-4, dtype=dtype)
         row = sync.gradient_stats([_dev(t, gpu, skew) for t in hg], BATCHES[K])
@@ -147,7 +148,7 @@ def test_stats_cosine_identities(gpu):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gram(gpu, K, dtype):
     from jabas_amd import sync
-    for n, skew in ((7, 0), (100003, 2), (1 << 20, 0)):
+    for n, skew in ((7, 0), (100003, 2), (1 << 20, 0), (100003, 61)):
         hg = _host_grads(K, n, 30 + K, dtype=dtype)
         G = sync.gram([_dev(t, gpu, skew) for t in hg]).cpu()
         want = O.gram(hg)
