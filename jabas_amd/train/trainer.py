@@ -243,6 +243,102 @@ class VSWSyncTrainer:
         self.similarity_state.subgroup_total_num_decoupled_workers = workers / 2
         torch.cuda.synchronize(self.gpu)
 
+    # ---------------------------------------------------------------- checkpoint / resume
+    def state_dict(self):
+        """What the sync path needs to resume (the reference checkpoints its trainer through
+        ``save`` / ``load``, jabas/train/trainer.py:105-170): the main VSW's weights and buffers, the
+        optimizer state in torch's own ``Optimizer.state_dict()`` format (so a stock torch optimizer
+        can load it, and the other way round), scheduler state, the step counters, the set of VSWs
+        and the learning-rate modifier. Tensors are copies, not views of the arenas."""
+        if self.engine is None:
+            raise RuntimeError("nothing to save before the weight-sync method is prepared")
+        torch.cuda.synchronize(self.gpu)
+        eng = self.engine
+        out = {
+            "model": {k: v.detach().clone() for k, v in self.main_model.state_dict().items()},
+            "sync_step": self.sync_step,
+            "engine_step": eng.step_count,
+            "similarity_step": self.similarity_state.step,
+            "global_lr_modifier": self.global_lr_modifier,
+            "local_batch_sizes": tuple(self.local_batch_sizes),
+            "schedulers": [sch.state_dict() for sch in self.local_schedulers],
+        }
+        if self.main_optimizer is not None:
+            sd = self.main_optimizer.state_dict()
+            sd["state"] = {idx: {k: (v.detach().clone() if torch.is_tensor(v) else v) for k, v in st.items()}
+                           for idx, st in sd["state"].items()}
+            out["optimizer"] = sd
+        else:
+            out["optimizer_arenas"] = {
+                "numel": eng.layout.total,
+                "state1": None if eng.state1 is None else eng.state1.detach().clone(),
+                "state2": None if eng.state2 is None else eng.state2.detach().clone(),
+                "groups": [dict(g) for g in self.opt["groups"]],
+            }
+        return out
+
+    def load_state_dict(self, state):
+        """Resumes from ``state_dict()`` (or from a dictionary with the ``model`` and ``optimizer``
+        entries of a plain torch training run). Weights and optimizer state are copied into the
+        arenas, every replica restarts from the main weights, and the set of VSWs follows the saved
+        one. The next step continues bit for bit where the saved run would have."""
+        if self.engine is None:
+            raise RuntimeError("prepare the weight-sync method before loading a checkpoint")
+        torch.cuda.synchronize(self.gpu)
+        saved_batches = tuple(state.get("local_batch_sizes", self.local_batch_sizes))
+        if saved_batches != tuple(self.local_batch_sizes):
+            if len(set(saved_batches)) != 1:
+                raise ValueError(f"cannot resume onto unequal local batch sizes {saved_batches}")
+            self._change_local_models_state(len(saved_batches), saved_batches[0])
+        eng = self.engine
+        for m in self.local_models:                     # in-place copies: the parameters stay views of the arenas
+            m.load_state_dict(state["model"])
+        if "optimizer" in state:
+            if self.main_optimizer is None:
+                raise ValueError("the checkpoint holds a torch optimizer's state; hand the optimizer over through "
+                                 "prepare_weight_sync_method first")
+            self.main_optimizer.load_state_dict(state["optimizer"])     # fresh tensors in optimizer.state ...
+            steps, has_momentum = set(), False
+            for i, p in enumerate(self.main_model.parameters()):        # ... copied into the arenas
+                st = self.main_optimizer.state.get(p, {})
+                for key, arena in (("momentum_buffer", eng.state1), ("exp_avg", eng.state1), ("exp_avg_sq", eng.state2)):
+                    if arena is not None and st.get(key) is not None:
+                        eng._view(arena, i).copy_(st[key].reshape(-1))
+                        has_momentum = has_momentum or key == "momentum_buffer"
+                if "step" in st:
+                    steps.add(int(float(st["step"])))
+            if len(steps) > 1:
+                raise ValueError(f"parameters at different step counts {sorted(steps)}: one fused launch cannot mirror that")
+            if "engine_step" in state:
+                eng.step_count = int(state["engine_step"])
+            else:       # a plain torch checkpoint: Adam's own count; SGD keeps none, but a stored momentum buffer means a step was taken
+                eng.step_count = steps.pop() if steps else (1 if has_momentum else 0)
+            self.opt["groups"] = [dict(lr=float(g["lr"]), weight_decay=float(g.get("weight_decay", 0.0)))
+                                  for g in self.main_optimizer.param_groups]
+            self._step_tensor = torch.full((), float(eng.step_count), dtype=torch.float32)
+            self._expose_state(self.main_optimizer)
+        elif "optimizer_arenas" in state:
+            arenas = state["optimizer_arenas"]
+            if arenas["numel"] != eng.layout.total:
+                raise ValueError("the checkpoint's state arenas belong to another layout")
+            for mine, theirs in ((eng.state1, arenas["state1"]), (eng.state2, arenas["state2"])):
+                if (mine is None) != (theirs is None):
+                    raise ValueError("the checkpoint's optimizer keeps other state than this one")
+                if mine is not None:
+                    mine.copy_(theirs)
+            for mine, theirs in zip(self.opt["groups"], arenas["groups"]):
+                mine.update(theirs)
+            eng.step_count = int(state.get("engine_step", 0))
+        for sch, sd in zip(self.local_schedulers, state.get("schedulers", [])):
+            sch.load_state_dict(sd)
+        self.sync_step = int(state.get("sync_step", eng.step_count))
+        self.similarity_state.step = int(state.get("similarity_step", self.sync_step))
+        self.global_lr_modifier = float(state.get("global_lr_modifier", 1.0))
+        self.accumulated = 0
+        for g in eng.grads:
+            g.zero_()
+        torch.cuda.synchronize(self.gpu)
+
     # ------------------------------------------------------------------- one iteration
     def compute(self, data):
         """data: one (input, target) pair per VSW, already on the GPU. May be called several times

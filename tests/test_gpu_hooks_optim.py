@@ -352,3 +352,76 @@ def test_trainer_accumulates_micro_batches_between_steps(gpu):
         assert trainer.accumulated == 0
         for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
             assert _close(p, rp, 1e-6, 1e-7), step
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
+    """state_dict() after 3 steps, through a file, into a fresh trainer (other initial weights, another
+    number of VSWs): the next 3 steps give the bits of the uninterrupted run. The optimizer entry is in
+    torch's own format: a stock torch optimizer loads it."""
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (4, 4, 4)
+    crit = torch.nn.MSELoss()
+
+    def make(seed, n_vsw):
+        t = VSWSyncTrainer(gpu, (4,) * n_vsw, interval=2)
+        t.prepare_stream_parallel(_mlp(seed), crit)
+        if kind == "sgd":
+            o = torch.optim.SGD(_groups(t.main_model), lr=0.05, momentum=0.9, foreach=False)
+        else:
+            o = torch.optim.AdamW(_groups(t.main_model), lr=1e-3, foreach=False)
+        sch = torch.optim.lr_scheduler.LambdaLR(o, lambda it: 1.0 / (1.0 + 0.25 * it))
+        t.prepare_weight_sync_method(o, sch)
+        return t, o
+
+    def run(t, first, last):
+        for step in range(first, last + 1):
+            gen = torch.Generator().manual_seed(900 + step)
+            data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu))
+                    for b in batches]
+            t.compute(data)
+            t.step()
+        torch.cuda.synchronize()
+
+    a, opt_a = make(21, 3)
+    run(a, 1, 3)
+    path = tmp_path / "trainer.pth"
+    torch.save(a.state_dict(), path)
+    run(a, 4, 6)
+
+    b, opt_b = make(22, 2)                                # other weights, 2 VSWs: both replaced by the checkpoint
+    b.load_state_dict(torch.load(path, map_location=gpu, weights_only=True))
+    assert b.num_models == 3 and b.sync_step == 3 and b.engine.step_count == 3
+    base_lr = 0.05 if kind == "sgd" else 1e-3
+    assert opt_b.param_groups[0]["lr"] == pytest.approx(base_lr / (1.0 + 0.25 * 3), rel=1e-12)
+    run(b, 4, 6)
+    assert b.sync_step == a.sync_step == 6
+    for pa, pb in zip(a.main_model.parameters(), b.main_model.parameters()):
+        assert torch.equal(pa.detach().view(torch.int32), pb.detach().view(torch.int32))
+    for m in b.local_models[1:]:
+        for pm, pb in zip(m.parameters(), b.main_model.parameters()):
+            assert torch.equal(pm, pb)
+    keys = ("momentum_buffer",) if kind == "sgd" else ("exp_avg", "exp_avg_sq")
+    for pa, pb in zip(a.main_model.parameters(), b.main_model.parameters()):
+        for key in keys:
+            assert torch.equal(opt_a.state[pa][key], opt_b.state[pb][key])
+            arena = b.engine.state2 if key == "exp_avg_sq" else b.engine.state1      # still views of the arenas
+            assert opt_b.state[pb][key].untyped_storage().data_ptr() == arena.untyped_storage().data_ptr()
+    assert opt_a.param_groups[0]["lr"] == opt_b.param_groups[0]["lr"]
+
+    # a stock torch optimizer over a plain copy of the model takes the optimizer entry as it is
+    plain = _mlp(5).to(gpu)
+    plain.load_state_dict(b.state_dict()["model"])
+    stock = (torch.optim.SGD(_groups(plain), lr=0.05, momentum=0.9) if kind == "sgd"
+             else torch.optim.AdamW(_groups(plain), lr=1e-3))
+    stock.load_state_dict(b.state_dict()["optimizer"])
+    for pp, pb in zip(plain.parameters(), b.main_model.parameters()):
+        assert torch.equal(stock.state[pp][keys[0]], opt_b.state[pb][keys[0]])
+
+    # and the other way round: a checkpoint of a plain torch run (no trainer entries) resumes here
+    c, opt_c = make(23, 3)
+    c.load_state_dict({"model": plain.state_dict(), "optimizer": stock.state_dict()})
+    assert c.engine.step_count == (1 if kind == "sgd" else 6)
+    for pc, pb in zip(c.main_model.parameters(), b.main_model.parameters()):
+        assert torch.equal(pc, pb)
+        assert torch.equal(opt_c.state[pc][keys[0]], opt_b.state[pb][keys[0]])
