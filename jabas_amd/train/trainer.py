@@ -383,8 +383,9 @@ class VSWSyncTrainer:
                 sched.step()
         if want:
             self._compute_cosine_similarity(rows)
-        for k in range(self.num_models):
-            self.engine.grads[k].zero_()
+        if self.grad_dtype == torch.float32:            # backward accumulates into the fp32 buckets; reduced-precision
+            for k in range(self.num_models):            # buckets are overwritten by the first compute() of the next step
+                self.engine.grads[k].zero_()
         for s in self.model_streams:
             s.wait_stream(cur)
         if want and self.controller is not None:

@@ -425,3 +425,43 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     for pc, pb in zip(c.main_model.parameters(), b.main_model.parameters()):
         assert torch.equal(pc, pb)
         assert torch.equal(opt_c.state[pc][keys[0]], opt_b.state[pb][keys[0]])
+
+
+def test_trainer_with_bf16_gradient_buckets(gpu):
+    """Reduced-precision buckets (the ViT-L/16 configuration): every VSW's gradient is rounded to bf16
+    into its bucket (added in bf16 on further micro-batches), the aggregate and AdamW run in fp32. The
+    buckets are not cleared between steps: the first micro-batch of a step overwrites them."""
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (6, 2)
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, interval=1, grad_dtype=torch.bfloat16)
+    trainer.prepare_stream_parallel(_mlp(31), crit)
+    mine = torch.optim.AdamW(_groups(trainer.main_model), lr=2e-3, foreach=False)
+    trainer.prepare_weight_sync_method(mine)
+    ref_model = _mlp(31).to(gpu)
+    ref_opt = torch.optim.AdamW(_groups(ref_model), lr=2e-3, foreach=False)
+    for step, micro in ((1, 1), (2, 2), (3, 1)):
+        w, _, _ = O.batch_weights(batches, accumulations=micro)
+        buckets = None
+        for mb in range(micro):
+            gen = torch.Generator().manual_seed(500 + 10 * step + mb)
+            data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu))
+                    for b in batches]
+            trainer.compute(data)
+            fresh = []
+            for x, y in data:
+                ref_model.zero_grad(set_to_none=True)
+                crit(ref_model(x), y).backward()
+                fresh.append([p.grad.detach().to(torch.bfloat16) for p in ref_model.parameters()])
+            buckets = fresh if buckets is None else [[a + b for a, b in zip(old, new)] for old, new in zip(buckets, fresh)]
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(buckets[0][i].float(), w[0]), torch.mul(buckets[1][i].float(), w[1]))
+        ref_opt.step()
+        trainer.step()
+        torch.cuda.synchronize()
+        assert trainer.cos_placeholder is not None and -1.0 <= float(trainer.cos_placeholder) <= 1.0
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), f"step {step}"
+        for m in trainer.local_models[1:]:
+            for pm, p in zip(m.parameters(), trainer.main_model.parameters()):
+                assert torch.equal(pm, p)
