@@ -178,6 +178,8 @@ size_t jabas_plan_workspace_bytes(const void* host_blob);
  * Aggregate + statistics + optimizer (+ fan-out) over every span of a plan, one
  * launch (plus a one-workgroup-per-span finalize launch when args->stats is set).
  * stats_out: n_span * JABAS_STATS_STRIDE doubles (device), required when stats != 0.
+ * A launch with statistics takes a plan of at most 65535 spans (JABAS_ERR_SIZE beyond,
+ * returned before anything is launched); without statistics up to 2^24.
  * Replaces, for one GPU:
  *   - the local aggregation of the K VSW buckets inside IIDPTrainer.compute()/step()
  *     and iidp_allreduce_hook's division by the worker count

@@ -255,6 +255,7 @@ constexpr int kFinalizeBlock = 256;
 constexpr uint32_t kStripeRows = 512;        // chunk rows one workgroup sums in the striped launch
 constexpr uint32_t kMaxStripes = 32;
 constexpr uint32_t kSingleLaunchRows = 2560; // up to here one workgroup per span finishes in about 6 us
+constexpr uint32_t kMaxStatsSpans = 65535;   // spans index the y dimension of the finalize grid
 template <int NS>
 __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const uint32_t* chunk_prefix, uint32_t n_chunks,
                                                                         uint32_t use_inline, uint32_t stripes,
@@ -344,6 +345,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
     const int stats = s->stats ? 1 : 0;
     if (stats) {
         if (!stats_out) return JABAS_ERR_NULL;
+        if (a.n_span > kMaxStatsSpans) return JABAS_ERR_SIZE;     // before anything is launched: no half-done step
         if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
         if (workspace_bytes < workspace_rows(a.n_chunks, a.n_span) * kStatsStride * sizeof(double)) return JABAS_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(stats_out) % 8) return JABAS_ERR_ALIGN;

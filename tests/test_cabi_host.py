@@ -351,3 +351,30 @@ print("all raised")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0 and "all raised" in res.stdout, res.stdout + res.stderr
+
+
+def test_statistics_over_too_many_spans_are_refused_before_any_launch():
+    """The finalize launch indexes spans by a grid dimension of 16 bits; a plan beyond that must be
+    turned down with a status, not fail after the weights have moved."""
+    lib = L.lib()
+    n_span = 65536
+    arr = (L.JabasSpan * n_span)()
+    base = 0x7f0000000000
+    for i in range(n_span):
+        arr[i].grads[0] = base + 4096 * i
+        arr[i].grads[1] = base + (1 << 36) + 4096 * i
+        arr[i].agg_out = base + (2 << 36) + 4096 * i
+        arr[i].numel = 8
+    nbytes = lib.jabas_plan_bytes(arr, n_span, 0, L.F32)
+    blob = np.zeros(nbytes // 8 + 1, dtype=np.uint64)
+    assert lib.jabas_plan_encode(arr, n_span, None, 0, 2, L.F32, L.OPT_NONE, blob.ctypes.data, nbytes) == L.OK
+    args = L.JabasStepArgs()
+    args.K, args.grad_dtype, args.opt_kind, args.stats = 2, L.F32, L.OPT_NONE, 1
+    args.weight[0] = args.weight[1] = 0.5
+    args.half_id[1] = 1
+    args.half_weight[0] = args.half_weight[1] = 1.0
+    fake_dev = 0x7e0000000000
+    ws_bytes = lib.jabas_plan_workspace_bytes(blob.ctypes.data)
+    rc = lib.jabas_sync_fused(blob.ctypes.data, fake_dev, C.byref(args), fake_dev + (1 << 30), fake_dev + (2 << 30),
+                              ws_bytes, None)
+    assert rc == L.ERR_SIZE
