@@ -378,3 +378,82 @@ def test_statistics_over_too_many_spans_are_refused_before_any_launch():
     rc = lib.jabas_sync_fused(blob.ctypes.data, fake_dev, C.byref(args), fake_dev + (1 << 30), fake_dev + (2 << 30),
                               ws_bytes, None)
     assert rc == L.ERR_SIZE
+
+
+def _shape_model(K, dtype, opt_class, stats):
+    """(threads per workgroup, tiles per workgroup) as documented for the launch shapes."""
+    if stats or opt_class == 0:
+        block = 256
+    elif K > 4:
+        block = 512
+    else:
+        block = 128 if (opt_class == 1 and dtype == L.F32) else 256
+    if K > 4:
+        tiles = 4 if (stats or opt_class == 0) else 1
+    else:
+        tiles = 2
+    return block, tiles
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
+    """Random spans at random addresses: the encoder's verdict (OK / JABAS_ERR_ALIGN) and its chunk
+    counts for both launch shapes must equal an independent statement of the rule: buffers must agree
+    within 4 elements; the element grid starts at the 256-byte line when they agree within 64 elements,
+    else at the 16-byte line; a span takes ceil(ceil((skew + numel) / tile) / tiles_per_workgroup) chunks."""
+    rng = np.random.RandomState(seed)
+    lib = L.lib()
+    K = int(rng.randint(1, 17))
+    dtype = L.BF16 if rng.rand() < 0.4 else L.F32
+    opt = [L.OPT_NONE, L.OPT_SGD, L.OPT_ADAM, L.OPT_ADAMW][int(rng.randint(0, 4))]
+    opt_class = {L.OPT_NONE: 0, L.OPT_SGD: 1, L.OPT_ADAM: 2, L.OPT_ADAMW: 2}[opt]
+    gs = 2 if dtype == L.BF16 else 4
+    n_span = int(rng.randint(1, 12))
+    spans, want_chunks, want_rc = [], [0, 0], L.OK
+    stride = 1 << 36
+    for i in range(n_span):
+        numel = int(rng.choice([0, 1, 3, 500, 1023, 1024, 1025, 4096, 4097, 70000, 1 << 20])) + int(rng.randint(0, 3))
+        mode = rng.rand()
+        base_off = int(rng.randint(0, 64))
+        n_buf = K + 4
+        if mode < 0.6:
+            offs = [base_off] * n_buf                                   # one place within the 256-byte line
+        elif mode < 0.9:
+            offs = [base_off % 4 + 4 * int(rng.randint(0, 16)) for _ in range(n_buf)]   # agree within 16 bytes only
+        else:
+            offs = [int(rng.randint(0, 64)) for _ in range(n_buf)]      # arbitrary
+        s = L.JabasSpan()
+        region = (2 * i + 1) * (1 << 28)                                # spans far apart: no overlap between buffers
+        for k in range(K):
+            s.grads[k] = 0x700000000000 + k * stride + region + offs[k] * gs
+        s.agg_out = 0x700000000000 + 16 * stride + region + offs[K] * 4
+        used = offs[:K + 1]
+        if opt_class:
+            s.param = 0x700000000000 + 17 * stride + region + offs[K + 1] * 4
+            s.state1 = 0x700000000000 + 18 * stride + region + offs[K + 2] * 4
+            used = offs[:K + 3]
+            if opt_class == 2:
+                s.state2 = 0x700000000000 + 19 * stride + region + offs[K + 3] * 4
+                used = offs[:K + 4]
+        s.numel = numel
+        spans.append(s)
+        if numel == 0:
+            continue
+        if len({o % 4 for o in used}) != 1:
+            want_rc = L.ERR_ALIGN
+            continue
+        skew = used[0] if len(set(used)) == 1 else used[0] % 4
+        for v, stats in enumerate((False, True)):
+            block, tiles = _shape_model(K, dtype, opt_class, stats)
+            te = block * 4
+            want_chunks[v] += -(-(-(-(skew + numel) // te)) // tiles)
+    arr = (L.JabasSpan * n_span)(*spans)
+    nbytes = lib.jabas_plan_bytes(arr, n_span, 0, dtype)
+    blob = np.zeros(nbytes // 8 + 1, dtype=np.uint64)
+    rc = lib.jabas_plan_encode(arr, n_span, None, 0, K, dtype, opt, blob.ctypes.data, nbytes)
+    if want_rc != L.OK:
+        assert rc == L.ERR_ALIGN
+        return
+    assert rc == L.OK, rc
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == want_chunks[0]
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == want_chunks[1]
