@@ -1,8 +1,8 @@
 // K x K Gram matrix of the K worker gradients of one span: gram[a][b] = sum_e g_a[e]*g_b[e].
 // fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums. Grid-stride over 4-element
 // vectors, K(K+1)/2 accumulators per thread, wave64 shuffle tree -> LDS -> one packed
-// partial row per workgroup, then a single-workgroup finalize that sums the rows in
-// workgroup order and mirrors the lower triangle.
+// partial row per workgroup, then a single-workgroup finalize that sums the rows in a fixed
+// order and mirrors the lower triangle.
 #include "jabas_internal.h"
 
 namespace jabas {
@@ -90,19 +90,38 @@ __global__ void __launch_bounds__(kBlock) gram_kernel(const SpanDev sp, double* 
     }
 }
 
-__global__ void __launch_bounds__(64) gram_finalize_kernel(int K, const double* partials, unsigned grid, double* gram_out) {
+// Sums the workgroup rows and writes the symmetric matrix. 256 threads: thread (value, part) adds rows
+// part, part + 16, ... of one packed entry in increasing order, the 16 parts of an entry sit in one
+// 16-lane row and are combined by a fixed DPP pattern, so the result does not depend on timing. (One
+// wave walking all rows of its entry one after the other took 0.23 ms for 1024 rows: more than the
+// Gram kernel itself.)
+constexpr int kGramFinalizeBlock = 256;
+__global__ void __launch_bounds__(kGramFinalizeBlock) gram_finalize_kernel(int K, const double* partials, unsigned grid,
+                                                                         double* gram_out) {
     const int np = K * (K + 1) / 2;
     const int t = threadIdx.x;
-    gram_out[t] = 0.0;                       // JABAS_GRAM_STRIDE == 64 == blockDim.x
+    if (t < JABAS_GRAM_STRIDE) gram_out[t] = 0.0;
     __syncthreads();
-    if (t >= np) return;
-    double s = 0.0;
-    for (unsigned b = 0; b < grid; ++b) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + t];
-    int a = 0;
-    while ((a + 1) * (a + 2) / 2 <= t) ++a;  // packed index t = a*(a+1)/2 + b, b <= a
-    const int b = t - a * (a + 1) / 2;
-    gram_out[a * JABAS_GRAM_MAX_K + b] = s;
-    gram_out[b * JABAS_GRAM_MAX_K + a] = s;
+    const int part = t & 15;
+    for (int v0 = 0; v0 < np; v0 += kGramFinalizeBlock / 16) {
+        const int v = v0 + (t >> 4);
+        double s = 0.0;
+        if (v < np) {
+#pragma unroll 8
+            for (unsigned b = part; b < grid; b += 16) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + v];
+        }
+        s += dpp_move<0xB1, 0xf>(s);     // quad_perm [1,0,3,2]
+        s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
+        s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
+        s += dpp_move<0x140, 0xf>(s);    // row_mirror
+        if (v < np && part == 0) {
+            int a = 0;
+            while ((a + 1) * (a + 2) / 2 <= v) ++a;  // packed index v = a*(a+1)/2 + b, b <= a
+            const int b = v - a * (a + 1) / 2;
+            gram_out[a * JABAS_GRAM_MAX_K + b] = s;
+            gram_out[b * JABAS_GRAM_MAX_K + a] = s;
+        }
+    }
 }
 
 template <int K>
@@ -129,7 +148,7 @@ int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsi
 }
 
 int launch_gram_finalize(int K, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
-    return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(64), 0, stream, K, partials, grid, gram_out));
+    return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(kGramFinalizeBlock), 0, stream, K, partials, grid, gram_out));
 }
 
 }  // namespace jabas
