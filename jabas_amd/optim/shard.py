@@ -30,6 +30,26 @@ class _ShardOptimizer(torch.optim.Optimizer):
     def __init__(self, params, defaults):
         super().__init__(params, defaults)
         self._plans = {}
+        self._recipes = {}          # call signature -> prepared launches (see _signature)
+
+    def load_state_dict(self, state_dict):
+        super().load_state_dict(state_dict)
+        self._plans.clear()         # the state tensors were replaced: prepared launches point at the old ones
+        self._recipes.clear()
+
+    # -- prepared calls -----------------------------------------------------------------
+    # A training loop hands step() the same parameters and the same gradient buffers every iteration
+    # (DDP bucket views keep their addresses). Matching, validating and marshalling ~150 tensors costs
+    # more host time than the launch takes on the GPU, so a call that found every state in place is
+    # remembered under its signature, and repeated calls only refresh the launch scalars.
+    @staticmethod
+    def _signature(pairs):
+        return tuple([(p.data_ptr(), g.data_ptr(), g.numel()) for _, p, g in pairs])
+
+    def _remember(self, sig, launches, copies):
+        if len(self._recipes) >= self._max_cached_plans:
+            self._recipes.clear()
+        self._recipes[sig] = (launches, copies)
 
     # -- matching ---------------------------------------------------------------------
     def _pairs(self, gradients):
@@ -68,6 +88,7 @@ class _ShardOptimizer(torch.optim.Optimizer):
         g = g.detach()
         if not g.is_contiguous():
             g = g.contiguous()
+            self._volatile = True                 # a fresh copy every call: nothing to remember
         g = g.view(-1)
         if not self._congruent(g, p):
             # a bucket view that starts off the weight's position in a 16-byte line: realign a copy
@@ -76,6 +97,7 @@ class _ShardOptimizer(torch.optim.Optimizer):
             base = (buf.data_ptr() // 4) % 4
             tmp = buf[(skew - base) % 4:][:g.numel()]
             tmp.copy_(g)
+            self._copies.append((tmp, g))
             g = tmp
         return g
 
@@ -87,6 +109,7 @@ class _ShardOptimizer(torch.optim.Optimizer):
                 self._plans.clear()
             plan = self._plans[key] = sync.SyncPlan(spans, args.opt_kind)
         plan.run(args)
+        return plan
 
     def _new_args(self, kind):
         a = L.JabasStepArgs()
@@ -114,9 +137,14 @@ class ShardSGD(_ShardOptimizer):
     @torch.no_grad()
     def step(self, gradients=None, closure=None):
         loss = closure() if closure is not None else None
+        pairs = self._pairs(gradients)
+        sig = self._signature(pairs)
+        if self._replay(self._recipes.get(sig)):
+            return loss
+        self._copies, self._volatile, launches = [], False, []
         # launches are split by (momentum, dampening, nesterov, first-step): launch-wide scalars
         batches = {}
-        for gi, p, g in self._pairs(gradients):
+        for gi, p, g in pairs:
             group = self.param_groups[gi]
             st = self.state[p]
             first = group["momentum"] != 0 and "momentum_buffer" not in st
@@ -140,8 +168,32 @@ class ShardSGD(_ShardOptimizer):
             args.n_groups = len(slots)
             args.momentum, args.dampening = float(momentum), float(dampening)
             args.nesterov, args.first_step = int(nesterov), int(first)
-            self._launch(spans, args)
+            plan = self._launch(spans, args)
+            launches.append((plan, args, (momentum, dampening, bool(nesterov)), list(slots.items())))
+            self._volatile = self._volatile or first
+        if not self._volatile:
+            self._remember(sig, launches, self._copies)
         return loss
+
+    def _replay(self, recipe):
+        """Repeats a remembered call with the hyperparameters as the groups hold them now. False (and
+        nothing done) when a group changed a scalar the launches were split by."""
+        if recipe is None:
+            return False
+        launches, copies = recipe
+        for _, _, key, slots in launches:
+            for gi, _ in slots:
+                group = self.param_groups[gi]
+                if (group["momentum"], group["dampening"], bool(group["nesterov"])) != key:
+                    return False
+        for tmp, g in copies:
+            tmp.copy_(g)
+        for plan, args, _, slots in launches:
+            for gi, slot in slots:
+                args.groups[slot].lr = float(self.param_groups[gi]["lr"])
+                args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
+            plan.run(args)
+        return True
 
 
 class ShardAdam(_ShardOptimizer):
@@ -163,13 +215,19 @@ class ShardAdam(_ShardOptimizer):
     @torch.no_grad()
     def step(self, gradients=None, closure=None):
         loss = closure() if closure is not None else None
+        pairs = self._pairs(gradients)
+        sig = self._signature(pairs)
+        if self._replay(self._recipes.get(sig)):
+            return loss
+        self._copies, self._volatile, launches = [], False, []
         batches = {}
-        for gi, p, g in self._pairs(gradients):
+        for gi, p, g in pairs:
             group = self.param_groups[gi]
             if group["amsgrad"]:
                 raise NotImplementedError("amsgrad is not part of the fused path")
             st = self.state[p]
             if len(st) == 0:
+                self._volatile = True             # state created in this call: remember the next one
                 st["step"] = 0
                 st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
@@ -191,8 +249,44 @@ class ShardAdam(_ShardOptimizer):
                 args.groups[slot].step = step
             args.n_groups = len(slots)
             args.beta1, args.beta2, args.eps = float(betas[0]), float(betas[1]), float(eps)
-            self._launch(spans, args)
+            plan = self._launch(spans, args)
+            # per slot: its group and one state that carries the slot's step count; per item: state and slot
+            reps = {}
+            for gi, step, p, g, st in items:
+                reps.setdefault(slots[(gi, step)], (gi, st))
+            launches.append((plan, args, (betas, eps), sorted(reps.items()),
+                             [(st, slots[(gi, step)]) for gi, step, p, g, st in items]))
+        if not self._volatile:
+            self._remember(sig, launches, self._copies)
         return loss
+
+    def _replay(self, recipe):
+        """Repeats a remembered call: bumps every parameter's step count and refreshes the launch scalars.
+        False (and nothing done) when betas / eps of a group changed or when parameters that shared a
+        step count no longer do (they were stepped apart in between)."""
+        if recipe is None:
+            return False
+        launches, copies = recipe
+        for _, _, key, reps, items in launches:
+            for _, (gi, _) in reps:
+                group = self.param_groups[gi]
+                if (tuple(group["betas"]), group["eps"]) != key or group["amsgrad"]:
+                    return False
+            steps = [st["step"] for _, (_, st) in reps]
+            for st, slot in items:
+                if st["step"] != steps[slot]:
+                    return False
+        for tmp, g in copies:
+            tmp.copy_(g)
+        for plan, args, _, reps, items in launches:
+            for st, _ in items:
+                st["step"] += 1
+            for slot, (gi, st) in reps:
+                args.groups[slot].lr = float(self.param_groups[gi]["lr"])
+                args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
+                args.groups[slot].step = int(st["step"])
+            plan.run(args)
+        return True
 
 
 class ShardAdamW(ShardAdam):

@@ -465,3 +465,77 @@ def test_trainer_with_bf16_gradient_buckets(gpu):
         for m in trainer.local_models[1:]:
             for pm, p in zip(m.parameters(), trainer.main_model.parameters()):
                 assert torch.equal(pm, p)
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_shard_optimizer_remembered_calls_follow_every_change(gpu, kind):
+    """step() remembers a call it has prepared once (same parameters, same gradient buffers) and then
+    only refreshes launch scalars. Everything that may change between two such calls must still take
+    effect: gradient values, learning rate and weight decay, gradients that need a realigned copy,
+    parameters stepped in different subsets (diverging Adam step counts), a changed momentum / betas,
+    and load_state_dict. Checked against torch.optim on a twin model over persistent gradient buffers."""
+    from jabas_amd import optim
+    from jabas_amd.train.trainer import tag_parameter_indices
+    model = tag_parameter_indices(_mlp(3).to(gpu))
+    ref_model = copy.deepcopy(model)
+    params, ref_params = list(model.parameters()), list(ref_model.parameters())
+    if kind == "sgd":
+        mine = optim.ShardSGD(_groups(model), lr=0.05, momentum=0.9, weight_decay=1e-4)
+        ref = torch.optim.SGD(_groups(ref_model), lr=0.05, momentum=0.9, weight_decay=1e-4, foreach=False)
+    else:
+        mine = optim.ShardAdamW(_groups(model), lr=1e-3)
+        ref = torch.optim.AdamW(_groups(ref_model), lr=1e-3, foreach=False)
+    # one flat persistent "bucket" with a view per parameter (several start off a 16-byte line)
+    flat = torch.zeros(sum(p.numel() for p in params), device=gpu)
+    views, off = [], 0
+    for i, p in enumerate(params):
+        v = flat[off:off + p.numel()].view_as(p)
+        v.index = i
+        views.append(v)
+        off += p.numel()
+
+    def one_step(step, subset=None):
+        flat.copy_(torch.randn(flat.numel(), generator=torch.Generator().manual_seed(100 + step)) * 1e-2)
+        chosen = range(len(params)) if subset is None else subset
+        mine.step([views[i] for i in chosen])
+        for i, rp in enumerate(ref_params):
+            rp.grad = views[i].detach().clone() if i in chosen else None
+        ref.step()
+        torch.cuda.synchronize()
+        for i, (p, rp) in enumerate(zip(params, ref_params)):
+            assert _close(p, rp, 1e-6, 1e-8), (kind, step, i)
+
+    for step in range(1, 5):                              # step 1 creates state, 2 is remembered, 3.. are replays
+        one_step(step)
+    assert len(mine._recipes) == 1
+    for opt_ in (mine, ref):                              # a scheduler at work
+        for g in opt_.param_groups:
+            g["lr"] *= 0.5
+        opt_.param_groups[1]["weight_decay"] = 0.02
+    one_step(5)
+    one_step(6)
+    one_step(7, subset=[0, 1, 4])                         # a bucket's worth of parameters: its own remembered call
+    one_step(8, subset=[0, 1, 4])
+    one_step(9)                                           # Adam: parameters 0, 1, 4 are now two steps ahead of the rest
+    one_step(10)
+    if kind == "sgd":
+        for opt_ in (mine, ref):
+            opt_.param_groups[0]["momentum"] = 0.5        # a scalar the launches are split by
+    else:
+        for opt_ in (mine, ref):
+            opt_.param_groups[1]["betas"] = (0.8, 0.99)
+    one_step(11)
+    one_step(12)
+    # load_state_dict replaces the state tensors: the next call must use the restored ones, not those its
+    # remembered launch pointed at (which by now hold the state after step 13)
+    saved, ref_saved = copy.deepcopy(mine.state_dict()), copy.deepcopy(ref.state_dict())
+    weights = [p.detach().clone() for p in params]
+    one_step(13)
+    mine.load_state_dict(saved)
+    ref.load_state_dict(ref_saved)
+    with torch.no_grad():
+        for p, rp, w in zip(params, ref_params, weights):
+            p.copy_(w)
+            rp.copy_(w)
+    one_step(14)
+    one_step(15)
