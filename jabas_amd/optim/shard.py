@@ -25,7 +25,7 @@ def _index_of(t):
 
 class _ShardOptimizer(torch.optim.Optimizer):
     _kind = None
-    _max_cached_plans = 64
+    _max_cached_plans = 1024       # one per distinct call (a DDP bucket each in the overlap mode): a few KB of tables apiece
 
     def __init__(self, params, defaults):
         super().__init__(params, defaults)
