@@ -17,8 +17,11 @@ from .sync import SpanSpec, SyncPlan, make_step_args, opt_kind, cosine_from_stat
 
 class VSWFlatSync:
     def __init__(self, specs, batches, grad_dtype=torch.float32, opt=None, device="cuda", in_place=None,
-                 n_fanout=0, per_tensor_spans=False, caps=None):
+                 n_fanout=0, per_tensor_spans=False, caps=None, keep_clipped_grads=True):
         self.K = len(batches)
+        # clipped steps: True leaves the clipped aggregate in the gradient arena, as clip_grad_norm_
+        # leaves the clipped .grad behind; False saves that write (4 of 52 bytes per element)
+        self.keep_clipped_grads = keep_clipped_grads
         self.batches = tuple(batches)
         self.grad_dtype = grad_dtype
         self.opt = opt
@@ -149,7 +152,8 @@ class VSWFlatSync:
         for (off, numel, bounds, _bucket) in self.layout.spans:
             sl = slice(off, off + numel)
             agg_spans.append(SpanSpec([g[sl] for g in self.grads], agg_out=self.agg[sl]))
-            opt_spans.append(SpanSpec([self.agg[sl]], agg_out=self.agg[sl], param=self.param[sl],
+            opt_spans.append(SpanSpec([self.agg[sl]], agg_out=self.agg[sl] if self.keep_clipped_grads else None,
+                                      param=self.param[sl],
                                       state1=None if self.state1 is None else self.state1[sl],
                                       state2=None if self.state2 is None else self.state2[sl],
                                       fanout=[f[sl] for f in self.fanout], bounds=bounds))

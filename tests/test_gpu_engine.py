@@ -70,11 +70,11 @@ def test_engine_steps_match_oracle(gpu, opt, dtype, per_tensor):
         assert torch.allclose(per_bucket.sum(0), rows.cpu().sum(0), rtol=1e-12)
 
 
-@pytest.mark.parametrize("clip_norm", [0.05, 1e3])
+@pytest.mark.parametrize("clip_norm,keep", [(0.05, True), (1e3, True), (0.05, False)])
 @pytest.mark.parametrize("opt", [SGD, ADAM])
-def test_global_norm_clipping(gpu, opt, clip_norm):
+def test_global_norm_clipping(gpu, opt, clip_norm, keep):
     batches = (128, 128, 64, 64)
-    eng, host, spans = _make(gpu, batches, opt, n_fanout=1)
+    eng, host, spans = _make(gpu, batches, opt, n_fanout=1, keep_clipped_grads=keep)
     adam = opt["kind"] != "sgd"
     for step in (1, 2):
         rows = eng.step(stats=True, clip_norm=clip_norm)
@@ -88,14 +88,18 @@ def test_global_norm_clipping(gpu, opt, clip_norm):
         assert _close(rows[:, :8], rows_h[:, :8], 1e-6, 1e-30)     # statistics are of the unclipped aggregate
         for off, cnt, _ in spans:
             sl = slice(off, off + cnt)
-            assert _close(eng.agg[sl], agg_h[sl], 1e-6, 1e-12), step
+            if keep:
+                assert _close(eng.agg[sl], agg_h[sl], 1e-6, 1e-12), step
+            else:                                                  # the unclipped aggregate stays behind
+                assert _close(eng.agg[sl] * c, agg_h[sl], 1e-6, 1e-12), step
             if c >= 1.0:
                 assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h[sl].view(torch.int32))
         assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
         for off, cnt, _ in spans:
             assert torch.equal(eng.fanout[0][off:off + cnt], eng.param[off:off + cnt])
-            host["g"][0][off:off + cnt] = agg_h[off:off + cnt]
-    if clip_norm < 1.0:
+            # the in-place aggregate is worker 0's input of the next step
+            host["g"][0][off:off + cnt] = agg_h[off:off + cnt] if keep else eng.agg[off:off + cnt].cpu()
+    if clip_norm < 1.0 and keep:
         norm = math.sqrt(sum(float(torch.dot(eng.agg[o:o + c_].double(), eng.agg[o:o + c_].double())) for o, c_, _ in spans))
         assert norm == pytest.approx(clip_norm, rel=1e-4)
 

@@ -539,3 +539,40 @@ def test_shard_optimizer_remembered_calls_follow_every_change(gpu, kind):
             rp.copy_(w)
     one_step(14)
     one_step(15)
+
+
+@pytest.mark.parametrize("max_norm", [0.05, 1e3])
+def test_trainer_clips_the_global_gradient_norm(gpu, max_norm):
+    """GNMT's step (examples/gnmt/seq2seq/train/trainer.py:157-161): clip_grad_norm_ over the synchronised
+    gradient, then the optimizer. Against torch on a twin model; the small bound clips, the large one
+    does not."""
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (6, 2)
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, interval=1, clip_norm=max_norm)
+    trainer.prepare_stream_parallel(_mlp(41), crit)
+    mine = torch.optim.Adam(_groups(trainer.main_model), lr=2e-3, foreach=False)
+    trainer.prepare_weight_sync_method(mine)
+    ref_model = _mlp(41).to(gpu)
+    ref_opt = torch.optim.Adam(_groups(ref_model), lr=2e-3, foreach=False)
+    w, _, _ = O.batch_weights(batches)
+    clipped = 0
+    for step in range(1, 4):
+        gen = torch.Generator().manual_seed(800 + step)
+        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        trainer.compute(data)
+        per_vsw = []
+        for x, y in data:
+            ref_model.zero_grad(set_to_none=True)
+            crit(ref_model(x), y).backward()
+            per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(per_vsw[0][i], w[0]), torch.mul(per_vsw[1][i], w[1]))
+        total = torch.nn.utils.clip_grad_norm_(list(ref_model.parameters()), max_norm)
+        clipped += int(float(total) > max_norm)
+        ref_opt.step()
+        trainer.step()
+        torch.cuda.synchronize()
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 2e-6, 1e-7), f"step {step}"
+    assert clipped == (3 if max_norm < 1.0 else 0)
