@@ -51,7 +51,18 @@ class LocalBucketSync:
     ``jabas_sync_bucket`` on VSW 0's stream.
     """
 
-    def __init__(self, batches, launcher=None, opt=None, param_buckets=None):
+    def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False):
+        """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
+        ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
+        overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
+        (one ramp-up and drain: 0.66 ms against 1.0 ms for the 14 buckets of ViT-B/16) and less host
+        time, and the buckets hold the aggregate only after ``finish_step``."""
+        if deferred and launcher is not None:
+            raise ValueError("the deferred mode drives the C ABI itself: no launcher can be injected")
+        self.deferred = bool(deferred)
+        self._ready = {}                       # deferred mode: bucket index -> complete _Slot of this step
+        self._vsw_streams = {}                 # deferred mode: VSW index -> the stream its hooks ran on
+        self._plan = self._plan_key = None
         self.batches = tuple(batches)
         self.K = len(self.batches)
         self.opt = opt
@@ -81,8 +92,11 @@ class LocalBucketSync:
         event = stream = None
         if tensor.is_cuda:
             stream = torch.cuda.current_stream(tensor.device)
-            event = torch.cuda.Event()
-            event.record(stream)
+            if self.deferred:                  # ordered once per VSW stream in finish_step, not once per bucket
+                self._vsw_streams[k] = stream
+            else:
+                event = torch.cuda.Event()
+                event.record(stream)
         with self._lock:
             slot = self._slots.setdefault(bucket_index, _Slot(self.K))
             if slot.tensors[k] is not None:
@@ -96,7 +110,11 @@ class LocalBucketSync:
             if ready:
                 del self._slots[bucket_index]
         if ready:
-            self._fire(bucket_index, slot)
+            if self.deferred:
+                with self._lock:
+                    self._ready[bucket_index] = slot
+            else:
+                self._fire(bucket_index, slot)
         return fut
 
     def _fire(self, bucket_index, slot):
@@ -140,17 +158,68 @@ class LocalBucketSync:
         workspace) is kept per bucket and rebuilt only when the buffers change."""
         call = self._calls.get(bucket_index)
         if call is None or not call.matches(tensors):
-            g0 = tensors[0]
-            pb = self.param_buckets.get(bucket_index)
-            opt = self.opt if pb is not None else None
-            span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
-                                 param=pb and pb.get("param"), state1=pb and pb.get("state1"),
-                                 state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
-                                 bounds=(pb or {}).get("bounds", ()) if opt else ())
+            span, with_opt = self._span_of(bucket_index, tensors)
             call = self._calls[bucket_index] = sync.BucketCall(span)
-            call.with_opt = opt is not None
+            call.with_opt = with_opt
         args = self._step_args(tensors[0].dtype, want_stats, call.with_opt)
         return call.run(args, stream=self._main_stream)
+
+    def _span_of(self, bucket_index, tensors):
+        """(span over the K buffers of one bucket, whether the optimizer runs in the same launch)."""
+        g0 = tensors[0]
+        pb = self.param_buckets.get(bucket_index)
+        opt = self.opt if pb is not None else None
+        span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
+                             param=pb and pb.get("param"), state1=pb and pb.get("state1"),
+                             state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
+                             bounds=(pb or {}).get("bounds", ()) if opt else ())
+        return span, opt is not None
+
+    def _fire_all(self):
+        """Deferred mode: one planned launch over every bucket of the step, in bucket order."""
+        with self._lock:
+            ready, self._ready = self._ready, {}
+        order = sorted(ready)
+        slots = [ready[i] for i in order]
+        with_opt = [self.opt is not None and i in self.param_buckets for i in order]
+        main = self._main_stream
+        if main is None or (any(with_opt) and not all(with_opt)):
+            for i, slot in zip(order, slots):          # host tensors (protocol tests), or buckets with and without
+                self._fire(i, slot)                    # weights behind them: one launch each after all
+            return
+        try:
+            # everything the other VSWs queued up to now (their whole backward) precedes the launch: one
+            # event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
+            # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
+            for k, stream in sorted(self._vsw_streams.items()):
+                if k != 0 and stream != main:
+                    ev = torch.cuda.Event()
+                    ev.record(stream)
+                    main.wait_event(ev)
+            key = tuple((i, slot.tensors[0].numel()) + tuple(t.data_ptr() for t in slot.tensors)
+                        for i, slot in zip(order, slots))
+            if key != self._plan_key:                   # DDP hands over the same buffers every step: built once
+                spans = [self._span_of(i, slot.tensors)[0] for i, slot in zip(order, slots)]
+                self._plan = sync.SyncPlan(spans, sync.opt_kind(self.opt) if with_opt[0] else L.OPT_NONE)
+                self._plan_key = key
+            want = any(slot.want_stats for slot in slots)
+            args = self._step_args(slots[0].tensors[0].dtype, want, with_opt[0])
+            rows = self._plan.run(args, stream=main)
+            if rows is not None:
+                with torch.cuda.stream(main):
+                    rows = rows.clone()                 # the plan's own rows are overwritten by its next launch
+            done = torch.cuda.Event()
+            done.record(main)
+            self._done_events.append(done)
+        except Exception as exc:
+            with self._lock:
+                self._errors.append((order[0], exc))
+            return
+        for j, (i, slot) in enumerate(zip(order, slots)):
+            if slot.on_done is not None:
+                slot.on_done(BucketStats(i, rows[j]) if slot.want_stats and rows is not None else None)
+        with self._lock:
+            self.launched += 1
 
     # ------------------------------------------------------------------ trainer calls this
     def pending(self):
@@ -163,6 +232,8 @@ class LocalBucketSync:
         left = self.pending()
         if left:
             raise RuntimeError(f"buckets {left} were not published by every VSW")
+        if self._ready:
+            self._fire_all()
         with self._lock:
             errors, self._errors = self._errors, []
         if errors:

@@ -97,7 +97,11 @@ def test_shard_step_with_bucket_gradients_updates_only_matching_parameters(gpu):
             assert len(opt.state[p]) == 0
 
 
-def test_k_vsw_rendezvous_with_streams_and_threads(gpu):
+@pytest.mark.parametrize("deferred", [False, True])
+def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
+    """K hook threads on K streams hand their buckets over in different orders. Per-bucket mode: the
+    last arrival queues that bucket's launch. Deferred mode: nothing is queued until finish_step, which
+    queues one planned launch over all buckets (built once, reused while DDP hands over the same buffers)."""
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
 
@@ -112,44 +116,54 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu):
             return self._t
 
     K, batches, sizes = 3, (4, 2, 2), [40001, 7, 250000]
-    host = [[torch.randn(n, generator=torch.Generator().manual_seed(100 * b + k)) * 1e-3 for k in range(K)]
-            for b, n in enumerate(sizes)]
-    local = LocalBucketSync(batches)
+    local = LocalBucketSync(batches, deferred=deferred)
     st = H.GradientSimilarityState(None, 4, None, [], 1).attach_local(local)
     main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
     streams = [torch.cuda.Stream(gpu) for _ in range(K)]
-    dev = [[None] * K for _ in sizes]
-    futs = {}
+    dev = [[torch.empty(n, device=gpu) for _ in range(K)] for n in sizes]      # DDP's bucket buffers: the same every step
+    plans = []
+    for step in range(3):
+        host = [[torch.randn(n, generator=torch.Generator().manual_seed(1000 * step + 100 * b + k)) * 1e-3
+                 for k in range(K)] for b, n in enumerate(sizes)]
+        futs = {}
 
-    def vsw(k):
-        with torch.cuda.stream(streams[k]):
-            order = range(len(sizes)) if k % 2 == 0 else reversed(range(len(sizes)))
-            for b in order:
-                dev[b][k] = host[b][k].to(gpu, non_blocking=False)          # "backward" fills the bucket on this stream
-                bucket = Bucket(b, dev[b][k])
-                futs[(k, b)] = main_hook(st, bucket) if k == 0 else H.dummy_hook(H.VSWPeerState(local, k), bucket)
+        def vsw(k):
+            with torch.cuda.stream(streams[k]):
+                order = range(len(sizes)) if k % 2 == 0 else reversed(range(len(sizes)))
+                for b in order:
+                    dev[b][k].copy_(host[b][k])                               # "backward" fills the bucket on this stream
+                    bucket = Bucket(b, dev[b][k])
+                    futs[(k, b)] = main_hook(st, bucket) if k == 0 else H.dummy_hook(H.VSWPeerState(local, k), bucket)
 
-    threads = [threading.Thread(target=vsw, args=(k,)) for k in range(K)]
-    for t in threads:
-        t.start()
-    for t in threads:
-        t.join()
-    for f in futs.values():
-        f.wait()
-    local.finish_step(streams)
-    torch.cuda.synchronize()
-    for b in range(len(sizes)):
-        want = O.aggregate(host[b], batches)
-        assert torch.equal(dev[b][0].cpu().view(torch.int32), want.view(torch.int32)), b
-        for k in range(1, K):
-            assert torch.equal(dev[b][k].cpu(), host[b][k])
-    rows = {s.index: s.cpu() for s in st.grad_placeholder}
-    assert sorted(rows) == [0, 1, 2]
-    for b in range(len(sizes)):
-        want = O.stats(host[b], batches)
-        assert _close(rows[b][:4 + K], want[:4 + K], 1e-6, 0.0)
-    whole = O.cosine_from_rows(torch.stack([O.stats(host[b], batches) for b in range(len(sizes))]))
-    assert H.cosine_similarity_from_placeholder(st.grad_placeholder) == pytest.approx(whole, rel=1e-9)
+        threads = [threading.Thread(target=vsw, args=(k,)) for k in range(K)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for f in futs.values():
+            f.wait()
+        before = local.launched
+        local.finish_step(streams)
+        assert local.launched - before == (1 if deferred else 0)
+        assert local.launched == (step + 1) * (1 if deferred else len(sizes))
+        plans.append(local._plan)
+        torch.cuda.synchronize()
+        for b in range(len(sizes)):
+            want = O.aggregate(host[b], batches)
+            assert torch.equal(dev[b][0].cpu().view(torch.int32), want.view(torch.int32)), (step, b)
+            for k in range(1, K):
+                assert torch.equal(dev[b][k].cpu(), host[b][k])
+        rows = {s.index: s.cpu() for s in st.grad_placeholder}
+        assert sorted(rows) == [0, 1, 2]
+        for b in range(len(sizes)):
+            want = O.stats(host[b], batches)
+            assert _close(rows[b][:4 + K], want[:4 + K], 1e-6, 0.0)
+        whole = O.cosine_from_rows(torch.stack([O.stats(host[b], batches) for b in range(len(sizes))]))
+        assert H.cosine_similarity_from_placeholder(st.grad_placeholder) == pytest.approx(whole, rel=1e-9)
+        st.grad_placeholder.clear()
+        st.step += 1
+    if deferred:
+        assert plans[0] is not None and plans[1] is plans[0] and plans[2] is plans[0]
 
 
 @pytest.mark.parametrize("kind", ["sgd", "adamw"])
