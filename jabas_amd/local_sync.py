@@ -76,7 +76,7 @@ class LocalBucketSync:
         self._main_stream = None
         self._calls = {}                       # bucket index -> prepared sync.BucketCall
         self._args_cache = {}
-        self._done_events = []
+        self._launch_streams = set()           # streams that carry launches of the current step
         self._errors = []
         self.launched = 0                      # fused launches queued so far
 
@@ -94,7 +94,7 @@ class LocalBucketSync:
             stream = torch.cuda.current_stream(tensor.device)
             if self.deferred:                  # ordered once per VSW stream in finish_step, not once per bucket
                 self._vsw_streams[k] = stream
-            else:
+            elif k != 0:                       # VSW 0's stream is the one the launch is queued on
                 event = torch.cuda.Event()
                 event.record(stream)
         with self._lock:
@@ -124,9 +124,7 @@ class LocalBucketSync:
                 for ev in slot.events[1:]:
                     main.wait_event(ev)
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
-                done = torch.cuda.Event()
-                done.record(main)
-                self._done_events.append(done)
+                self._launch_streams.add(main)
             else:
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
         except Exception as exc:                       # reported by finish_step
@@ -208,9 +206,7 @@ class LocalBucketSync:
             if rows is not None:
                 with torch.cuda.stream(main):
                     rows = rows.clone()                 # the plan's own rows are overwritten by its next launch
-            done = torch.cuda.Event()
-            done.record(main)
-            self._done_events.append(done)
+            self._launch_streams.add(main)
         except Exception as exc:
             with self._lock:
                 self._errors.append((order[0], exc))
@@ -234,13 +230,18 @@ class LocalBucketSync:
             raise RuntimeError(f"buckets {left} were not published by every VSW")
         if self._ready:
             self._fire_all()
+        # the launches of a step sit on VSW 0's stream in order: one event behind the last of them orders
+        # every VSW stream behind all of them
+        launch_streams, self._launch_streams = self._launch_streams, set()
+        for main in launch_streams:
+            done = torch.cuda.Event()
+            done.record(main)
+            for s in streams:
+                if s != main:
+                    s.wait_event(done)
         with self._lock:
             errors, self._errors = self._errors, []
         if errors:
             idx, exc = errors[0]
             raise RuntimeError(f"fused launch of bucket {idx} failed: {exc}") from exc
-        for s in streams:
-            for ev in self._done_events:
-                s.wait_event(ev)
-        self._done_events = []
         self.step_count += 1
