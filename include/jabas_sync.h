@@ -14,9 +14,9 @@
  *   - plain C types only; every buffer is caller-owned device memory;
  *   - no entry point allocates, frees or synchronises the device; all work is queued
  *     on the stream passed in (jabas_stream_t is a hipStream_t);
- *   - the library keeps no mutable global state, so
- *     calls from different threads on different streams do not interfere as long as
- *     they use different workspaces;
+ *   - the library keeps no mutable global state (jabas_sync_bucket_static apart, which says
+ *     so), so calls from different threads on different streams do not interfere as long
+ *     as they use different workspaces;
  *   - return value: JABAS_OK (0) or a negative JabasStatus; nothing is launched when a
  *     negative status is returned (except JABAS_ERR_LAUNCH, reported after the fact).
  *     JABAS_ERR_LAUNCH is the return value of this call's own hipLaunchKernel: a HIP
@@ -40,6 +40,7 @@ extern "C" {
 #define JABAS_STATS_STRIDE 20   /* doubles per span in stats_out: 4 + JABAS_MAX_K     */
 #define JABAS_GRAM_MAX_K 8      /* VSWs of one jabas_gram call                        */
 #define JABAS_GRAM_STRIDE 64    /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
+#define JABAS_STATIC_MAX_NUMEL (1ull << 26)  /* largest span of jabas_sync_bucket_static  */
 
 typedef void* jabas_stream_t;   /* hipStream_t */
 
@@ -207,6 +208,22 @@ int jabas_sync_fused(const void* plan_host, const void* plan_dev,
 int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev,
                       const JabasStepArgs* args, double* stats_out,
                       void* workspace, size_t workspace_bytes, jabas_stream_t stream);
+
+/* jabas_sync_bucket without a workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc) and so cannot size a workspace for whatever bucket comes next. No counterpart
+ * in the reference. The partial rows of the statistics reduction go to a static device
+ * array of 5.25 MB that every GPU the process uses holds until the process ends; its
+ * address is looked up once per GPU, on the first call made with that GPU current (the
+ * stream must belong to the current device). Calls neither allocate nor free anything.
+ * span->numel above JABAS_STATIC_MAX_NUMEL (64 Mi elements, a 256 MB fp32 bucket) is refused
+ * with JABAS_ERR_SIZE before anything is launched. All calls on one GPU share that GPU's
+ * array: calls with statistics that overlap in time on one GPU (different streams or
+ * threads) race on it and must be serialised by the caller; calls without statistics do
+ * not touch it. Results are those of jabas_sync_bucket, bit for bit. */
+int jabas_sync_bucket_static(const JabasSpan* span, const JabasBound* bounds_dev,
+                             const JabasStepArgs* args, double* stats_out,
+                             jabas_stream_t stream);
 
 /* --- single-purpose entry points (thin fronts over the same kernels) ---------------- */
 

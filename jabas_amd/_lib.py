@@ -16,6 +16,7 @@ MAX_GROUPS = 16
 STATS_STRIDE = 20
 GRAM_MAX_K = 8
 GRAM_STRIDE = 64
+STATIC_MAX_NUMEL = 1 << 26
 
 F32, BF16 = 0, 1
 OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW = 0, 1, 2, 3
@@ -87,6 +88,8 @@ SIGNATURES = {
                                    C.c_void_p, C.c_size_t, C.c_void_p]),
     "jabas_sync_bucket": (C.c_int, [C.POINTER(JabasSpan), C.c_void_p, C.POINTER(JabasStepArgs), C.c_void_p,
                                     C.c_void_p, C.c_size_t, C.c_void_p]),
+    "jabas_sync_bucket_static": (C.c_int, [C.POINTER(JabasSpan), C.c_void_p, C.POINTER(JabasStepArgs), C.c_void_p,
+                                           C.c_void_p]),
     "jabas_aggregate": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.POINTER(C.c_float),
                                   C.c_void_p, C.c_uint64, C.c_void_p]),
     "jabas_stats": (C.c_int, [C.POINTER(C.c_void_p), C.c_int32, C.c_int32, C.POINTER(C.c_float),

@@ -4,6 +4,8 @@
 #include <math.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "jabas_internal.h"
 
 #define JABAS_API extern "C" __attribute__((visibility("default")))
@@ -328,7 +330,7 @@ inline uint32_t stripes_for(uint32_t max_span_chunks) {
     return st > kMaxStripes ? kMaxStripes : st;
 }
 // workspace rows: one per chunk, then one per (span, stripe)
-inline size_t workspace_rows(uint64_t n_chunks, uint64_t n_span) { return n_chunks + n_span * kMaxStripes + 1; }
+constexpr size_t workspace_rows(uint64_t n_chunks, uint64_t n_span) { return n_chunks + n_span * kMaxStripes + 1; }
 
 // One wave: fixed-order sum of slot NORM_AGG over the rows, then the coefficient.
 __global__ void __launch_bounds__(64) clip_coef_kernel(const double* rows, uint32_t n_rows, double max_norm, double eps,
@@ -390,7 +392,7 @@ JABAS_API const char* jabas_status_string(int status) {
         case JABAS_ERR_GROUP: return "parameter group index/count out of range or bounds not sorted";
         case JABAS_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case JABAS_ERR_PLAN: return "plan blob malformed, too small or not matching the step arguments";
-        case JABAS_ERR_SIZE: return "element, span or fan-out count out of range";
+        case JABAS_ERR_SIZE: return "element, span or fan-out count out of range (jabas_sync_bucket_static: more than JABAS_STATIC_MAX_NUMEL elements)";
         case JABAS_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
         case JABAS_ERR_ALIAS: return "a written buffer overlaps another buffer of the span (only agg_out == grads[k], fp32, may alias)";
         default: return "unknown status";
@@ -617,6 +619,54 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     a.n_chunks = static_cast<uint32_t>(chunks_of_tiles(tiles, a.chunk_tiles));
     a.use_inline = 1;
     return run_fused(a, args, a.n_chunks, stats_out, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+// --- the entry point that allocates nothing -------------------------------------------------
+// The partial rows of the statistics reduction live in a file-scope device array instead of a
+// caller-provided workspace. Every GPU the library runs on holds its own copy of the array at its
+// own address until the process ends; the address is looked up once per device, on the first call
+// made with that device current.
+namespace {
+constexpr uint64_t kStaticMaxNumel = JABAS_STATIC_MAX_NUMEL;
+// statistics launches run 256 threads x 2 tiles at the least: 2048 elements per partial row
+constexpr uint64_t kStaticMinChunkElems = 4ull * kBlock * kMinChunkTiles;
+constexpr size_t kStaticScratchBytes =
+    workspace_rows((kStaticMaxNumel + kWideElems - 1 + kStaticMinChunkElems - 1) / kStaticMinChunkElems, 1) *
+    kStatsStride * sizeof(double);
+static_assert(kStaticScratchBytes <= (6u << 20), "static scratch stays modest");
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+namespace {
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Device address of this GPU's copy of `scratch`. In host code the array's name is only a handle for
+// the runtime, never an address a kernel could use.
+int static_scratch(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return JABAS_ERR_LAUNCH;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return JABAS_ERR_LAUNCH;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);     // racing first calls look up the same address
+    }
+    *out = p;
+    return JABAS_OK;
+}
+}  // namespace
+
+JABAS_API int jabas_sync_bucket_static(const JabasSpan* span, const JabasBound* bounds_dev, const JabasStepArgs* args,
+                                       double* stats_out, jabas_stream_t stream) {
+    if (!span || !args) return JABAS_ERR_NULL;
+    if (span->numel > kStaticMaxNumel) return JABAS_ERR_SIZE;
+    void* ws = nullptr;
+    if (args->stats) {
+        const int rc = static_scratch(&ws);
+        if (rc != JABAS_OK) return rc;
+    }
+    // Every partial row the finalize launches read is written by this call's own launches first, so
+    // nothing has to be cleared between calls.
+    return jabas_sync_bucket(span, bounds_dev, args, stats_out, ws, ws ? kStaticScratchBytes : 0, stream);
 }
 
 JABAS_API int jabas_aggregate(const void* const* grads, int32_t K, int32_t grad_dtype, const float* weight,

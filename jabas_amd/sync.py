@@ -269,6 +269,22 @@ def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
     return workspace.stats[0] if args.stats else None
 
 
+def sync_bucket_static(span, args, stats_out=None, bounds_dev=None, stream=None):
+    """``jabas_sync_bucket_static``: one span by value with the statistics scratch in the library's static
+    device array (no workspace, nothing allocated by the call). ``stats_out``: caller-owned device row of
+    STATS_STRIDE doubles, required when args.stats is set; ``bounds_dev``: device bound table from
+    ``bounds_to_device`` when the span has bounds. Calls with statistics on one GPU must not overlap."""
+    c_span = span.to_c()
+    if span.bounds and bounds_dev is None:
+        raise ValueError("pass the span's bound table on the device (bounds_to_device): this call allocates nothing")
+    if args.stats and stats_out is None:
+        raise ValueError("pass stats_out: this call allocates nothing")
+    L.check(L.lib().jabas_sync_bucket_static(C.byref(c_span), None if bounds_dev is None else bounds_dev.data_ptr(),
+                                             C.byref(args), None if stats_out is None else stats_out.data_ptr(),
+                                             _stream_ptr(stream)), "jabas_sync_bucket_static")
+    return stats_out
+
+
 def bounds_to_device(bounds, device):
     """Device copy of a span's bound table in JabasBound layout (for ``jabas_sync_bucket``)."""
     host = np.zeros((len(bounds), 2), dtype=np.uint64)
