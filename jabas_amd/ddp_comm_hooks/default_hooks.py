@@ -59,4 +59,5 @@ def dummy_hook(state, bucket):
     tensor = bucket_tensor(bucket)
     if state is None or getattr(state, "local", None) is None:
         return completed(bucket_value(bucket, tensor))
-    return state.local.publish(state.vsw_index, bucket_index(bucket), tensor, value=bucket_value(bucket, tensor))
+    return state.local.publish(state.vsw_index, bucket_index(bucket), tensor, value=bucket_value(bucket, tensor),
+                               bucket=bucket)

@@ -35,4 +35,5 @@ def iidp_allreduce_hook(state, bucket, want_stats=False, on_done=None):
         if on_done is not None:
             on_done(None)
         return completed(value)
-    return local.publish(0, bucket_index(bucket), tensor, want_stats=want_stats, on_done=on_done, value=value)
+    return local.publish(0, bucket_index(bucket), tensor, want_stats=want_stats, on_done=on_done, value=value,
+                         bucket=bucket)

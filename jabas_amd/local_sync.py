@@ -4,14 +4,21 @@ In IIDP every VSW runs its own DDP reducer on its own thread and stream; only VS
 comm hook communicates, the others register ``dummy_hook``
 (jabas/train/trainer.py:452-468). ``LocalBucketSync`` is where those K hooks meet on one
 GPU: each hook publishes the flat bucket it was handed; when the K buckets with the same
-index are in, whichever thread arrived last queues ONE fused kernel on VSW 0's stream
-(aggregate into VSW 0's bucket, statistics when asked, optimizer update when the weights
-are laid out like the buckets). The Future a hook gets back is already complete: stock
-DDP waits on it at the end of that replica's backward on the autograd engine's device
-thread, which every replica on the GPU shares, so a Future that needed another replica's
-backward to make progress would deadlock. Ordering is by stream instead: the launch waits
-on an event from every VSW's stream, and ``finish_step`` makes every VSW stream wait for
-the launches (and reports anything that went wrong in them) before gradients are reused.
+index are in, whichever thread arrived last queues ONE fused kernel (aggregate into VSW 0's
+bucket, statistics when asked, optimizer update and weight fan-out when an optimizer is
+bound). The Future a hook gets back is already complete: stock DDP waits on it at the end
+of that replica's backward on the autograd engine's device thread, which every replica on
+the GPU shares, so a Future that needed another replica's backward to make progress would
+deadlock. Ordering is by stream instead: the launch waits on an event from every VSW's
+stream, and ``finish_step`` makes every VSW stream wait for the launches (and reports
+anything that went wrong in them) before gradients and weights are reused.
+
+The "overlap" weight-sync mode (jabas/train/trainer.py:327-333: an optimizer hook on VSW 0
+that updates the weights of a bucket as soon as its gradients are synchronised, on a stream
+of its own) is this class with an optimizer bound (``bind_optimizer``) and a launch stream
+(``stream=``): the weights and optimizer state of a bucket's parameters are laid out in
+flat arenas exactly like the bucket, so aggregate, update and the copy of the new weights
+to the other replicas are one launch per bucket.
 """
 import threading
 
@@ -37,10 +44,22 @@ class BucketStats:
 class _Slot:
     def __init__(self, K):
         self.tensors = [None] * K
+        self.buckets = [None] * K
         self.events = [None] * K
         self.want_stats = False
         self.on_done = None
         self.count = 0
+
+
+def _arena_like(buf, dtype=torch.float32, zero=True):
+    """Flat tensor of ``buf.numel()`` elements of ``dtype`` whose first element sits at the same element
+    position of a 256-byte line as ``buf``'s (the layout the kernels stream fastest, and the congruence
+    they require)."""
+    n = buf.numel()
+    raw = (torch.zeros if zero else torch.empty)(n + 64, dtype=dtype, device=buf.device)
+    want = (buf.data_ptr() // buf.element_size()) % 64
+    have = (raw.data_ptr() // raw.element_size()) % 64
+    return raw[(want - have) % 64:][:n]
 
 
 class LocalBucketSync:
@@ -48,43 +67,187 @@ class LocalBucketSync:
 
     launcher(bucket_index, tensors, want_stats) -> stats row or None replaces the C-ABI
     call (CPU tests of the protocol inject a recorder); the default queues
-    ``jabas_sync_bucket`` on VSW 0's stream.
+    ``jabas_sync_bucket`` on the launch stream.
     """
 
-    def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False):
+    def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
+                 optimizer=None):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
         (one ramp-up and drain: 0.68 ms against 0.9 ms wall for the 14 buckets of ViT-B/16) and less host
-        time, and the buckets hold the aggregate only after ``finish_step``."""
+        time, and the buckets hold the aggregate only after ``finish_step``.
+
+        stream: the stream the fused launches are queued on (the reference's dedicated optimizer
+        stream, jabas/train/trainer.py:328); default: the stream VSW 0's hooks run on.
+
+        opt + param_buckets: hyperparameter dictionary and, per bucket index, dict(param=, state1=,
+        state2=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket; the launch of
+        such a bucket also runs the optimizer. ``optimizer=`` (or ``bind_optimizer``) takes a
+        torch.optim.SGD / Adam / AdamW or Shard* object instead and builds those arenas itself from the
+        ``parameters()`` / ``gradients()`` of the bucket objects the hooks publish."""
         if deferred and launcher is not None:
             raise ValueError("the deferred mode drives the C ABI itself: no launcher can be injected")
         self.deferred = bool(deferred)
         self._ready = {}                       # deferred mode: bucket index -> complete _Slot of this step
-        self._vsw_streams = {}                 # deferred mode: VSW index -> the stream its hooks ran on
+        self._vsw_streams = {}                 # VSW index -> the stream its hooks ran on in this step
         self._plan = self._plan_key = None
         self.batches = tuple(batches)
         self.K = len(self.batches)
         self.opt = opt
-        self.param_buckets = param_buckets or {}     # bucket index -> dict(param=, state1=, state2=, bounds=, fanout=)
+        self.optimizer = None
+        self.param_buckets = dict(param_buckets or {})   # bucket index -> dict(param=, state1=, state2=, bounds=, fanout=, agg_out=)
         self.step_count = 0
         self.lr_scale = 1.0
         self.accumulations = 1                 # micro-batches each VSW summed into its buckets (no_sync() steps + 1)
+        self.grad_clip = float("inf")          # per-bucket norm bound (ShardGNMTAdam's grad_clip)
         self._launcher = launcher or self._launch_fused
         self._lock = threading.Lock()
         self._slots = {}
         self._main_stream = None
-        self._calls = {}                       # bucket index -> prepared sync.BucketCall
+        self._sync_stream = stream
+        self._calls = {}                       # bucket index -> prepared sync.BucketCall(s)
         self._args_cache = {}
         self._launch_streams = set()           # streams that carry launches of the current step
         self._errors = []
+        self._momentum_ready = False           # SGD: the momentum buffers hold a first step
+        self._bound_steps = []                 # optimizer.state dictionaries whose 'step' follows step_count
         self.launched = 0                      # fused launches queued so far
+        self.launched_with_opt = 0             # of them, launches that updated weights
+        if optimizer is not None:
+            self.bind_optimizer(optimizer)
+
+    # ------------------------------------------------------------------ optimizer binding
+    def bind_optimizer(self, optimizer):
+        """The optimizer object whose update the fused launches perform (overlap weight-sync mode).
+        Hyperparameters are read from its ``param_groups`` at every step, so learning-rate policies and
+        torch schedulers act on it as usual; its state dictionaries hold views of the state arenas; its
+        own ``step`` is not called. A ``grad_clip`` attribute (ShardGNMTAdam,
+        examples/gnmt/seq2seq/train/shard_optimizer.py:8-29) bounds every bucket's gradient norm."""
+        from .train.trainer import opt_from_torch_optimizer
+        if self.optimizer is optimizer:
+            return self
+        if self.optimizer is not None:
+            raise RuntimeError("another optimizer is already bound")
+        self.opt = opt_from_torch_optimizer(optimizer)
+        self.optimizer = optimizer
+        self._group_of = {id(p): gi for gi, g in enumerate(optimizer.param_groups) for p in g["params"]}
+        self.grad_clip = float(getattr(optimizer, "grad_clip", float("inf")))
+        return self
+
+    def _refresh_hyperparameters(self):
+        if self.optimizer is None:
+            return
+        for mine, theirs in zip(self.opt["groups"], self.optimizer.param_groups):
+            mine["lr"] = float(theirs["lr"])
+            mine["weight_decay"] = float(theirs.get("weight_decay", 0.0))
+
+    def _bind_bucket(self, bucket_index, slot):
+        """Arenas for the weights and optimizer state of one bucket's parameters, laid out like the
+        bucket (built on the first launch of the bucket and again when DDP hands over other buffers, as
+        after its bucket rebuild). Module parameters, replica parameters and ``optimizer.state`` tensors
+        become views into the arenas, so the rest of the program keeps reading and writing them as
+        before. Runs on the thread that queues the launch, after every VSW has published the bucket:
+        each replica is past every use of these parameters in its backward pass."""
+        b0 = slot.buckets[0]
+        pb = self.param_buckets.get(bucket_index)
+        if self.optimizer is None or b0 is None or not hasattr(b0, "parameters"):
+            return pb
+        # the buffers and the parameters they carry, in order (a bucket packs them back to back): DDP's bucket
+        # rebuild frees the old buffers first, so new buckets can sit at old addresses with other contents
+        params = list(b0.parameters())
+        key = tuple(t.data_ptr() for t in slot.tensors) + (slot.tensors[0].numel(),) + tuple(id(p) for p in params)
+        if pb is not None and pb.get("_key") == key:
+            return pb
+        buf0 = slot.tensors[0]
+        es = buf0.element_size()
+        offs = [(g.data_ptr() - buf0.data_ptr()) // es for g in b0.gradients()]
+        n = buf0.numel()
+        for p, o in zip(params, offs):
+            if p.dtype != torch.float32:
+                raise TypeError("the fused update keeps fp32 weights")
+            if not 0 <= o <= n - p.numel():
+                raise RuntimeError(f"bucket {bucket_index}: a gradient view lies outside the bucket buffer")
+            if id(p) not in self._group_of:
+                raise ValueError(f"bucket {bucket_index} carries a parameter no group of the optimizer holds")
+        order = sorted(range(len(params)), key=lambda i: offs[i])
+        sgd = self.opt["kind"] == "sgd"
+        with torch.no_grad(), torch.cuda.stream(self._launch_stream()):
+            new = dict(_key=key, param=_arena_like(buf0), fanout=[])
+            if not sgd or self.opt.get("momentum", 0.0) != 0.0:
+                new["state1"] = _arena_like(buf0)
+            if not sgd:
+                new["state2"] = _arena_like(buf0)
+            if buf0.dtype != torch.float32:
+                new["agg_out"] = _arena_like(buf0)
+            names = ("momentum_buffer",) if sgd else ("exp_avg", "exp_avg_sq")
+            had_state = 0
+            for p, o in zip(params, offs):
+                view = new["param"][o:o + p.numel()].view(p.shape)
+                view.copy_(p.data)
+                p.data = view
+                st = self.optimizer.state[p]
+                for name, arena in zip(names, ("state1", "state2")):
+                    if arena not in new:
+                        continue
+                    sview = new[arena][o:o + p.numel()].view(p.shape)
+                    if torch.is_tensor(st.get(name)):
+                        sview.copy_(st[name])
+                        had_state += name != "exp_avg_sq"
+                    st[name] = sview
+                if not sgd:
+                    if "step" in st and int(float(st["step"])) != self.step_count:
+                        if self.launched_with_opt:
+                            raise RuntimeError("a parameter's Adam step count differs from the steps taken here")
+                        self.step_count = int(float(st["step"]))        # state carried in from earlier steps
+                    st["step"] = self.step_count
+                    self._bound_steps.append(st)
+            if sgd and had_state:
+                if had_state != len(params) and self.opt.get("dampening", 0.0) != 0.0:
+                    raise RuntimeError("some parameters of a bucket hold a momentum buffer and some do not: "
+                                       "with dampening the first step of the latter cannot share a launch")
+                self._momentum_ready = True
+            for k in range(1, self.K):
+                bk = slot.buckets[k]
+                if bk is None or not hasattr(bk, "parameters"):
+                    continue                                   # that replica's weights are not ours to refresh
+                bufk = slot.tensors[k]
+                peers = list(bk.parameters())
+                poffs = [(g.data_ptr() - bufk.data_ptr()) // es for g in bk.gradients()]
+                if poffs != offs or [q.shape for q in peers] != [p.shape for p in params]:
+                    raise RuntimeError(f"bucket {bucket_index}: VSW {k} lays its parameters out differently from VSW 0")
+                arena = _arena_like(buf0)
+                new["fanout"].append(arena)
+                for q, o in zip(peers, offs):
+                    view = arena[o:o + q.numel()].view(q.shape)
+                    view.copy_(q.data)
+                    q.data = view
+        bounds = []
+        for i in order:
+            gi = self._group_of[id(params[i])]
+            if not bounds:
+                bounds.append((0, gi))
+            elif bounds[-1][1] != gi:
+                bounds.append((offs[i], gi))
+        new["bounds"] = tuple(bounds)
+        new["params"] = params
+        self.param_buckets[bucket_index] = new
+        with self._lock:
+            self._calls.pop(bucket_index, None)
+            self._plan_key = None
+        return new
+
+    def aggregate_of(self, bucket_index):
+        """The fp32 aggregate of a reduced-precision bucket (fp32 buckets hold theirs in place)."""
+        pb = self.param_buckets.get(bucket_index) or {}
+        return pb.get("agg_out")
 
     # ------------------------------------------------------------------ hooks call this
-    def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None):
+    def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None, bucket=None):
         """Hands VSW k's bucket ``bucket_index`` over; the fused launch for that bucket is
         queued by whichever VSW hands its bucket over last. Returns a completed Future
-        carrying ``value`` (default the tensor)."""
+        carrying ``value`` (default the tensor). ``bucket``: the bucket object itself, whose
+        ``parameters()`` / ``gradients()`` place the weights when an optimizer is bound."""
         if not 0 <= k < self.K:
             raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
         fut = torch.futures.Future()
@@ -92,16 +255,16 @@ class LocalBucketSync:
         event = stream = None
         if tensor.is_cuda:
             stream = torch.cuda.current_stream(tensor.device)
-            if self.deferred:                  # ordered once per VSW stream in finish_step, not once per bucket
-                self._vsw_streams[k] = stream
-            elif k != 0:                       # VSW 0's stream is the one the launch is queued on
-                event = torch.cuda.Event()
+            if not self.deferred and (k != 0 or self._sync_stream is not None):
+                event = torch.cuda.Event()     # VSW 0's own stream needs none when the launch is queued on it
                 event.record(stream)
         with self._lock:
+            if stream is not None:
+                self._vsw_streams[k] = stream  # deferred mode orders once per VSW stream in finish_step
             slot = self._slots.setdefault(bucket_index, _Slot(self.K))
             if slot.tensors[k] is not None:
                 raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
-            slot.tensors[k], slot.events[k] = tensor, event
+            slot.tensors[k], slot.events[k], slot.buckets[k] = tensor, event, bucket
             slot.count += 1
             if k == 0:
                 slot.want_stats, slot.on_done = want_stats, on_done
@@ -109,22 +272,26 @@ class LocalBucketSync:
             ready = slot.count == self.K
             if ready:
                 del self._slots[bucket_index]
-        if ready:
-            if self.deferred:
-                with self._lock:
+                if self.deferred:
                     self._ready[bucket_index] = slot
-            else:
-                self._fire(bucket_index, slot)
+        if ready and not self.deferred:
+            self._fire(bucket_index, slot)
         return fut
 
+    def _launch_stream(self):
+        return self._sync_stream if self._sync_stream is not None else self._main_stream
+
     def _fire(self, bucket_index, slot):
-        main = self._main_stream
+        main = self._launch_stream()
         try:
             if main is not None:
-                for ev in slot.events[1:]:
-                    main.wait_event(ev)
+                for ev in slot.events:
+                    if ev is not None:
+                        main.wait_event(ev)
+                self._bind_bucket(bucket_index, slot)
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
-                self._launch_streams.add(main)
+                with self._lock:
+                    self._launch_streams.add(main)
             else:
                 row = self._launcher(bucket_index, slot.tensors, slot.want_stats)
         except Exception as exc:                       # reported by finish_step
@@ -137,37 +304,74 @@ class LocalBucketSync:
             self.launched += 1
 
     # ------------------------------------------------------------- the default launcher
-    def _step_args(self, dtype, want_stats, with_opt):
+    def _step_args(self, dtype, want_stats, with_opt, grad_scale=None, batches=None):
         """JabasStepArgs of this step, built once per (step, kind of launch) and shared by its buckets."""
-        key = (self.step_count, self.lr_scale, self.accumulations, dtype, bool(want_stats), bool(with_opt))
-        hit = self._args_cache.get(key)
-        if hit is None:
-            if len(self._args_cache) > 8:
-                self._args_cache.clear()
-            hit = self._args_cache[key] = sync.make_step_args(
-                self.batches, dtype, stats=want_stats, opt=self.opt if with_opt else None,
-                step=self.step_count + 1, first_step=self.step_count == 0, lr_scale=self.lr_scale,
-                accumulations=self.accumulations)
+        key = (self.step_count, self.lr_scale, self.accumulations, dtype, bool(want_stats), bool(with_opt),
+               None if grad_scale is None else grad_scale.data_ptr(), batches)
+        with self._lock:
+            hit = self._args_cache.get(key)
+            if hit is None:
+                if len(self._args_cache) > 64:
+                    self._args_cache.clear()
+                if with_opt and not self._args_cache_fresh:
+                    self._refresh_hyperparameters()
+                    self._args_cache_fresh = True
+                hit = self._args_cache[key] = sync.make_step_args(
+                    self.batches if batches is None else batches, dtype, stats=want_stats,
+                    opt=self.opt if with_opt else None, step=self.step_count + 1,
+                    first_step=not self._momentum_ready, lr_scale=self.lr_scale,
+                    accumulations=self.accumulations if batches is None else 1, grad_scale=grad_scale)
         return hit
 
+    _args_cache_fresh = False
+
     def _launch_fused(self, bucket_index, tensors, want_stats):
-        """Queues ``jabas_sync_bucket`` for one bucket on VSW 0's stream. DDP hands a hook the same
+        """Queues ``jabas_sync_bucket`` for one bucket on the launch stream. DDP hands a hook the same
         bucket buffers every step, so the prepared call (validated span, C struct, device bound table,
-        workspace) is kept per bucket and rebuilt only when the buffers change."""
-        call = self._calls.get(bucket_index)
+        workspace) is kept per bucket and rebuilt only when the buffers change.
+
+        With a finite ``grad_clip`` (the per-bucket clipping of ShardGNMTAdam.step,
+        examples/gnmt/seq2seq/train/shard_optimizer.py:75-76) the bucket takes two launches: aggregate +
+        statistics, the coefficient max_norm / (norm + 1e-6) on the device, then the update over the
+        aggregate scaled by it: the norm has to be known before any weight moves."""
+        main = self._launch_stream()
+        with self._lock:
+            call = self._calls.get(bucket_index)
         if call is None or not call.matches(tensors):
             span, with_opt = self._span_of(bucket_index, tensors)
-            call = self._calls[bucket_index] = sync.BucketCall(span)
-            call.with_opt = with_opt
-        args = self._step_args(tensors[0].dtype, want_stats, call.with_opt)
-        return call.run(args, stream=self._main_stream)
+            clipped = with_opt and self.grad_clip != float("inf")
+            if clipped:
+                agg_span = sync.SpanSpec(tensors, agg_out=span.agg_out)
+                call = sync.BucketCall(agg_span)
+                call.update = sync.BucketCall(sync.SpanSpec(
+                    [span.agg_out], agg_out=span.agg_out, param=span.param, state1=span.state1, state2=span.state2,
+                    fanout=span.fanout, bounds=span.bounds))
+                with torch.cuda.stream(main):
+                    call.coef = torch.ones(1, dtype=torch.float32, device=tensors[0].device)
+            else:
+                call = sync.BucketCall(span)
+            call.with_opt, call.clipped = with_opt, clipped
+            with self._lock:
+                self._calls[bucket_index] = call
+        if call.with_opt:
+            with self._lock:
+                self.launched_with_opt += 1
+        if not call.clipped:
+            return call.run(self._step_args(tensors[0].dtype, want_stats, call.with_opt), stream=main)
+        row = call.run(self._step_args(tensors[0].dtype, True, False), stream=main)
+        sync.clip_coef(row, self.grad_clip, out=call.coef, stream=main)
+        call.update.run(self._step_args(torch.float32, False, True, grad_scale=call.coef, batches=(1,)), stream=main)
+        return row if want_stats else None
 
     def _span_of(self, bucket_index, tensors):
         """(span over the K buffers of one bucket, whether the optimizer runs in the same launch)."""
         g0 = tensors[0]
         pb = self.param_buckets.get(bucket_index)
         opt = self.opt if pb is not None else None
-        span = sync.SpanSpec(tensors, agg_out=g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out"),
+        agg_out = g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out")
+        if opt is not None and self.grad_clip != float("inf") and agg_out is None:
+            raise ValueError("clipping a reduced-precision bucket needs an fp32 agg_out arena")
+        span = sync.SpanSpec(tensors, agg_out=agg_out,
                              param=pb and pb.get("param"), state1=pb and pb.get("state1"),
                              state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
                              bounds=(pb or {}).get("bounds", ()) if opt else ())
@@ -177,23 +381,36 @@ class LocalBucketSync:
         """Deferred mode: one planned launch over every bucket of the step, in bucket order."""
         with self._lock:
             ready, self._ready = self._ready, {}
+            vsw_streams = sorted(self._vsw_streams.items())
         order = sorted(ready)
         slots = [ready[i] for i in order]
-        with_opt = [self.opt is not None and i in self.param_buckets for i in order]
-        main = self._main_stream
-        if main is None or (any(with_opt) and not all(with_opt)):
-            for i, slot in zip(order, slots):          # host tensors (protocol tests), or buckets with and without
-                self._fire(i, slot)                    # weights behind them: one launch each after all
+        main = self._launch_stream()
+        if main is None:
+            for i, slot in zip(order, slots):          # host tensors (protocol tests)
+                self._fire(i, slot)
             return
         try:
-            # everything the other VSWs queued up to now (their whole backward) precedes the launch: one
+            # everything the VSWs queued up to now (their whole backward) precedes the launch: one
             # event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
             # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
-            for k, stream in sorted(self._vsw_streams.items()):
-                if k != 0 and stream != main:
+            for k, stream in vsw_streams:
+                if stream != main:
                     ev = torch.cuda.Event()
                     ev.record(stream)
                     main.wait_event(ev)
+            for i, slot in zip(order, slots):
+                self._bind_bucket(i, slot)
+        except Exception as exc:
+            with self._lock:
+                self._errors.append((order[0], exc))
+            return
+        with_opt = [self.opt is not None and i in self.param_buckets for i in order]
+        if (any(with_opt) and not all(with_opt)) or (with_opt[0] and self.grad_clip != float("inf")):
+            for i, slot in zip(order, slots):          # buckets with and without weights behind them, or a norm
+                slot.events = [None] * self.K          # per bucket to wait for: one launch each after all
+                self._fire(i, slot)
+            return
+        try:
             key = tuple((i, slot.tensors[0].numel()) + tuple(t.data_ptr() for t in slot.tensors)
                         for i, slot in zip(order, slots))
             if key != self._plan_key:                   # DDP hands over the same buffers every step: built once
@@ -203,10 +420,13 @@ class LocalBucketSync:
             want = any(slot.want_stats for slot in slots)
             args = self._step_args(slots[0].tensors[0].dtype, want, with_opt[0])
             rows = self._plan.run(args, stream=main)
+            if with_opt[0]:
+                self.launched_with_opt += 1
             if rows is not None:
                 with torch.cuda.stream(main):
                     rows = rows.clone()                 # the plan's own rows are overwritten by its next launch
-            self._launch_streams.add(main)
+            with self._lock:
+                self._launch_streams.add(main)
         except Exception as exc:
             with self._lock:
                 self._errors.append((order[0], exc))
@@ -222,26 +442,46 @@ class LocalBucketSync:
         with self._lock:
             return sorted(self._slots)
 
+    def reset(self):
+        """Forgets the buckets of an unfinished step (after an error), so that the next step starts clean."""
+        with self._lock:
+            self._slots.clear()
+            self._ready.clear()
+            self._launch_streams = set()
+            self._vsw_streams = {}
+            self._errors = []
+
     def finish_step(self, streams=()):
         """End of a sync step: every VSW stream waits for the fused launches that read its
-        buckets, and the step count (Adam's t, SGD's first-step flag) advances."""
+        buckets (and, with an optimizer bound, write its weights), and the step count (Adam's t, SGD's
+        first-step flag) advances. ``streams``: the VSW streams; default: the streams the hooks of this
+        step ran on."""
         left = self.pending()
         if left:
+            self.reset()
             raise RuntimeError(f"buckets {left} were not published by every VSW")
         if self._ready:
             self._fire_all()
-        # the launches of a step sit on VSW 0's stream in order: one event behind the last of them orders
+        # the launches of a step sit on one stream in order: one event behind the last of them orders
         # every VSW stream behind all of them
-        launch_streams, self._launch_streams = self._launch_streams, set()
+        with self._lock:
+            launch_streams, self._launch_streams = self._launch_streams, set()
+            recorded, self._vsw_streams = self._vsw_streams, {}
+            errors, self._errors = self._errors, []
+            self._args_cache_fresh = False
+        streams = tuple(streams) or tuple(recorded.values())
         for main in launch_streams:
             done = torch.cuda.Event()
             done.record(main)
             for s in streams:
                 if s != main:
                     s.wait_event(done)
-        with self._lock:
-            errors, self._errors = self._errors, []
         if errors:
             idx, exc = errors[0]
+            self.reset()
             raise RuntimeError(f"fused launch of bucket {idx} failed: {exc}") from exc
         self.step_count += 1
+        if self.launched_with_opt:
+            self._momentum_ready = True
+        for st in self._bound_steps:
+            st["step"] = self.step_count

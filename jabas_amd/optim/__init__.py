@@ -1,3 +1,3 @@
-from .shard import ShardSGD, ShardAdam, ShardAdamW
+from .shard import ShardSGD, ShardAdam, ShardAdamW, ShardGNMTAdam
 
-__all__ = ["ShardSGD", "ShardAdam", "ShardAdamW"]
+__all__ = ["ShardSGD", "ShardAdam", "ShardAdamW", "ShardGNMTAdam"]

@@ -118,6 +118,9 @@ class _ShardOptimizer(torch.optim.Optimizer):
         a.weight[0] = 1.0                       # g * 1.0f is exact: the gradient goes in unchanged
         a.half_weight[0] = 1.0
         a.opt_kind = kind
+        scale = getattr(self, "_grad_scale", None)
+        if scale is not None:                   # device scalar of a clipped step
+            a.grad_scale = scale.data_ptr()
         return a
 
 
@@ -294,3 +297,57 @@ class ShardAdamW(ShardAdam):
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=1e-2, amsgrad=False):
         super().__init__(params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=amsgrad)
+
+
+class ShardGNMTAdam(ShardAdam):
+    """ShardAdam with gradient clipping inside ``step`` (examples/gnmt/seq2seq/train/shard_optimizer.py:8-90):
+    the gradients handed to one ``step(gradients)`` call (one DDP bucket in the overlap mode) are scaled to a
+    joint 2-norm of at most ``grad_clip`` before the update, torch.nn.utils.clip_grad_norm_'s rule
+    (coefficient max_norm / (norm + 1e-6), applied when below 1). One statistics launch over the gradients
+    forms the norm, the coefficient stays on the device, and the Adam launch multiplies it in; the gradient
+    buffers themselves are left as they were."""
+
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0, amsgrad=False,
+                 grad_clip=float('inf')):
+        super().__init__(params, lr=lr, betas=betas, eps=eps, weight_decay=weight_decay, amsgrad=amsgrad)
+        self.grad_clip = grad_clip
+        self._clip_plans = {}
+        self._coef = None
+        if len(self.param_groups) > 1:
+            raise ValueError(
+                "Length of self.param_groups must not be > 1 "
+                "because of applying gradient clipping")
+
+    @torch.no_grad()
+    def step(self, gradients=None, closure=None):
+        if self.grad_clip == float('inf'):
+            return super().step(gradients, closure)
+        pairs = self._pairs(gradients)
+        if not pairs:
+            return super().step(gradients, closure)
+        flat = []
+        for _, p, g in pairs:
+            if g.is_sparse:
+                raise RuntimeError('Adam does not support sparse gradients, please consider SparseAdam instead')
+            if not p.is_cuda:
+                raise RuntimeError(f"{type(self).__name__} updates GPU parameters only (no CPU fallback)")
+            g = g.detach()
+            flat.append((g if g.is_contiguous() else g.contiguous()).view(-1))
+        sig = tuple((g.data_ptr(), g.numel()) for g in flat)
+        plan = self._clip_plans.get(sig)
+        if plan is None:
+            if len(self._clip_plans) >= self._max_cached_plans:
+                self._clip_plans.clear()
+            plan = self._clip_plans[sig] = sync.SyncPlan([sync.SpanSpec([g]) for g in flat], L.OPT_NONE)
+        args = L.JabasStepArgs()
+        args.K, args.grad_dtype, args.stats, args.opt_kind = 1, L.F32, 1, L.OPT_NONE
+        args.weight[0] = args.half_weight[0] = 1.0
+        rows = plan.run(args)
+        if self._coef is None:
+            self._coef = torch.ones(1, dtype=torch.float32, device=flat[0].device)
+        sync.clip_coef(rows, self.grad_clip, out=self._coef)
+        self._grad_scale = self._coef
+        try:
+            return super().step(gradients, closure)
+        finally:
+            self._grad_scale = None

@@ -33,13 +33,29 @@ from .. import sync
 
 
 def create_optimizer_hook(hook, optimizer):
-    """Counterpart of IIDPTrainer._create_optimizer_hook (call site
-    jabas/train/trainer.py:332): run ``hook`` and, once its Future resolves, apply
-    ``optimizer.step(gradients)`` to the parameters of that bucket. Gradients are taken
-    from ``bucket.gradients()`` / ``bucket.parameters()`` (torch >= 1.10 GradBucket) and
-    tagged with ``.index`` the way the reference matches them
+    """Counterpart of IIDPTrainer._create_optimizer_hook (call site jabas/train/trainer.py:332): the
+    hook VSW 0 registers in the overlap weight-sync mode, which updates the parameters of a bucket as
+    soon as the bucket's gradients are synchronised.
+
+    With a ``LocalBucketSync`` attached to the state (K VSWs on the GPU) the optimizer is bound to it and
+    the update is part of the fused launch the rendezvous queues for that bucket, when the last VSW has
+    handed its bucket over, on the rendezvous' launch stream: aggregate, ``optimizer``'s update rule and
+    the refresh of the other replicas' weights in one pass. ``optimizer.step`` itself is never called;
+    its ``param_groups`` supply the hyperparameters at every step and its ``state`` shows the arenas.
+    Calling ``optimizer.step`` on this thread right after ``hook`` would read VSW 0's own bucket before
+    the other VSWs' gradients are in it.
+
+    Without a rendezvous (state None or a one-worker state) the bucket already holds the final gradient
+    when the hook's Future resolves, and ``optimizer.step(gradients)`` runs then, gradients tagged with
+    the ``.index`` of their parameters the way the reference matches them
     (examples/gnmt/seq2seq/train/shard_optimizer.py:41-46)."""
     def hook_then_step(state, bucket):
+        local = getattr(state, "local", None)
+        if local is not None:
+            local.bind_optimizer(optimizer)
+            return hook(state, bucket)
+        if getattr(state, "total_num_decoupled_workers", 1) != 1:
+            raise RuntimeError("create_optimizer_hook: several workers but no LocalBucketSync attached to the state")
         fut = hook(state, bucket)
 
         def run(done):
@@ -54,6 +70,32 @@ def create_optimizer_hook(hook, optimizer):
 
         return fut.then(run)
     return hook_then_step
+
+
+def create_stream_for_optimizer(device=None):
+    """Counterpart of IIDPTrainer._create_stream_for_optimizer (call site jabas/train/trainer.py:328): the
+    stream the weight updates of the overlap mode run on, apart from every VSW's own stream, so that a
+    bucket's update overlaps the rest of the backward passes. Default priority."""
+    return torch.cuda.Stream(device)
+
+
+def prepare_overlap_optimizer_with_ddp(local_models, states, hooks, optimizer, local):
+    """jabas/train/trainer.py:327-333 for one GPU: a launch stream of its own for ``local`` (the GPU's
+    LocalBucketSync) unless it has one, the optimizer hook on VSW 0, every other VSW's hook as it is.
+    ``local_models`` are the K DistributedDataParallel replicas (built with
+    ``gradient_as_bucket_view=True``: the fused launch writes the aggregate into the bucket, and only a
+    ``.grad`` that is a view of the bucket sees it)."""
+    if local._sync_stream is None:
+        p = next(iter(local_models[0].parameters()))
+        local._sync_stream = create_stream_for_optimizer(p.device)
+    for i, (model, state, hook) in enumerate(zip(local_models, states, hooks)):
+        if getattr(model, "gradient_as_bucket_view", True) is False:
+            raise ValueError("build the DistributedDataParallel replicas with gradient_as_bucket_view=True")
+        if i == 0:
+            local.bind_optimizer(optimizer)
+            hook = create_optimizer_hook(hook, optimizer)
+        model.register_comm_hook(state=state, hook=hook)
+    return local
 
 
 def tag_parameter_indices(model):

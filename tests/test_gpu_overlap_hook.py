@@ -1,0 +1,303 @@
+"""GPU parity of the overlap weight-sync mode (jabas/train/trainer.py:327-333): the optimizer hook on
+VSW 0. K hook threads on K streams publish their buckets; the fused launch of a bucket (queued by the
+last VSW to arrive, on a launch stream of its own) aggregates, updates the weights of that bucket's
+parameters and refreshes the other replicas. Everything is compared bit for bit with the CPU oracle's
+``sync_step`` over several steps: aggregate, weights, optimizer state, replica weights.
+VSW 0 publishes FIRST in every case, so an update that ran at VSW 0's hook time would see its own
+un-aggregated bucket and fail here.
+"""
+import math
+import threading
+
+import pytest
+import torch
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(t):
+    t = t.detach().cpu().contiguous()
+    return t.view({8: torch.int64, 4: torch.int32, 2: torch.int16}[t.element_size()])
+
+
+def _same(a, b):
+    return torch.equal(_bits(a.reshape(-1)), _bits(b.reshape(-1)))
+
+
+class ParamBucket:
+    """What a comm hook is handed: index(), buffer(), parameters(), gradients() (views of the buffer)."""
+
+    def __init__(self, i, buf, params, offs):
+        self._i, self._buf, self._params, self._offs = i, buf, params, offs
+
+    def index(self):
+        return self._i
+
+    def buffer(self):
+        return self._buf
+
+    def parameters(self):
+        return list(self._params)
+
+    def gradients(self):
+        return [self._buf[o:o + p.numel()].view(p.shape) for p, o in zip(self._params, self._offs)]
+
+
+# three buckets; 1-D tensors (group 0: no weight decay) and matrices (group 1) alternate, odd sizes so
+# that group changes fall inside 16-byte vectors and tiles
+SHAPES = [[(33,), (129, 61), (61,), (70, 70)], [(5,)], [(300, 257), (257,), (3, 3), (9,), (1000, 41)]]
+
+
+def _opt_dict(kind):
+    if kind == "sgd":
+        return dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+                    groups=[dict(lr=0.1, weight_decay=0.0), dict(lr=0.1, weight_decay=1e-4)])
+    return dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+                groups=[dict(lr=5e-4, weight_decay=0.0), dict(lr=5e-4, weight_decay=0.05)])
+
+
+def _torch_optimizer(kind, params):
+    groups = [{"params": [p for p in params if p.dim() <= 1], "weight_decay": 0.0},
+              {"params": [p for p in params if p.dim() > 1], "weight_decay": 1e-4 if kind == "sgd" else 0.05}]
+    if kind == "sgd":
+        return torch.optim.SGD(groups, lr=0.1, momentum=0.9)
+    return torch.optim.AdamW(groups, lr=5e-4)
+
+
+def _layout(shapes):
+    offs, bounds, o = [], [], 0
+    for s in shapes:
+        n = math.prod(s)
+        g = 0 if len(s) <= 1 else 1
+        if not bounds or bounds[-1][1] != g:
+            bounds.append((o if bounds else 0, g))
+        offs.append(o)
+        o += n
+    return offs, tuple(bounds), o
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("deferred", [False, True])
+def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, deferred):
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
+
+    K, batches = 3, (4, 2, 2)
+    opt = _opt_dict(kind)
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    # K replicas of the "model": one Parameter per tensor, the same initial values
+    gen = torch.Generator().manual_seed(5)
+    init = [[torch.randn(s, generator=gen) * 0.05 for s in shapes] for shapes in SHAPES]
+    replicas = [[[torch.nn.Parameter(t.clone().to(gpu)) for t in bucket] for bucket in init] for _ in range(K)]
+    layouts = [_layout(shapes) for shapes in SHAPES]
+    bufs = [[torch.zeros(n, dtype=gdt, device=gpu) for _ in range(K)] for (_, _, n) in layouts]
+    optimizer = _torch_optimizer(kind, [p for bucket in replicas[0] for p in bucket])
+    local = LocalBucketSync(batches, deferred=deferred, stream=create_stream_for_optimizer(gpu))
+    st = H.GradientSimilarityState(None, 4, None, [], 2).attach_local(local)
+    main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
+    # the oracle's flat state per bucket
+    p_h = [torch.cat([t.reshape(-1) for t in bucket]) for bucket in init]
+    s1_h = [torch.zeros_like(p) for p in p_h]
+    s2_h = [torch.zeros_like(p) for p in p_h]
+    gate = [threading.Event() for _ in range(len(SHAPES))]
+    for step in range(1, 4):
+        local.lr_scale = (1.0, math.sqrt(20 / 8), 0.75)[step - 1]              # the adaptive-batching modifier moves
+        host = [[(torch.randn(n, generator=torch.Generator().manual_seed(1000 * step + 10 * b + k)) * 1e-3).to(gdt)
+                 for k in range(K)] for b, (_, _, n) in enumerate(layouts)]
+        for g in gate:
+            g.clear()
+        errors = []
+
+        def vsw(k):
+            try:
+                with torch.cuda.stream(streams[k]):
+                    order = range(len(SHAPES)) if k % 2 == 0 else reversed(range(len(SHAPES)))
+                    for b in order:
+                        if k != 0:
+                            gate[b].wait(30)                                    # VSW 0 always hands its bucket over first
+                        bufs[b][k].copy_(host[b][k].to(gpu))                    # "backward" fills the bucket on this stream
+                        bucket = ParamBucket(b, bufs[b][k], replicas[k][b], layouts[b][0])
+                        if k == 0:
+                            main_hook(st, bucket).wait()
+                            gate[b].set()
+                        else:
+                            H.dummy_hook(H.VSWPeerState(local, k), bucket).wait()
+            except Exception as exc:                                            # pragma: no cover - reported below
+                errors.append(exc)
+                for g in gate:
+                    g.set()
+
+        threads = [threading.Thread(target=vsw, args=(k,), daemon=True) for k in range(K)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(60)
+        assert not errors, errors
+        local.finish_step()
+        torch.cuda.synchronize()
+        want_stats = st.step % st.interval == 0
+        for b, (offs, bounds, n) in enumerate(layouts):
+            agg_h, rows_h = O.sync_step(host[b], batches, [(0, n, bounds)], opt, p_h[b], s1_h[b], s2_h[b], step=step,
+                                        first_step=(step == 1), want_stats=want_stats, lr_scale=local.lr_scale)
+            agg_d = bufs[b][0] if gdt == torch.float32 else local.aggregate_of(b)
+            assert _same(agg_d, agg_h), (step, b, "aggregate")
+            for i, (p, o) in enumerate(zip(replicas[0][b], offs)):
+                sl = slice(o, o + p.numel())
+                assert _same(p.data, p_h[b][sl]), (step, b, i, "weights")
+                state = optimizer.state[p]
+                if kind == "sgd":
+                    assert _same(state["momentum_buffer"], s1_h[b][sl]), (step, b, i, "momentum")
+                else:
+                    assert _same(state["exp_avg"], s1_h[b][sl]) and _same(state["exp_avg_sq"], s2_h[b][sl]), (step, b, i)
+                    assert int(state["step"]) == step
+                for k in range(1, K):
+                    assert _same(replicas[k][b][i].data, p.data), (step, b, i, k, "replica")
+            for k in range(1, K):                                               # the peers' buckets are only read
+                assert _same(bufs[b][k], host[b][k])
+        if want_stats:
+            rows = {s.index: s.cpu() for s in st.grad_placeholder}
+            assert sorted(rows) == [0, 1, 2]
+            for b, (_, _, n) in enumerate(layouts):
+                want = O.stats(host[b], batches)
+                tol = 1e-6 if gdt == torch.float32 else 1e-2
+                assert torch.allclose(rows[b][:4 + K], want[:4 + K], rtol=tol, atol=0.0)
+        else:
+            assert st.grad_placeholder == []
+        st.grad_placeholder.clear()
+        st.step += 1
+    assert local.launched == 3 * (1 if deferred else len(SHAPES))
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adam"])
+def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
+    """The arenas handed over by the caller (``opt=`` + ``param_buckets=``) instead of built from bucket
+    objects: views into one weight arena, one state arena each, two parameter groups, one replica."""
+    from jabas_amd.local_sync import LocalBucketSync
+    K, batches, sizes = 2, (3, 1), [70001, 2049]
+    opt = _opt_dict("sgd") if kind == "sgd" else dict(kind="adam", betas=(0.9, 0.999), eps=1e-8,
+                                                     groups=[dict(lr=2e-3, weight_decay=0.0),
+                                                             dict(lr=1e-3, weight_decay=1e-2)])
+    total = sum(sizes)
+    gen = torch.Generator().manual_seed(9)
+    p_h = torch.randn(total, generator=gen) * 0.05
+    s1_h, s2_h = torch.zeros(total), torch.zeros(total)
+    p_d, s1_d, s2_d, fan = p_h.to(gpu), s1_h.to(gpu), s2_h.to(gpu), torch.zeros(total, device=gpu)
+    spans, pbs, off = [], {}, 0
+    for b, n in enumerate(sizes):
+        bounds = ((0, 0), (n // 3, 1), (2 * n // 3 + 1, 0))
+        sl = slice(off, off + n)
+        pbs[b] = dict(param=p_d[sl], state1=s1_d[sl], state2=None if kind == "sgd" else s2_d[sl], bounds=bounds,
+                      fanout=[fan[sl]])
+        spans.append((off, n, bounds))
+        off += n
+    local = LocalBucketSync(batches, opt=opt, param_buckets=pbs)
+    bufs = [torch.zeros(total, device=gpu) for _ in range(K)]
+    for step in range(1, 4):
+        host = [torch.randn(total, generator=torch.Generator().manual_seed(50 * step + k)) * 1e-3 for k in range(K)]
+        for k in range(K):
+            bufs[k].copy_(host[k])
+        for b, (o, n, _) in enumerate(spans):
+            for k in (0, 1):                                                    # VSW 0 first
+                local.publish(k, b, bufs[k][o:o + n])
+        local.finish_step()
+        torch.cuda.synchronize()
+        agg_h, _ = O.sync_step(host, batches, spans, opt, p_h, s1_h, s2_h, step=step, first_step=(step == 1))
+        assert _same(bufs[0], agg_h) and _same(p_d, p_h) and _same(s1_d, s1_h) and _same(fan, p_h), step
+        if kind != "sgd":
+            assert _same(s2_d, s2_h), step
+
+
+def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
+    """ShardGNMTAdam(grad_clip=) in the hook (examples/gnmt/seq2seq/train/shard_optimizer.py:8-29,75-76):
+    every bucket's aggregate is scaled to norm <= grad_clip before Adam sees it. Oracle: the aggregate,
+    torch.nn.utils.clip_grad_norm_'s coefficient from its float64 norm, one fp32 product, Adam."""
+    from jabas_amd import ddp_comm_hooks as H, optim
+    from jabas_amd.local_sync import LocalBucketSync
+    from jabas_amd.train import create_optimizer_hook
+    K, batches = 2, (128, 64)
+    shapes = [[(257, 33), (33,)], [(4000,)]]
+    gen = torch.Generator().manual_seed(3)
+    init = [[torch.randn(s, generator=gen) * 0.05 for s in bucket] for bucket in shapes]
+    replicas = [[[torch.nn.Parameter(t.clone().to(gpu)) for t in bucket] for bucket in init] for _ in range(K)]
+    layouts = [_layout(bucket) for bucket in shapes]
+    bufs = [[torch.zeros(n, device=gpu) for _ in range(K)] for (_, _, n) in layouts]
+    clip = 0.05
+    optimizer = optim.ShardGNMTAdam([p for bucket in replicas[0] for p in bucket], lr=2e-3, grad_clip=clip)
+    opt = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, groups=[dict(lr=2e-3, weight_decay=0.0)])
+    local = LocalBucketSync(batches)
+    st = H.IIDPState(None, 2).attach_local(local)
+    main_hook = create_optimizer_hook(H.iidp_allreduce_hook, optimizer)
+    p_h = [torch.cat([t.reshape(-1) for t in bucket]) for bucket in init]
+    s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
+    clipped_any = kept_any = False
+    for step in range(1, 4):
+        scale = (1e-3, 1e-5, 1e-3)[step - 1]                                   # step 2 stays under the bound
+        host = [[torch.randn(n, generator=torch.Generator().manual_seed(77 * step + 5 * b + k)) * scale
+                 for k in range(K)] for b, (_, _, n) in enumerate(layouts)]
+        for b in range(len(shapes)):
+            for k in range(K):
+                bufs[b][k].copy_(host[b][k])
+                bucket = ParamBucket(b, bufs[b][k], replicas[k][b], layouts[b][0])
+                (main_hook(st, bucket) if k == 0 else H.dummy_hook(H.VSWPeerState(local, k), bucket)).wait()
+        local.finish_step()
+        torch.cuda.synchronize()
+        for b, (offs, _, n) in enumerate(layouts):
+            agg = O.aggregate(host[b], batches)
+            agg, c = O.clip(agg, clip)
+            clipped_any, kept_any = clipped_any or c < 1.0, kept_any or c >= 1.0
+            O.opt_step(opt, 0, p_h[b], agg, s1_h[b], s2_h[b], step, step == 1)
+            assert _same(bufs[b][0], agg), (step, b, "clipped aggregate")
+            for i, (p, o) in enumerate(zip(replicas[0][b], offs)):
+                assert _same(p.data, p_h[b][o:o + p.numel()]), (step, b, i)
+                assert _same(replicas[1][b][i].data, p.data)
+    assert clipped_any and kept_any
+
+
+def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
+    """ShardGNMTAdam.step(gradients) outside any hook: torch.nn.utils.clip_grad_norm_ over the gradients
+    of the call, then torch.optim.Adam, is the library statement of the same step (1e-6; the oracle's
+    sequence bit for bit)."""
+    from jabas_amd import optim
+    from jabas_amd.train.trainer import tag_parameter_indices
+    torch.manual_seed(0)
+    model = tag_parameter_indices(torch.nn.Sequential(torch.nn.Linear(40, 50), torch.nn.Linear(50, 7)).to(gpu))
+    ref = torch.nn.Sequential(torch.nn.Linear(40, 50), torch.nn.Linear(50, 7)).to(gpu)
+    ref.load_state_dict(model.state_dict())
+    mine = optim.ShardGNMTAdam(model.parameters(), lr=2e-3, grad_clip=5e-3)
+    theirs = torch.optim.Adam(ref.parameters(), lr=2e-3, foreach=False)
+    params = list(model.parameters())
+    p_h = [p.detach().cpu().clone().reshape(-1) for p in params]
+    m_h, v_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
+    opt = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, groups=[dict(lr=2e-3, weight_decay=0.0)])
+    flat = torch.zeros(sum(p.numel() for p in params), device=gpu)            # one "bucket"
+    for step in range(1, 5):
+        scale = (1e-3, 1e-6, 1e-3, 1e-2)[step - 1]                             # step 2 stays under the bound
+        host = torch.randn(flat.numel(), generator=torch.Generator().manual_seed(step)) * scale
+        flat.copy_(host)
+        grads, off = [], 0
+        for p, rp in zip(params, ref.parameters()):
+            v = flat[off:off + p.numel()].view(p.shape)
+            v.index = p.index
+            grads.append(v)
+            rp.grad = v.detach().clone()
+            off += p.numel()
+        mine.step(grads)
+        torch.nn.utils.clip_grad_norm_(ref.parameters(), 5e-3)
+        theirs.step()
+        torch.cuda.synchronize()
+        clipped, c = O.clip(host, 5e-3)
+        assert (c < 1.0) == (step != 2)
+        off = 0
+        for i, (p, rp) in enumerate(zip(params, ref.parameters())):
+            n = p.numel()
+            O.opt_step(opt, 0, p_h[i], clipped[off:off + n], m_h[i], v_h[i], step, step == 1)
+            off += n
+            assert _same(p.data, p_h[i]), (step, i)
+            assert torch.allclose(p.data, rp.data, rtol=1e-6, atol=1e-8), (step, i)
+        assert _same(flat, host)                                                # the gradient buffers are left alone
+    with pytest.raises(ValueError, match="param_groups"):
+        optim.ShardGNMTAdam([{"params": params[:1]}, {"params": params[1:]}], grad_clip=1.0)

@@ -201,12 +201,18 @@ def test_threads_in_random_order_over_many_buckets():
 def test_finish_step_reports_missing_vsws_and_double_publish_is_an_error():
     local = LocalBucketSync([1, 1], launcher=Recorder())
     local.publish(0, 3, torch.ones(2))
-    with pytest.raises(RuntimeError, match="not published"):
-        local.finish_step()
     with pytest.raises(RuntimeError, match="twice"):
         local.publish(0, 3, torch.ones(2))
     with pytest.raises(ValueError):
         local.publish(2, 3, torch.ones(2))
+    with pytest.raises(RuntimeError, match="not published"):
+        local.finish_step()
+    # a failed step leaves nothing behind: the next one starts clean
+    assert local.pending() == [] and local.step_count == 0
+    local.publish(0, 3, torch.ones(2))
+    local.publish(1, 3, torch.ones(2))
+    local.finish_step()
+    assert local.step_count == 1
 
 
 def test_launcher_failure_is_reported_at_the_end_of_the_step():

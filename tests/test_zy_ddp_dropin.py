@@ -2,8 +2,9 @@
 DistributedDataParallel (gradient_as_bucket_view=True, one process group of size 1),
 driven by K threads on K streams as IIDP drives its VSWs. VSW 0 registers the similarity
 hook, the others dummy_hook with a VSWPeerState (jabas/train/trainer.py:452-468); the real
-GradBucket objects DDP hands to the hooks go through the fused launch. Checked against a
-plain-torch batch-weighted aggregate of the same per-replica gradients.
+GradBucket objects DDP hands to the hooks go through the fused launch. Checked bit for bit
+against the CPU oracle fed with the very gradient bits every replica's backward left in its
+bucket (VSW 0's bucket is copied by a recording hook before the launch overwrites it).
 Collected late: it initialises a process group."""
 import os
 import threading
@@ -19,78 +20,188 @@ pytestmark = pytest.mark.gpu
 
 def _model(seed):
     torch.manual_seed(seed)
-    return torch.nn.Sequential(torch.nn.Linear(64, 256), torch.nn.ReLU(), torch.nn.Linear(256, 256), torch.nn.ReLU(),
-                               torch.nn.Linear(256, 16))
+    return torch.nn.Sequential(torch.nn.Linear(64, 256), torch.nn.ReLU(), torch.nn.Linear(256, 255), torch.nn.ReLU(),
+                               torch.nn.Linear(255, 16))
+
+
+def _bits(t):
+    return t.detach().cpu().contiguous().reshape(-1).view(torch.int32)
+
+
+def _init_pg():
+    if not dist.is_initialized():
+        os.environ.setdefault("MASTER_ADDR", "127.0.0.1")
+        os.environ.setdefault("MASTER_PORT", "29517")
+        dist.init_process_group("nccl", rank=0, world_size=1)
+
+
+def _replicas(gpu, K, streams):
+    from torch.nn.parallel import DistributedDataParallel as DDP
+    out = []
+    for k in range(K):
+        with torch.cuda.stream(streams[k]):
+            out.append(DDP(_model(0).to(gpu), device_ids=[gpu.index], gradient_as_bucket_view=True, bucket_cap_mb=0.1))
+    torch.cuda.synchronize()
+    return out
+
+
+class Recorder:
+    """Wraps VSW 0's hook: keeps a copy of every bucket as backward left it, and which parameters it
+    carries where (the launch aggregates in place into that bucket). ``hook`` is what DDP registers."""
+
+    def __init__(self, inner, model):
+        self.index_of = {id(p): i for i, p in enumerate(model.parameters())}
+        self.seen = {}
+
+        def recording_hook(state, bucket):
+            buf = bucket.buffer()
+            offs = [(g.data_ptr() - buf.data_ptr()) // 4 for g in bucket.gradients()]
+            self.seen[bucket.index()] = (buf.clone(), [self.index_of[id(p)] for p in bucket.parameters()], offs)
+            return inner(state, bucket)
+
+        self.hook = recording_hook
+
+
+def _backward_all(replicas, streams, data, crit):
+    K = len(replicas)
+    errors, losses = [], []
+    # forward passes one after the other (DDP's forward may use the process group: bucket
+    # rebuild after the first step); backward passes concurrently, one thread per VSW
+    for k in range(K):
+        with torch.cuda.stream(streams[k]):
+            replicas[k].zero_grad(set_to_none=False)
+            losses.append(crit(replicas[k](data[k][0]), data[k][1]))
+
+    def run(k):
+        try:
+            with torch.cuda.stream(streams[k]):
+                losses[k].backward()
+        except Exception as exc:                      # pragma: no cover - reported below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=run, args=(k,), daemon=True) for k in range(K)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=60)
+    assert not errors, errors
+    assert not any(t.is_alive() for t in threads), "a VSW thread is stuck in backward"
+
+
+def _per_parameter_grads(rec, replicas):
+    """[k][i]: gradient of parameter i as VSW k's backward produced it (host)."""
+    n = len(rec.index_of)
+    out = [[None] * n for _ in replicas]
+    for (buf, idxs, offs) in rec.seen.values():
+        for i, o in zip(idxs, offs):
+            out[0][i] = buf[o:o + list(replicas[0].module.parameters())[i].numel()].cpu()
+    for k in range(1, len(replicas)):
+        for i, p in enumerate(replicas[k].module.parameters()):
+            out[k][i] = p.grad.detach().reshape(-1).cpu()
+    return out
 
 
 def test_stock_ddp_buckets_through_the_hooks(gpu):
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
-    from torch.nn.parallel import DistributedDataParallel as DDP
 
-    if not dist.is_initialized():
-        os.environ.setdefault("MASTER_ADDR", "127.0.0.1")
-        os.environ.setdefault("MASTER_PORT", "29517")
-        dist.init_process_group("nccl", rank=0, world_size=1)
+    _init_pg()
     K, batches = 2, (6, 2)
     crit = torch.nn.MSELoss()
     streams = [torch.cuda.Stream(gpu) for _ in range(K)]
-    replicas = []
-    for k in range(K):
-        with torch.cuda.stream(streams[k]):
-            replicas.append(DDP(_model(0).to(gpu), device_ids=[gpu.index], gradient_as_bucket_view=True,
-                                bucket_cap_mb=0.1))
-    torch.cuda.synchronize()
+    replicas = _replicas(gpu, K, streams)
     local = LocalBucketSync(batches)
     state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 1).attach_local(local)
-    replicas[0].register_comm_hook(state=state, hook=H.similimarity_allreduce_hook(H.subgroup_allreduce_hook))
+    rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), replicas[0].module)
+    replicas[0].register_comm_hook(state=state, hook=rec.hook)
     replicas[1].register_comm_hook(state=H.VSWPeerState(local, 1), hook=H.dummy_hook)
 
-    plain = _model(0).to(gpu)
-    w, _, _ = O.batch_weights(batches)
     for step in range(1, 4):                              # step 1 is the one in which DDP rebuilds its buckets
         gen = torch.Generator().manual_seed(step)
         data = [(torch.randn(b, 64, generator=gen).to(gpu), torch.randn(b, 16, generator=gen).to(gpu)) for b in batches]
-        per_vsw = []
-        for x, y in data:
-            plain.zero_grad(set_to_none=True)
-            crit(plain(x), y).backward()
-            per_vsw.append([p.grad.detach().clone() for p in plain.parameters()])
-        errors, losses = [], []
-        # forward passes one after the other (DDP's forward may use the process group: bucket
-        # rebuild after the first step); backward passes concurrently, one thread per VSW
-        for k in range(K):
-            with torch.cuda.stream(streams[k]):
-                replicas[k].zero_grad(set_to_none=False)
-                losses.append(crit(replicas[k](data[k][0]), data[k][1]))
-
-        def run(k):
-            try:
-                with torch.cuda.stream(streams[k]):
-                    losses[k].backward()
-            except Exception as exc:                      # pragma: no cover - reported below
-                errors.append(exc)
-
-        threads = [threading.Thread(target=run, args=(k,), daemon=True) for k in range(K)]
-        for t in threads:
-            t.start()
-        for t in threads:
-            t.join(timeout=60)
-        assert not errors, errors
-        assert not any(t.is_alive() for t in threads), "a VSW thread is stuck in backward"
-        local.finish_step(streams)
+        rec.seen.clear()
+        _backward_all(replicas, streams, data, crit)
+        local.finish_step()                               # the VSW streams are the ones the hooks ran on
         torch.cuda.synchronize()
+        per_vsw = _per_parameter_grads(rec, replicas)
         for i, p in enumerate(replicas[0].module.parameters()):
-            want = torch.add(torch.mul(per_vsw[0][i], w[0]), torch.mul(per_vsw[1][i], w[1]))
-            assert torch.allclose(p.grad, want, rtol=1e-5, atol=1e-8), (step, i)
+            want = O.aggregate([per_vsw[0][i], per_vsw[1][i]], batches)
+            assert torch.equal(_bits(p.grad), _bits(want)), (step, i)
         # statistic step every step here: cosine between the two workers' whole gradients
-        flat = [torch.cat([g.reshape(-1) for g in gs]).double() for gs in per_vsw]
+        flat = [torch.cat(gs).double() for gs in per_vsw]
         want_cos = torch.nn.functional.cosine_similarity(flat[0], flat[1], dim=0).item()
         got = H.cosine_similarity_from_placeholder(state.grad_placeholder)
-        assert got == pytest.approx(want_cos, rel=1e-4, abs=1e-6)
+        assert got == pytest.approx(want_cos, rel=1e-9, abs=1e-12)
         if step >= 2:                                     # DDP has rebuilt its buckets by now
             assert len(state.grad_placeholder) >= 2       # several buckets at this cap
         state.grad_placeholder.clear()
         state.step += 1
+    del replicas
+    dist.destroy_process_group()
+
+
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind):
+    """Overlap weight-sync mode end to end with stock DDP (jabas/train/trainer.py:327-333): the optimizer
+    hook on VSW 0, a launch stream of its own, the weights of both replicas and the optimizer state
+    bit-exact against the oracle over four steps, across DDP's bucket rebuild after the first."""
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    from jabas_amd.train import prepare_overlap_optimizer_with_ddp
+
+    _init_pg()
+    K, batches = 2, (6, 2)
+    crit = torch.nn.MSELoss()
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    replicas = _replicas(gpu, K, streams)
+    main = replicas[0].module
+    groups = [{"params": [p for p in main.parameters() if p.dim() <= 1], "weight_decay": 0.0},
+              {"params": [p for p in main.parameters() if p.dim() > 1], "weight_decay": 0.05}]
+    if kind == "sgd":
+        optimizer = torch.optim.SGD(groups, lr=0.05, momentum=0.9)
+        opt = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
+                   groups=[dict(lr=0.05, weight_decay=0.0), dict(lr=0.05, weight_decay=0.05)])
+    else:
+        optimizer = torch.optim.AdamW(groups, lr=1e-3)
+        opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+                   groups=[dict(lr=1e-3, weight_decay=0.0), dict(lr=1e-3, weight_decay=0.05)])
+    group_of = [0 if p.dim() <= 1 else 1 for p in main.parameters()]
+    p_h = [p.detach().cpu().clone().reshape(-1) for p in main.parameters()]
+    s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
+
+    local = LocalBucketSync(batches)
+    state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 2).attach_local(local)
+    rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), main)
+    prepare_overlap_optimizer_with_ddp(replicas, [state, H.VSWPeerState(local, 1)], [rec.hook, H.dummy_hook], optimizer, local)
+    assert local._sync_stream is not None and local.optimizer is optimizer
+
+    for step in range(1, 5):
+        for g in optimizer.param_groups:                  # a learning-rate policy writing param_groups, as the reference's do
+            g["lr"] = opt["groups"][0]["lr"] * (0.9 ** (step - 1))
+        gen = torch.Generator().manual_seed(40 + step)
+        data = [(torch.randn(b, 64, generator=gen).to(gpu), torch.randn(b, 16, generator=gen).to(gpu)) for b in batches]
+        rec.seen.clear()
+        _backward_all(replicas, streams, data, crit)
+        local.finish_step()
+        torch.cuda.synchronize()
+        per_vsw = _per_parameter_grads(rec, replicas)
+        step_opt = dict(opt, groups=[dict(g, lr=g["lr"] * (0.9 ** (step - 1))) for g in opt["groups"]])
+        for i, (p, q) in enumerate(zip(main.parameters(), replicas[1].module.parameters())):
+            agg = O.aggregate([per_vsw[0][i], per_vsw[1][i]], batches)
+            O.opt_step(step_opt, group_of[i], p_h[i], agg, s1_h[i], s2_h[i], step, step == 1)
+            assert torch.equal(_bits(p.grad), _bits(agg)), (step, i, "aggregate")
+            assert torch.equal(_bits(p.data), _bits(p_h[i])), (step, i, "weights")
+            assert torch.equal(_bits(q.data), _bits(p_h[i])), (step, i, "replica weights")
+            st = optimizer.state[p]
+            if kind == "sgd":
+                assert torch.equal(_bits(st["momentum_buffer"]), _bits(s1_h[i])), (step, i)
+            else:
+                assert torch.equal(_bits(st["exp_avg"]), _bits(s1_h[i])), (step, i)
+                assert torch.equal(_bits(st["exp_avg_sq"]), _bits(s2_h[i])), (step, i)
+                assert int(st["step"]) == step
+        state.grad_placeholder.clear()
+        state.step += 1
+    sd = optimizer.state_dict()                           # the caller's optimizer object checkpoints as usual
+    assert len(sd["state"]) == len(p_h)
     del replicas
     dist.destroy_process_group()
