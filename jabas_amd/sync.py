@@ -264,8 +264,10 @@ def sync_bucket(span, args, workspace=None, bounds_dev=None, stream=None):
     L.check(L.lib().jabas_sync_bucket(C.byref(c_span), None if bounds_dev is None else bounds_dev.data_ptr(),
                                       C.byref(args), stats_ptr, ws_ptr, ws_bytes, _stream_ptr(stream)),
             "jabas_sync_bucket")
-    if bounds_dev is not None:
-        bounds_dev.record_stream(torch.cuda.current_stream() if stream is None else stream)
+    if stream is not None:                          # temporaries made here are freed on return: the allocator
+        for t in (bounds_dev, workspace and workspace.buf, workspace and workspace.stats):   # must know who uses them
+            if t is not None:
+                t.record_stream(stream)
     return workspace.stats[0] if args.stats else None
 
 
@@ -375,6 +377,9 @@ def gradient_stats(grads, batches, half_id=None, workspace=None, stream=None):
                                 (C.c_float * K)(*[float(x) for x in hw]), n,
                                 workspace.stats.data_ptr(), workspace.buf.data_ptr(), workspace.nbytes,
                                 _stream_ptr(stream)), "jabas_stats")
+    if stream is not None:
+        workspace.buf.record_stream(stream)
+        workspace.stats.record_stream(stream)
     return workspace.stats[0]
 
 
@@ -387,7 +392,9 @@ def gram(grads, stream=None):
     out = torch.empty(L.GRAM_STRIDE, dtype=torch.float64, device=dev)
     L.check(L.lib().jabas_gram(_ptr_array(grads), K, grad_dtype_code(gdt), n, out.data_ptr(), ws.data_ptr(),
                                ws.numel() * 8, _stream_ptr(stream)), "jabas_gram")
-    ws.record_stream(torch.cuda.current_stream() if stream is None else stream)
+    if stream is not None:
+        ws.record_stream(stream)
+        out.record_stream(stream)
     return out.view(L.GRAM_MAX_K, L.GRAM_MAX_K)[:K, :K]
 
 

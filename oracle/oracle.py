@@ -160,6 +160,7 @@ def opt_step(opt, group, p, g, s1, s2, step, first_step, lr_scale=1.0):
     """Dispatch on the optimizer dictionary used throughout the build."""
     grp = opt["groups"][group]
     lr = grp["lr"] * lr_scale
+    step = grp.get("step", step)               # a group may carry its own Adam step count
     wd = grp.get("weight_decay", 0.0)
     if opt["kind"] == "sgd":
         sgd_step(p, g, s1, lr, wd, opt.get("momentum", 0.0), opt.get("dampening", 0.0),

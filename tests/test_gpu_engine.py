@@ -133,3 +133,71 @@ def test_reconfigure_changes_k_and_keeps_weights_and_state(gpu):
         assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
         assert _close(rows[:, :4 + eng.K], rows_h[:, :4 + eng.K], 1e-6, 1e-30)
         p_before, m_before = eng.param.clone(), eng.state1.clone()
+
+
+@pytest.mark.parametrize("opt", [SGD, ADAM])
+def test_lr_modifier_that_moves_between_steps_is_bit_exact(gpu, opt):
+    """The adaptive-batching LR modifier (jabas/train/trainer.py:693-700: lr *= modifier before the
+    step, /= after) travels as ``lr_scale`` of the launch: weights and state bit for bit against the
+    oracle stepping at lr * modifier, with the modifier changing from step to step."""
+    batches = (48, 32, 32, 16)
+    eng, host, spans = _make(gpu, batches, opt, n_fanout=1)
+    adam = opt["kind"] != "sgd"
+    mods = (1.0, math.sqrt(20 / 8), math.sqrt(20 / 8), 0.5, 1.0 / 3.0)
+    for step, m in enumerate(mods, 1):
+        gen = torch.Generator().manual_seed(90 + step)
+        for k in range(len(batches)):
+            host["g"][k] = torch.randn(eng.layout.total, generator=gen) * 1e-2
+            eng.grads[k].copy_(host["g"][k])
+        eng.step(lr_scale=m)
+        torch.cuda.synchronize()
+        O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"] if adam else None, step=step,
+                    first_step=(step == 1), lr_scale=m)
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            assert torch.equal(eng.param[sl].cpu().view(torch.int32), host["p"][sl].view(torch.int32)), (step, m)
+            assert torch.equal(eng.state1[sl].cpu().view(torch.int32), host["s1"][sl].view(torch.int32)), (step, m)
+            if adam:
+                assert torch.equal(eng.state2[sl].cpu().view(torch.int32), host["s2"][sl].view(torch.int32)), (step, m)
+            assert torch.equal(eng.fanout[0][sl], eng.param[sl])
+    # the modifier did change the trajectory: the same steps at modifier 1 end elsewhere
+    eng2, host2, _ = _make(gpu, batches, opt)
+    for step in range(1, len(mods) + 1):
+        gen = torch.Generator().manual_seed(90 + step)
+        for k in range(len(batches)):
+            eng2.grads[k].copy_(torch.randn(eng2.layout.total, generator=gen) * 1e-2)
+        eng2.step()
+    assert not torch.equal(eng2.param, eng.param)
+
+
+@pytest.mark.parametrize("kind", ["adam", "adamw"])
+def test_parameter_groups_at_different_adam_step_counts(gpu, kind):
+    """Groups whose parameters were stepped apart (a group added later, Shard* steps over some buckets
+    only) carry their own step count: bias corrections per group, bit for bit against the oracle."""
+    from jabas_amd import sync
+    n, K, batches = 200_003, 2, (3, 1)
+    bounds = ((0, 0), (70_001, 1), (150_002, 0))
+    gen = torch.Generator().manual_seed(11)
+    p_h = torch.randn(n, generator=gen) * 0.05
+    m_h, v_h = torch.randn(n, generator=gen) * 1e-3, torch.rand(n, generator=gen) * 1e-6
+    p_d, m_d, v_d = p_h.to(gpu), m_h.to(gpu), v_h.to(gpu)
+    steps = [3, 7]
+    for it in range(3):
+        opt = dict(kind=kind, betas=(0.9, 0.999), eps=1e-8,
+                   groups=[dict(lr=1e-3, weight_decay=0.01, step=steps[0] + it),
+                           dict(lr=2e-3, weight_decay=0.0, step=steps[1] + it)])
+        hg = [torch.randn(n, generator=gen) * 1e-3 for _ in range(K)]
+        dg = [g.to(gpu) for g in hg]
+        span = sync.SpanSpec(dg, agg_out=dg[0], param=p_d, state1=m_d, state2=v_d, bounds=bounds)
+        args = sync.make_step_args(batches, torch.float32, opt=opt, step=1)
+        assert [args.groups[i].step for i in range(2)] == [steps[0] + it, steps[1] + it]
+        sync.sync_bucket(span, args)
+        torch.cuda.synchronize()
+        O.sync_step(hg, batches, [(0, n, bounds)], opt, p_h, m_h, v_h, step=1)
+        for got, want in ((p_d, p_h), (m_d, m_h), (v_d, v_h)):
+            assert torch.equal(got.cpu().view(torch.int32), want.view(torch.int32)), it
+    # one common step count gives other weights: the per-group counts were used
+    q_h = p_h.clone()
+    O.sync_step(hg, batches, [(0, n, bounds)], dict(opt, groups=[dict(g, step=5) for g in opt["groups"]]), q_h,
+                m_h.clone(), v_h.clone(), step=1)
+    assert not torch.equal(q_h, p_h)

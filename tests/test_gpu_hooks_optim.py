@@ -249,6 +249,59 @@ def test_trainer_adds_and_removes_workers_from_the_similarity(gpu):
     assert trainer.num_models == 4 and len(trainer.model_streams) == 4 and trainer.engine.K == 4
 
 
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_trainer_steps_at_lr_times_the_controllers_modifier(gpu, kind):
+    """jabas/train/trainer.py:693-700: once adaptive batching has moved the global batch size, every step
+    runs at lr * global_lr_modifier (lr *= modifier before the update, /= after). Weights against a
+    plain-torch optimizer driven exactly that way, while the number of VSWs changes underneath."""
+    from jabas_amd.train import VSWSyncTrainer
+    from jabas_amd.train.adaptive import AdaptiveBatchController
+    import math
+    crit = torch.nn.MSELoss()
+    ctl = AdaptiveBatchController(8, 4, similarity_target=2.0, adjust_rate=0.1)     # cos < 2 always: grow
+    trainer = VSWSyncTrainer(gpu, (4, 4), interval=2, controller=ctl)
+    trainer.prepare_stream_parallel(_mlp(21), crit)
+    ref_model = _mlp(21).to(gpu)
+    if kind == "sgd":
+        mine = torch.optim.SGD(_groups(trainer.main_model), lr=0.05, momentum=0.9)
+        ref_opt = torch.optim.SGD(_groups(ref_model), lr=0.05, momentum=0.9, foreach=False)
+    else:
+        mine = torch.optim.AdamW(_groups(trainer.main_model), lr=1e-3)
+        ref_opt = torch.optim.AdamW(_groups(ref_model), lr=1e-3, foreach=False)
+    trainer.prepare_weight_sync_method(mine, None, _groups)
+    seen = []
+    for step in range(1, 7):
+        K = trainer.num_models
+        batches = trainer.local_batch_sizes
+        modifier = trainer.global_lr_modifier
+        seen.append(modifier)
+        gen = torch.Generator().manual_seed(300 + step)
+        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        trainer.compute(data)
+        w, _, _ = O.batch_weights(batches)
+        per_vsw = []
+        for x, y in data:
+            ref_model.zero_grad(set_to_none=True)
+            crit(ref_model(x), y).backward()
+            per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+        for i, p in enumerate(ref_model.parameters()):
+            acc = torch.mul(per_vsw[0][i], w[0])
+            for k in range(1, K):
+                acc = torch.add(acc, torch.mul(per_vsw[k][i], w[k]))
+            p.grad = acc
+        for g in ref_opt.param_groups:
+            g["lr"] *= modifier
+        ref_opt.step()
+        for g in ref_opt.param_groups:
+            g["lr"] /= modifier
+        trainer.step()
+        torch.cuda.synchronize()
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), f"{kind} step {step} modifier {modifier}"
+    assert seen[0] == 1.0 and seen[-1] == pytest.approx(math.sqrt(16 / 8)) and len(set(seen)) >= 3
+    assert mine.param_groups[0]["lr"] == (0.05 if kind == "sgd" else 1e-3)      # the caller's lr itself is left alone
+
+
 @pytest.mark.parametrize("kind", ["sgd", "adamw", "shard_adam"])
 def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
     """The reference's order of calls (examples/resnet50/main.py:351-366, examples/vit/main.py:425-478):
