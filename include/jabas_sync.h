@@ -61,6 +61,12 @@ typedef enum JabasStatus {
 
 enum { JABAS_F32 = 0, JABAS_BF16 = 1 };
 enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAMW = 3 };
+/* Statistics level of a launch (JabasStepArgs.stats). SIMILARITY: the four sums the cosine
+ * similarity between the halves and global-norm clipping read (slots DOT_AB .. NORM_AGG of a
+ * row; the per-VSW slots are written as 0): the reference's adaptive batching consumes nothing
+ * else (jabas/train/trainer.py:470-483), and the kernels that skip the K per-VSW norms keep more
+ * loads in flight. FULL adds sum g_k^2 of every VSW. */
+enum { JABAS_STATS_NONE = 0, JABAS_STATS_FULL = 1, JABAS_STATS_SIMILARITY = 2 };
 
 /* Slots of one stats_out row (JABAS_STATS_STRIDE doubles per span). A = VSWs with
  * half_id 0, B = VSWs with half_id 1; g_A = sum_{k in A} g_k*half_weight_k formed in
@@ -123,7 +129,7 @@ typedef struct JabasStepArgs {
     int32_t grad_dtype;                 /* JABAS_F32 / JABAS_BF16                      */
     float   weight[JABAS_MAX_K];        /* w_k = fp32(b_k / B); with A micro-batches summed
                                            into every bucket, fp32(b_k / (B*A))         */
-    int32_t stats;                      /* 0: none, 1: write a stats_out row per span  */
+    int32_t stats;                      /* JABAS_STATS_*: none / full row / similarity sums */
     uint8_t half_id[JABAS_MAX_K];       /* 0 = half A, 1 = half B                      */
     float   half_weight[JABAS_MAX_K];   /* fp32(b_k / sum of b over k's half)          */
     int32_t opt_kind;                   /* JABAS_OPT_*                                 */
@@ -167,9 +173,9 @@ int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span,
                       const JabasBound* bounds, uint32_t n_bounds,
                       int32_t K, int32_t grad_dtype, int32_t opt_kind,
                       void* host_blob, size_t blob_bytes);
-/* Number of workgroups (chunks) one launch of the plan uses, without (stats == 0) or with
- * statistics: the two kinds of launch may run different workgroup shapes, the plan holds a
- * chunk table for each. Negative JabasStatus on a malformed blob. */
+/* Number of workgroups (chunks) one launch of the plan uses at statistics level `stats`
+ * (JABAS_STATS_*): the levels may run different workgroup shapes, the plan holds a chunk
+ * table for each shape. Negative JabasStatus on a malformed blob or an unknown level. */
 int64_t jabas_plan_chunks(const void* host_blob, int32_t stats);
 /* Bytes of device workspace jabas_sync_fused needs for this plan when statistics are
  * requested (0 on a malformed blob). */

@@ -20,6 +20,7 @@ STATIC_MAX_NUMEL = 1 << 26
 
 F32, BF16 = 0, 1
 OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW = 0, 1, 2, 3
+STATS_NONE, STATS_FULL, STATS_SIMILARITY = 0, 1, 2
 
 STAT_DOT_AB, STAT_NORM_A, STAT_NORM_B, STAT_NORM_AGG, STAT_NORM_VSW0 = 0, 1, 2, 3, 4
 

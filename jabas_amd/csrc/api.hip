@@ -19,10 +19,10 @@ namespace {
 
 constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 6;
+constexpr uint32_t kPlanVersion = 7;
 
-// A plan holds one chunk table per launch shape: index 0 for launches without statistics, 1 with.
-// When both shapes are the same the two entries describe the same table.
+// A plan holds one chunk table per launch shape, indexed by the statistics level of the launch (0 none,
+// 1 full rows, 2 similarity sums). Levels whose shapes are the same share one table.
 struct PlanShape {
     uint32_t block;           // threads per workgroup the chunk table was cut for
     uint32_t chunk_tiles;     // tiles per workgroup
@@ -37,11 +37,11 @@ struct PlanHeader {
     uint32_t max_group;       // largest group index any bound names
     uint32_t all_have_s1;     // every non-empty span carries a state1 pointer
     uint32_t pad;
-    PlanShape shape[2];
+    PlanShape shape[3];
     uint64_t off_spans, off_bounds, total_bytes;
 };
-static_assert(sizeof(PlanShape) == 32 && sizeof(PlanHeader) == 128, "plan header layout");
-constexpr size_t kHeaderBytes = 128;
+static_assert(sizeof(PlanShape) == 32 && sizeof(PlanHeader) == 160, "plan header layout");
+constexpr size_t kHeaderBytes = 160;
 static_assert(kHeaderBytes >= sizeof(PlanHeader) && kHeaderBytes % 16 == 0, "plan header slot");
 
 inline size_t align16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
@@ -195,6 +195,7 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
     if (s->grad_dtype != JABAS_F32 && s->grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
     const int oc = opt_class_of(s->opt_kind);
     if (oc < 0) return JABAS_ERR_OPT;
+    if (s->stats < JABAS_STATS_NONE || s->stats > JABAS_STATS_SIMILARITY) return JABAS_ERR_OPT;
     memset(a, 0, sizeof(*a));
     uint32_t mask = 0;
     for (int k = 0; k < s->K; ++k) {
@@ -312,12 +313,12 @@ hipError_t launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32
     return launch_kernel(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
                          a.use_inline, stripes, in_stripes, out_stride, in, out);
 }
-// One instantiation per row width 4 + K, K = 1..16.
+// One instantiation per row width: 4 (similarity sums) and 4 + K, K = 1..16.
 hipError_t finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
                     uint32_t out_stride, const double* in, double* out) {
     switch (ns) {
 #define JABAS_FIN(n) case n: return launch_finalize<n>(grid, stream, a, stripes, in_stripes, out_stride, in, out);
-        JABAS_FIN(5) JABAS_FIN(6) JABAS_FIN(7) JABAS_FIN(8) JABAS_FIN(9) JABAS_FIN(10) JABAS_FIN(11) JABAS_FIN(12)
+        JABAS_FIN(4) JABAS_FIN(5) JABAS_FIN(6) JABAS_FIN(7) JABAS_FIN(8) JABAS_FIN(9) JABAS_FIN(10) JABAS_FIN(11) JABAS_FIN(12)
         JABAS_FIN(13) JABAS_FIN(14) JABAS_FIN(15) JABAS_FIN(16) JABAS_FIN(17) JABAS_FIN(18) JABAS_FIN(19) JABAS_FIN(20)
 #undef JABAS_FIN
         default: return hipErrorInvalidValue;
@@ -344,7 +345,7 @@ __global__ void __launch_bounds__(64) clip_coef_kernel(const double* rows, uint3
 int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double* stats_out, void* workspace,
               size_t workspace_bytes, hipStream_t stream) {
     const int oc = opt_class_of(s->opt_kind);
-    const int stats = s->stats ? 1 : 0;
+    const int stats = s->stats;                  // level, checked by fill_kargs
     if (stats) {
         if (!stats_out) return JABAS_ERR_NULL;
         if (a.n_span > kMaxStatsSpans) return JABAS_ERR_SIZE;     // before anything is launched: no half-done step
@@ -359,7 +360,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
     }
     if (stats) {
         const uint32_t st = stripes_for(max_span_chunks);
-        const int ns = 4 + s->K;
+        const int ns = stats == JABAS_STATS_FULL ? 4 + s->K : 4;    // width of the partial rows
         hipError_t err;
         if (st == 1) {
             err = finalize(ns, dim3(1, a.n_span), stream, a, 1u, 0u, kStatsStride, a.partials, stats_out);
@@ -426,9 +427,9 @@ size_t plan_fixed_bytes(uint32_t n_span, uint32_t n_bounds) {
 
 JABAS_API size_t jabas_plan_bytes(const JabasSpan* spans, uint32_t n_span, uint32_t n_bounds, int32_t grad_dtype) {
     if (!spans || (grad_dtype != JABAS_F32 && grad_dtype != JABAS_BF16)) return 0;
-    // K and the optimizer are not known here: two chunk tables of the launch shape with the smallest chunks
+    // K and the optimizer are not known here: one chunk table per statistics level, of the launch shape with the smallest chunks
     return plan_fixed_bytes(n_span, n_bounds) +
-           2 * table_bytes(n_span, plan_chunks_bound(spans, n_span));
+           3 * table_bytes(n_span, plan_chunks_bound(spans, n_span));
 }
 
 JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const JabasBound* bounds,
@@ -459,9 +460,9 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     h.grad_dtype = grad_dtype;
     h.opt_kind = opt_kind;
     h.all_have_s1 = 1;
-    for (int v = 0; v < 2; ++v) {
-        h.shape[v].block = static_cast<uint32_t>(launch_block(K, grad_dtype, oc, v != 0));
-        h.shape[v].chunk_tiles = static_cast<uint32_t>(launch_chunk_tiles(K, grad_dtype, oc, v != 0));
+    for (int v = 0; v < 3; ++v) {
+        h.shape[v].block = static_cast<uint32_t>(launch_block(K, grad_dtype, oc, v));
+        h.shape[v].chunk_tiles = static_cast<uint32_t>(launch_chunk_tiles(K, grad_dtype, oc, v));
     }
 
     // spans first: where a span's element grid starts (and so how many chunks it has) depends on
@@ -478,12 +479,13 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
         if (spans[i].numel && !spans[i].state1) h.all_have_s1 = 0;
     }
     size_t cursor = fixed;
-    for (int v = 0; v < 2; ++v) {
+    int table_of[3];                             // level -> the level whose table it uses (itself when it owns one)
+    for (int v = 0; v < 3; ++v) {
         PlanShape& ps = h.shape[v];
-        if (v == 1 && ps.block == h.shape[0].block && ps.chunk_tiles == h.shape[0].chunk_tiles) {
-            ps = h.shape[0];                     // same shape: one table serves both kinds of launch
-            break;
-        }
+        table_of[v] = v;
+        for (int u = 0; u < v; ++u)
+            if (h.shape[u].block == ps.block && h.shape[u].chunk_tiles == ps.chunk_tiles) { table_of[v] = table_of[u]; break; }
+        if (table_of[v] != v) continue;          // same shape: one table serves both kinds of launch
         uint64_t n_chunks = 0;
         for (uint32_t i = 0; i < n_span; ++i) {
             const uint64_t tiles = tiles_of(sd[i].hi, static_cast<int>(ps.block));
@@ -500,8 +502,8 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
     if (blob_bytes < need) return JABAS_ERR_PLAN;
     memset(base + fixed, 0, need - fixed);
     h.total_bytes = need;
-    const int n_tables = (h.shape[1].off_prefix == h.shape[0].off_prefix) ? 1 : 2;
-    for (int v = 0; v < n_tables; ++v) {
+    for (int v = 0; v < 3; ++v) {
+        if (table_of[v] != v) continue;
         PlanShape& ps = h.shape[v];
         uint32_t* prefix = reinterpret_cast<uint32_t*>(base + ps.off_prefix);
         ChunkDesc* cd = reinterpret_cast<ChunkDesc*>(base + ps.off_chunks);
@@ -529,7 +531,8 @@ JABAS_API int jabas_plan_encode(const JabasSpan* spans, uint32_t n_span, const J
         prefix[n_span] = c;
         if (c != ps.n_chunks) return JABAS_ERR_PLAN;
     }
-    if (n_tables == 1) h.shape[1] = h.shape[0];
+    for (int v = 0; v < 3; ++v)
+        if (table_of[v] != v) h.shape[v] = h.shape[table_of[v]];
     if (n_bounds) memcpy(base + h.off_bounds, bounds, static_cast<size_t>(n_bounds) * sizeof(JabasBound));
     memcpy(base, &h, sizeof(h));
     return JABAS_OK;
@@ -546,14 +549,16 @@ JABAS_API int64_t jabas_plan_chunks(const void* host_blob, int32_t stats) {
     if (!host_blob) return JABAS_ERR_NULL;
     PlanHeader h;
     if (!read_plan_header(host_blob, &h)) return JABAS_ERR_PLAN;
-    return h.shape[stats ? 1 : 0].n_chunks;
+    if (stats < JABAS_STATS_NONE || stats > JABAS_STATS_SIMILARITY) return JABAS_ERR_OPT;
+    return h.shape[stats].n_chunks;
 }
 
 JABAS_API size_t jabas_plan_workspace_bytes(const void* host_blob) {
     if (!host_blob) return 0;
     PlanHeader h;
     if (!read_plan_header(host_blob, &h)) return 0;
-    return workspace_rows(h.shape[1].n_chunks, h.n_span) * kStatsStride * sizeof(double);
+    const uint32_t rows = h.shape[1].n_chunks > h.shape[2].n_chunks ? h.shape[1].n_chunks : h.shape[2].n_chunks;
+    return workspace_rows(rows, h.n_span) * kStatsStride * sizeof(double);
 }
 
 JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, const JabasStepArgs* args,
@@ -572,8 +577,8 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     // the chunk tables are cut for the launch shapes of (K, dtype, optimizer class), and the state pointers
     // were validated for that class only
     if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;
-    const bool stats = args->stats != 0;
-    const PlanShape& ps = h.shape[stats ? 1 : 0];
+    const int stats = args->stats;
+    const PlanShape& ps = h.shape[stats];
     if (ps.block != static_cast<uint32_t>(launch_block(h.K, h.grad_dtype, oc, stats)) ||
         ps.chunk_tiles != static_cast<uint32_t>(launch_chunk_tiles(h.K, h.grad_dtype, oc, stats)))
         return JABAS_ERR_PLAN;
@@ -602,7 +607,7 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
     if (rc != JABAS_OK) return rc;
     uint32_t tiles = 0;
     const int oc = opt_class_of(args->opt_kind);
-    const bool stats = args->stats != 0;
+    const int stats = args->stats;
     rc = encode_span(*span, args->K, args->grad_dtype, args->opt_kind,
                      launch_block(args->K, args->grad_dtype, oc, stats), &a.span0, &tiles);
     if (rc != JABAS_OK) return rc;
@@ -628,8 +633,7 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
 // made with that device current.
 namespace {
 constexpr uint64_t kStaticMaxNumel = JABAS_STATIC_MAX_NUMEL;
-// statistics launches run 256 threads x 2 tiles at the least: 2048 elements per partial row
-constexpr uint64_t kStaticMinChunkElems = 4ull * kBlock * kMinChunkTiles;
+constexpr uint64_t kStaticMinChunkElems = kMinStatsChunkElems;    // one partial row per chunk of a statistics launch
 constexpr size_t kStaticScratchBytes =
     workspace_rows((kStaticMaxNumel + kWideElems - 1 + kStaticMinChunkElems - 1) / kStaticMinChunkElems, 1) *
     kStatsStride * sizeof(double);

@@ -46,13 +46,27 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bit_cast(float, u); }
 
+// Address of element e of a buffer whose base is uniform over the workgroup. NARROW: the byte offset
+// fits 32 bits (spans of up to kNarrowElems elements), so the address is "scalar base + zero-extended
+// 32-bit lane offset": the form a global access takes with the base in scalar registers and ONE vector
+// register of offset shared by every stream of the same element size, instead of a 64-bit vector
+// address (two registers and two additions) per stream and tile.
+template <bool NARROW, int ES> __device__ __forceinline__ const char* elem_addr(const void* base, uint64_t e) {
+    if constexpr (NARROW) {
+        const uint32_t off = static_cast<uint32_t>(e) * static_cast<uint32_t>(ES);
+        return static_cast<const char*>(base) + static_cast<uint64_t>(off);
+    } else {
+        return static_cast<const char*>(base) + e * ES;
+    }
+}
+
 template <int DT> struct Grad;
 
 template <> struct Grad<JABAS_F32> {
     static constexpr int EPT = 4;
     using Raw = f32x4;
-    static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
-        return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + e));
+    template <bool NARROW> static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(elem_addr<NARROW, 4>(base, e)));
     }
     static __device__ __forceinline__ void widen(const Raw& r, float (&x)[4]) {
         x[0] = r.x; x[1] = r.y; x[2] = r.z; x[3] = r.w;
@@ -65,8 +79,8 @@ template <> struct Grad<JABAS_F32> {
 template <> struct Grad<JABAS_BF16> {
     static constexpr int EPT = 4;
     using Raw = u32x2;
-    static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
-        return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(base) + e));
+    template <bool NARROW> static __device__ __forceinline__ Raw load(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(elem_addr<NARROW, 2>(base, e)));
     }
     // bf16 -> fp32 is exact: the 16 bits become the high half of the fp32 pattern.
     static __device__ __forceinline__ void widen(const Raw& r, float (&x)[4]) {
@@ -79,8 +93,29 @@ template <> struct Grad<JABAS_BF16> {
 };
 
 constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2;
+// Kernels with statistics over more than four gradient streams form the addresses of the vector path as
+// scalar base + 32-bit lane offset (measured on the ViT-L/16 set, K = 8 bf16: +0.5 % with full rows, +2 % with
+// similarity sums); their spans of more than kNarrowElems elements (over 4 GiB of fp32 per buffer) go
+// through the careful path tile by tile: correct but slower. Everywhere else 64-bit vector addresses are
+// faster (the scalar bases compete with the launch constants for scalar registers: -0.5 ... -2.5 %).
+constexpr uint64_t kNarrowElems = 1ull << 30;
+__host__ __device__ constexpr bool narrow_addressing(int K, int SL) { return SL != 0 && K > 4; }
 
-template <int K, bool STATS> struct NStats { static constexpr int value = STATS ? 4 + K : 1; };
+// Statistics level of a launch: 0 none, 1 the full row (4 + K sums), 2 the four sums of the halves and of
+// the aggregate only (what the cosine similarity and global-norm clipping read).
+template <int K, int SL> struct NStats { static constexpr int value = SL == 1 ? 4 + K : (SL == 2 ? 4 : 1); };
+
+// Per-thread running sums of the statistics. fp32 gradients: fp64 (a product of two fp32 values is exact
+// in fp64). bf16 gradients: fp32 within the thread's chunk (at most 16 elements), widened to fp64 when the
+// workgroup reduces: a product of two bf16 values is exact in fp32 and the few fp32 additions keep the
+// sums within 1e-6 relative, four orders inside the 1e-2 bar of reduced-precision gradients, at a third
+// of the arithmetic and half the registers (fp64 multiply-adds and conversions run at half rate).
+template <int DT> struct StatAcc { using type = double; };
+template <> struct StatAcc<JABAS_BF16> { using type = float; };
+__device__ __forceinline__ double stat_fma(float a, float b, double acc) {
+    return __builtin_fma(static_cast<double>(a), static_cast<double>(b), acc);
+}
+__device__ __forceinline__ float stat_fma(float a, float b, float acc) { return __builtin_fmaf(a, b, acc); }
 
 // One element of the optimizer step. g is the aggregated gradient.
 template <int OPT>
@@ -106,10 +141,10 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
 }
 
 // Aggregate, statistics and optimizer for N consecutive elements held in registers.
-template <int K, int N, int OPT, bool STATS, bool HD>
+template <int K, int N, int DT, int OPT, int SL, bool HD>
 __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
                                         float (&s2)[N], float (&agg)[N], const KArgs& a,
-                                        const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
+                                        const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
         float s = g[0][i] * a.w[0];
@@ -117,7 +152,7 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
         for (int k = 1; k < K; ++k) s = s + g[k][i] * a.w[k];
         if (clip < 1.0f) s = s * clip;         // global-norm clipping: only ever scales down
         agg[i] = s;
-        if constexpr (STATS) {
+        if constexpr (SL) {
             float ga = 0.0f, gb = 0.0f;
 #pragma unroll
             for (int k = 0; k < K; ++k) {
@@ -129,33 +164,32 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
                     gb = in_b ? gb + t : gb;
                     ga = in_b ? ga : ga + t;
                 }
-                const double gk = static_cast<double>(g[k][i]);
-                acc[JABAS_STAT_NORM_VSW0 + k] = __builtin_fma(gk, gk, acc[JABAS_STAT_NORM_VSW0 + k]);
+                if constexpr (SL == 1)
+                    acc[JABAS_STAT_NORM_VSW0 + k] = stat_fma(g[k][i], g[k][i], acc[JABAS_STAT_NORM_VSW0 + k]);
             }
-            // fp32 x fp32 products are exact in fp64, so fma == mul followed by add here.
-            const double da = static_cast<double>(ga), db = static_cast<double>(gb);
-            const double ds = static_cast<double>(s);
-            acc[JABAS_STAT_DOT_AB] = __builtin_fma(da, db, acc[JABAS_STAT_DOT_AB]);
-            acc[JABAS_STAT_NORM_A] = __builtin_fma(da, da, acc[JABAS_STAT_NORM_A]);
-            acc[JABAS_STAT_NORM_B] = __builtin_fma(db, db, acc[JABAS_STAT_NORM_B]);
-            acc[JABAS_STAT_NORM_AGG] = __builtin_fma(ds, ds, acc[JABAS_STAT_NORM_AGG]);
+            // fp64 sums: fp32 x fp32 products are exact in fp64, so fma == mul followed by add there.
+            acc[JABAS_STAT_DOT_AB] = stat_fma(ga, gb, acc[JABAS_STAT_DOT_AB]);
+            acc[JABAS_STAT_NORM_A] = stat_fma(ga, ga, acc[JABAS_STAT_NORM_A]);
+            acc[JABAS_STAT_NORM_B] = stat_fma(gb, gb, acc[JABAS_STAT_NORM_B]);
+            acc[JABAS_STAT_NORM_AGG] = stat_fma(s, s, acc[JABAS_STAT_NORM_AGG]);
         }
         if constexpr (OPT != OPT_NONE) opt_elem<OPT>(s, p[i], s1[i], s2[i], G, a.opt);
         // keep the elements' dependency chains apart: interleaving them costs the statistics
         // kernels a third of their occupancy in registers and buys nothing in a memory-bound loop
-        if constexpr (STATS) __builtin_amdgcn_sched_barrier(0);
+        if constexpr (SL) __builtin_amdgcn_sched_barrier(0);
     }
 }
 
-template <int NV> __device__ __forceinline__ void load_vec(f32x4 (&r)[NV], const float* base, uint64_t e) {
+template <int NV, bool NARROW> __device__ __forceinline__ void load_vec(f32x4 (&r)[NV], const float* base, uint64_t e) {
 #pragma unroll
-    for (int v = 0; v < NV; ++v) r[v] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(base + e + 4 * v));
+    for (int v = 0; v < NV; ++v)
+        r[v] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(elem_addr<NARROW, 4>(base, e + 4 * v)));
 }
-template <int NV> __device__ __forceinline__ void store_vec(const float (&x)[4 * NV], float* base, uint64_t e) {
+template <int NV, bool NARROW> __device__ __forceinline__ void store_vec(const float (&x)[4 * NV], float* base, uint64_t e) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         f32x4 r = {x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
-        __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(base + e + 4 * v));
+        __builtin_nontemporal_store(r, reinterpret_cast<f32x4*>(const_cast<char*>(elem_addr<NARROW, 4>(base, e + 4 * v))));
     }
 }
 template <int NV> __device__ __forceinline__ void unpack_vec(const f32x4 (&r)[NV], float (&x)[4 * NV]) {
@@ -171,7 +205,7 @@ template <int K, int DT, int U> struct TileRegs {
 
 // Issues every load of U consecutive full tiles. e is the (rebased) index of this
 // thread's first element in the first tile.
-template <int K, int DT, int OPT, int U, int BS>
+template <int K, int DT, int OPT, int U, int BS, bool NARROW>
 __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
@@ -180,23 +214,23 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
 #pragma unroll
-        for (int k = 0; k < K; ++k) r.g[u][k] = GR::load(sp.g[k], eu);
+        for (int k = 0; k < K; ++k) r.g[u][k] = GR::template load<NARROW>(sp.g[k], eu);
         if constexpr (OPT != OPT_NONE) {
-            load_vec<NV>(r.p[u], sp.p, eu);
-            if (load_s1) load_vec<NV>(r.s1[u], sp.s1, eu);
-            if constexpr (OPT == OPT_ADAM) load_vec<NV>(r.s2[u], sp.s2, eu);
+            load_vec<NV, NARROW>(r.p[u], sp.p, eu);
+            if (load_s1) load_vec<NV, NARROW>(r.s1[u], sp.s1, eu);
+            if constexpr (OPT == OPT_ADAM) load_vec<NV, NARROW>(r.s2[u], sp.s2, eu);
         }
     }
 }
 
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
-template <int K, int DT, int OPT, bool STATS, bool HD, int U>
+template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW>
 __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const KArgs& a,
                                         const GroupDev& G, float clip, bool use_s1, bool load_s1,
-                                        double (&acc)[NStats<K, STATS>::value]) {
+                                        typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, STATS)) * EPT;
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, SL)) * EPT;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
@@ -212,33 +246,33 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
             }
             if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r.s2[u], s2);
         }
-        compute<K, EPT, OPT, STATS, HD>(g, p, s1, s2, agg, a, G, clip, acc);
-        if (sp.out) store_vec<NV>(agg, sp.out, eu);
+        compute<K, EPT, DT, OPT, SL, HD>(g, p, s1, s2, agg, a, G, clip, acc);
+        if (sp.out) store_vec<NV, NARROW>(agg, sp.out, eu);
         if constexpr (OPT != OPT_NONE) {
-            store_vec<NV>(p, sp.p, eu);
-            if (use_s1) store_vec<NV>(s1, sp.s1, eu);
-            if constexpr (OPT == OPT_ADAM) store_vec<NV>(s2, sp.s2, eu);
-            for (uint32_t f = 0; f < sp.n_fan; ++f) store_vec<NV>(p, sp.fan[f], eu);
+            store_vec<NV, NARROW>(p, sp.p, eu);
+            if (use_s1) store_vec<NV, NARROW>(s1, sp.s1, eu);
+            if constexpr (OPT == OPT_ADAM) store_vec<NV, NARROW>(s2, sp.s2, eu);
+            for (uint32_t f = 0; f < sp.n_fan; ++f) store_vec<NV, NARROW>(p, sp.fan[f], eu);
         }
     }
 }
 
 // Vector path over nfull consecutive full tiles of one parameter group: groups of U tiles,
 // then U/2, ... down to single tiles.
-template <int K, int DT, int OPT, bool STATS, bool HD, int U>
+template <int K, int DT, int OPT, int SL, bool HD, int U>
 __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
-                                         const GroupDev& G, float clip, double (&acc)[NStats<K, STATS>::value]) {
-    constexpr int BS = launch_block(K, DT, OPT, STATS);
+                                         const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
+    constexpr int BS = launch_block(K, DT, OPT, SL);
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     uint32_t i = 0;
     for (; i + U <= nfull; i += U, e += U * TE) {
         TileRegs<K, DT, U> r;
-        issue_loads<K, DT, OPT, U, BS>(r, sp, e, load_s1);
-        consume<K, DT, OPT, STATS, HD, U>(r, sp, e, a, G, clip, use_s1, load_s1, acc);
+        issue_loads<K, DT, OPT, U, BS, narrow_addressing(K, SL)>(r, sp, e, load_s1);
+        consume<K, DT, OPT, SL, HD, U, narrow_addressing(K, SL)>(r, sp, e, a, G, clip, use_s1, load_s1, acc);
     }
-    if constexpr (U > 1) fast_run<K, DT, OPT, STATS, HD, U / 2>(sp, e, nfull - i, a, G, clip, acc);
+    if constexpr (U > 1) fast_run<K, DT, OPT, SL, HD, U / 2>(sp, e, nfull - i, a, G, clip, acc);
 }
 
 // One tile that touches a span edge or a group change. tile_e0 is the (rebased) index of the first
@@ -248,12 +282,12 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
 // vector straddles the span's first or last element or a bound take the slow way, so such a tile costs
 // little more than a full one (ResNet-50's batch-norm tensors and ViT's biases put a group change
 // into roughly every hundredth tile; one span per tensor puts an edge into every tensor).
-template <int K, int DT, int OPT, bool STATS>
+template <int K, int DT, int OPT, int SL>
 __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const KArgs& a, uint32_t j,
-                                             float clip, double (&acc)[NStats<K, STATS>::value]) {
+                                             float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
-    constexpr int BS = launch_block(K, DT, OPT, STATS);
+    constexpr int BS = launch_block(K, DT, OPT, SL);
     const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     const BoundDev* bd = sp.bound_count ? a.bounds + sp.bound_begin : nullptr;
@@ -271,8 +305,8 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
     if (all_live && one_group) {
         const GroupDev G = a.groups[gid_first];
         TileRegs<K, DT, 1> r;
-        issue_loads<K, DT, OPT, 1, BS>(r, sp, e_first, load_s1);
-        consume<K, DT, OPT, STATS, false, 1>(r, sp, e_first, a, G, clip, use_s1, load_s1, acc);   // halves from the mask: always right
+        issue_loads<K, DT, OPT, 1, BS, false>(r, sp, e_first, load_s1);
+        consume<K, DT, OPT, SL, false, 1, false>(r, sp, e_first, a, G, clip, use_s1, load_s1, acc);   // halves from the mask: always right
         return;
     }
     for (int i = 0; i < EPT; ++i) {
@@ -294,7 +328,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
             if (load_s1) s1[0] = sp.s1[e];
             if constexpr (OPT == OPT_ADAM) s2[0] = sp.s2[e];
         }
-        compute<K, 1, OPT, STATS, false>(g, p, s1, s2, agg, a, G, clip, acc);
+        compute<K, 1, DT, OPT, SL, false>(g, p, s1, s2, agg, a, G, clip, acc);
         if (sp.out) sp.out[e] = agg[0];
         if constexpr (OPT != OPT_NONE) {
             sp.p[e] = p[0];
@@ -306,15 +340,15 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 }
 
 // Tiles [lt0, lt1) of one span (tile indices local to the span).
-template <int K, int DT, int OPT, bool STATS, bool HD>
+template <int K, int DT, int OPT, int SL, bool HD>
 __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
-                                           const KArgs& a, double (&acc)[NStats<K, STATS>::value]) {
+                                           const KArgs& a, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
-    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, STATS)) * EPT;
-    constexpr int UW = STATS ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
-    constexpr int CT = launch_chunk_tiles(K, DT, OPT, STATS);
+    constexpr uint64_t TE = static_cast<uint64_t>(launch_block(K, DT, OPT, SL)) * EPT;
+    constexpr int UW = SL ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
+    constexpr int CT = launch_chunk_tiles(K, DT, OPT, SL);
     constexpr int U0 = UW < CT ? UW : CT;     // never more than a chunk holds
     constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
@@ -333,17 +367,18 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
             if (j + 1 < nb) stretch_end = sp.lo + bd[j + 1].start;
         }
         uint32_t nfull = 0;
-        if (e0 >= sp.lo && stretch_end >= e0 + TE) {
+        // spans beyond 32-bit byte offsets take the careful path tile by tile (64-bit addresses there)
+        if (e0 >= sp.lo && stretch_end >= e0 + TE && (!narrow_addressing(K, SL) || sp.hi <= kNarrowElems)) {
             const uint64_t fit = (stretch_end - e0) / TE;
             const uint32_t left = lt1 - lt;
             nfull = fit < left ? static_cast<uint32_t>(fit) : left;
         }
         if (nfull) {
             const GroupDev G = a.groups[gid];
-            fast_run<K, DT, OPT, STATS, HD, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, clip, acc);
+            fast_run<K, DT, OPT, SL, HD, U>(sp, e0 + static_cast<uint64_t>(threadIdx.x) * EPT, nfull, a, G, clip, acc);
             lt += nfull;
         } else {
-            careful_tile<K, DT, OPT, STATS>(sp, e0, a, j, clip, acc);
+            careful_tile<K, DT, OPT, SL>(sp, e0, a, j, clip, acc);
             lt += 1;
         }
     }
@@ -351,21 +386,21 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
 
 // Statistics kernels carry two copies of the arithmetic: one with the default halves
 // (even worker -> A, odd -> B) resolved at compile time, one driven by the half mask.
-template <int K, int DT, int OPT, bool STATS>
+template <int K, int DT, int OPT, int SL>
 __device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const KArgs& a,
-                                          double (&acc)[NStats<K, STATS>::value]) {
-    if constexpr (STATS) {
+                                          typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
+    if constexpr (SL) {
         constexpr uint32_t kDefaultMask = 0xAAAAu & ((1u << K) - 1u);
-        if (a.half_mask == kDefaultMask) span_range<K, DT, OPT, true, true>(sp, lt0, lt1, j0, a, acc);
-        else span_range<K, DT, OPT, true, false>(sp, lt0, lt1, j0, a, acc);
+        if (a.half_mask == kDefaultMask) span_range<K, DT, OPT, SL, true>(sp, lt0, lt1, j0, a, acc);
+        else span_range<K, DT, OPT, SL, false>(sp, lt0, lt1, j0, a, acc);
     } else {
-        span_range<K, DT, OPT, false, true>(sp, lt0, lt1, j0, a, acc);
+        span_range<K, DT, OPT, 0, true>(sp, lt0, lt1, j0, a, acc);
     }
 }
 
-// Workgroup sum of NS per-thread accumulators -> one partial row. Through LDS rather than
-// wave shuffles: NS stores + 16 loads per thread instead of ~18 DPP-and-add instructions per
-// value, which matters because a workgroup only covers a few thousand elements.
+// Workgroup sum of NS per-thread accumulators -> one partial row, fp64 accumulators (fp32 gradients).
+// Through LDS rather than wave shuffles: NS stores + 16 loads per thread instead of ~18 DPP-and-add
+// instructions per value, which matters because a workgroup only covers a few thousand elements.
 //   stage 1  thread (v, part) adds entries part, part+16, ..., part+240 of value v (in order);
 //   stage 2  the 16 parts of a value sit in one 16-lane row: DPP row reduction.
 // The order is fixed, so the row is bit-identical from run to run.
@@ -394,16 +429,58 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
     }
 }
 
-template <int K, int DT, int OPT, bool STATS>
-__global__ void __launch_bounds__(launch_block(K, DT, OPT, STATS)) fused_kernel(const KArgs a) {
-    constexpr int NS = NStats<K, STATS>::value;
-    constexpr int BS = launch_block(K, DT, OPT, STATS);
-    constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT, STATS);     // the host cuts the chunk table for the same shape
+template <int CTRL> __device__ __forceinline__ float dpp_move_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// The same for fp32 accumulators (bf16 gradients). The sums of a 16-lane row are formed first, in fp32 by
+// DPP (one instruction per step and value, no LDS traffic, no wait); only one entry per row and value goes
+// through LDS, and what follows the barrier is short: thread (v, part) adds entries part, part+16, ... of
+// value v in fp64 and the 16 parts meet by DPP. Every lane of the workgroup is active here.
+template <int NS, int BS>
+__device__ __forceinline__ void flush_stats(float (&acc)[NS], double* row) {
+    constexpr int kParts = 16;
+    constexpr int kRows = BS / 16;                   // 16-lane rows of the workgroup
+    constexpr int kPerPass = BS / kParts;
+    __shared__ float buf[NS][kRows];
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+        float v = acc[i];
+        v += dpp_move_f32<0xB1>(v);          // quad_perm [1,0,3,2]
+        v += dpp_move_f32<0x4E>(v);          // quad_perm [2,3,0,1]
+        v += dpp_move_f32<0x141>(v);         // row_half_mirror
+        v += dpp_move_f32<0x140>(v);         // row_mirror
+        if ((tid & 15) == 0) buf[i][tid >> 4] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v0 = 0; v0 < NS; v0 += kPerPass) {
+        if (tid < (NS - v0) * kParts) {
+            const int v = v0 + (tid >> 4), part = tid & 15;
+            double s = 0.0;
+#pragma unroll
+            for (int i = 0; i < (kRows + kParts - 1) / kParts; ++i)
+                if (i * kParts + part < kRows) s += static_cast<double>(buf[v][i * kParts + part]);
+            s += dpp_move<0xB1, 0xf>(s);
+            s += dpp_move<0x4E, 0xf>(s);
+            s += dpp_move<0x141, 0xf>(s);
+            s += dpp_move<0x140, 0xf>(s);
+            if (part == 0) row[v] = s;
+        }
+    }
+}
+
+template <int K, int DT, int OPT, int SL>
+__global__ void __launch_bounds__(launch_block(K, DT, OPT, SL)) fused_kernel(const KArgs a) {
+    constexpr int NS = NStats<K, SL>::value;
+    constexpr int BS = launch_block(K, DT, OPT, SL);
+    constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT, SL);     // the host cuts the chunk table for the same shape
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
     const uint32_t b = blockIdx.x;
-    double acc[NS];
+    typename StatAcc<DT>::type acc[NS];
 #pragma unroll
-    for (int i = 0; i < NS; ++i) acc[i] = 0.0;
+    for (int i = 0; i < NS; ++i) acc[i] = 0;
 
     if (a.use_inline) {
         const SpanDev& sp = a.span0;
@@ -422,18 +499,18 @@ __global__ void __launch_bounds__(launch_block(K, DT, OPT, STATS)) fused_kernel(
             }
             j0 = lo;
         }
-        run_chunk<K, DT, OPT, STATS>(sp, lt0, lt1, j0, a, acc);
+        run_chunk<K, DT, OPT, SL>(sp, lt0, lt1, j0, a, acc);
     } else {
         const ChunkDesc c = a.chunks[b];
         const SpanDev& sp = a.spans[c.span];
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
         const uint32_t lt1 = c.tile0 + CT < tiles ? c.tile0 + CT : tiles;
-        run_chunk<K, DT, OPT, STATS>(sp, c.tile0, lt1, c.bound0, a, acc);
+        run_chunk<K, DT, OPT, SL>(sp, c.tile0, lt1, c.bound0, a, acc);
     }
-    if constexpr (STATS) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * NS);   // compact rows of 4 + K
+    if constexpr (SL) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * NS);   // compact rows of 4 + K
 }
 
-template <int K, int DT, int OPT, bool STATS>
+template <int K, int DT, int OPT, int SL>
 int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
     // Residency cap through idle dynamic LDS (160 KB per CU). Fewer resident workgroups keep the
     // streamed window of every buffer more compact, which the memory system rewards on write-heavy
@@ -443,8 +520,8 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
 #ifndef JABAS_IDLE_LDS_BYTES
 #define JABAS_IDLE_LDS_BYTES 32768u
 #endif
-    constexpr unsigned idle = (OPT == OPT_ADAM && !STATS && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
-    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, STATS>, dim3(grid), dim3(launch_block(K, DT, OPT, STATS)),
+    constexpr unsigned idle = (OPT == OPT_ADAM && !SL && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
+    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL>, dim3(grid), dim3(launch_block(K, DT, OPT, SL)),
                                           idle, stream, a));
 }
 
@@ -454,20 +531,26 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
 #define JABAS_CAT(a, b) JABAS_CAT_(a, b)
 
 #define JABAS_DISPATCH(FN, ...)                                                              \
-    const int key = (grad_dtype == JABAS_BF16 ? 6 : 0) + opt_class * 2 + (stats ? 1 : 0);    \
+    const int key = (grad_dtype == JABAS_BF16 ? 9 : 0) + opt_class * 3 + stats;              \
     switch (key) {                                                                           \
-        case 0:  return FN<JABAS_K, JABAS_F32, OPT_NONE, false>(__VA_ARGS__);                \
-        case 1:  return FN<JABAS_K, JABAS_F32, OPT_NONE, true>(__VA_ARGS__);                 \
-        case 2:  return FN<JABAS_K, JABAS_F32, OPT_SGD, false>(__VA_ARGS__);                 \
-        case 3:  return FN<JABAS_K, JABAS_F32, OPT_SGD, true>(__VA_ARGS__);                  \
-        case 4:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, false>(__VA_ARGS__);                \
-        case 5:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, true>(__VA_ARGS__);                 \
-        case 6:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, false>(__VA_ARGS__);               \
-        case 7:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, true>(__VA_ARGS__);                \
-        case 8:  return FN<JABAS_K, JABAS_BF16, OPT_SGD, false>(__VA_ARGS__);                \
-        case 9:  return FN<JABAS_K, JABAS_BF16, OPT_SGD, true>(__VA_ARGS__);                 \
-        case 10: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, false>(__VA_ARGS__);               \
-        case 11: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, true>(__VA_ARGS__);                \
+        case 0:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 0>(__VA_ARGS__);                    \
+        case 1:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 1>(__VA_ARGS__);                    \
+        case 2:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 2>(__VA_ARGS__);                    \
+        case 3:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 0>(__VA_ARGS__);                     \
+        case 4:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 1>(__VA_ARGS__);                     \
+        case 5:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 2>(__VA_ARGS__);                     \
+        case 6:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 0>(__VA_ARGS__);                    \
+        case 7:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 1>(__VA_ARGS__);                    \
+        case 8:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 2>(__VA_ARGS__);                    \
+        case 9:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, 0>(__VA_ARGS__);                   \
+        case 10: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 1>(__VA_ARGS__);                   \
+        case 11: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 2>(__VA_ARGS__);                   \
+        case 12: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 0>(__VA_ARGS__);                    \
+        case 13: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 1>(__VA_ARGS__);                    \
+        case 14: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 2>(__VA_ARGS__);                    \
+        case 15: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 0>(__VA_ARGS__);                   \
+        case 16: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 1>(__VA_ARGS__);                   \
+        case 17: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 2>(__VA_ARGS__);                   \
         default: return -1;                                                                  \
     }
 

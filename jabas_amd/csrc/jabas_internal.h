@@ -12,11 +12,13 @@ namespace jabas {
 
 // Launch shape: threads per workgroup and tiles per workgroup (a tile = one 16-byte fp32 vector per
 // thread; a chunk = the tiles one workgroup processes). Small chunks keep the streamed window of every
-// buffer compact (higher HBM rate) and cut the ramp-up / drain of a launch; kernels that carry fp64
+// buffer compact (higher HBM rate) and cut the ramp-up / drain of a launch; kernels that carry many
 // statistics have low occupancy and a long epilogue, and do better with more work per workgroup.
 // Measured per kernel family (A/B builds of the whole library, every shape passes the parity suite):
-//   with statistics               256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
+//   full statistics rows          256 threads x 2 tiles (K <= 4) or 4 tiles (K > 4); 64, 128, 512 and
 //                                 1024 threads were all slower (-2 ... -15 %)
+//   similarity sums only          256 threads x 2 tiles: with four sums the K > 4 kernels fit 4 waves per SIMD
+//                                 with two tiles of loads in flight
 //   plain with optimizer, K > 4   512 threads x 1 tile: +3 ... +8 % over 256 x 4 (bf16 and fp32, SGD and Adam);
 //                                 aggregate-only launches lose 20 % there and stay at 256 x 4
 //   plain, SGD, fp32, K <= 4      128 threads x 2 tiles: +2 ... +5 % over 256 x 2
@@ -31,6 +33,9 @@ namespace jabas {
 #ifndef JABAS_BLOCK_MANYK
 #define JABAS_BLOCK_MANYK 512
 #endif
+#ifndef JABAS_BLOCK_SIM_MANYK
+#define JABAS_BLOCK_SIM_MANYK 256
+#endif
 #ifndef JABAS_CHUNK_TILES_LO
 #define JABAS_CHUNK_TILES_LO 2
 #endif
@@ -40,28 +45,41 @@ namespace jabas {
 #ifndef JABAS_CHUNK_TILES_MANYK
 #define JABAS_CHUNK_TILES_MANYK 1
 #endif
+#ifndef JABAS_CHUNK_TILES_SIM_MANYK
+#define JABAS_CHUNK_TILES_SIM_MANYK 2
+#endif
+#ifndef JABAS_CHUNK_TILES_SIM_LO
+#define JABAS_CHUNK_TILES_SIM_LO JABAS_CHUNK_TILES_LO
+#endif
 constexpr int kBlock = JABAS_BLOCK;         // default threads per workgroup (256 = 4 wave64)
 constexpr int kWaves = kBlock / 64;
 constexpr bool block_ok(int b) { return b % 64 == 0 && b >= 64 && b <= 1024; }
-static_assert(block_ok(JABAS_BLOCK) && block_ok(JABAS_BLOCK_SGD) && block_ok(JABAS_BLOCK_MANYK), "whole waves");
+static_assert(block_ok(JABAS_BLOCK) && block_ok(JABAS_BLOCK_SGD) && block_ok(JABAS_BLOCK_MANYK) &&
+              block_ok(JABAS_BLOCK_SIM_MANYK), "whole waves");
 constexpr int kMinChunkTiles = JABAS_CHUNK_TILES_LO;
 constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
-// opt_class: 0 none, 1 SGD, 2 Adam/AdamW. The shape depends on what a plan is encoded for (K, gradient
-// dtype, optimizer class) and on whether the launch carries statistics; a plan holds one chunk table
-// per shape, so it serves every step.
-__host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, bool stats) {
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW; stats: 0 none, 1 full rows, 2 similarity sums. The shape depends
+// on what a plan is encoded for (K, gradient dtype, optimizer class) and on the statistics level of the
+// launch; a plan holds one chunk table per shape, so it serves every step.
+__host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, int stats) {
+    if (stats == 2 && K > 4) return JABAS_BLOCK_SIM_MANYK;
     if (stats || opt_class == 0) return kBlock;
     if (K > 4) return JABAS_BLOCK_MANYK;
     return (opt_class == 1 && grad_dtype == JABAS_F32) ? JABAS_BLOCK_SGD : kBlock;
 }
-__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int opt_class, bool stats) {
+__host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int opt_class, int stats) {
+    if (stats == 2) return K > 4 ? JABAS_CHUNK_TILES_SIM_MANYK : JABAS_CHUNK_TILES_SIM_LO;
     if (K > 4) return (stats || opt_class == 0) ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
     return kMinChunkTiles;
 }
 constexpr int imin(int a, int b) { return a < b ? a : b; }
-// Fewest elements any chunk covers, over all shapes: sizes workspaces and blobs that must fit every launch.
-constexpr int kMinChunkElems = 4 * imin(imin(JABAS_BLOCK_SGD * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
-                                        imin(JABAS_BLOCK_MANYK * JABAS_CHUNK_TILES_MANYK, JABAS_BLOCK * JABAS_CHUNK_TILES_HI));
+// Fewest elements a chunk of a launch with statistics covers (one partial row per chunk): sizes workspaces.
+constexpr int kMinStatsChunkElems = 4 * imin(imin(JABAS_BLOCK * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_SIM_LO),
+                                             JABAS_BLOCK_SIM_MANYK * JABAS_CHUNK_TILES_SIM_MANYK);
+// Fewest elements any chunk covers, over all shapes: sizes blobs that must fit every launch.
+constexpr int kMinChunkElems = imin(kMinStatsChunkElems,
+                                    4 * imin(imin(JABAS_BLOCK_SGD * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
+                                             imin(JABAS_BLOCK_MANYK * JABAS_CHUNK_TILES_MANYK, JABAS_BLOCK * JABAS_CHUNK_TILES_HI)));
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 
 // Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer

@@ -124,7 +124,8 @@ class VSWFlatSync:
 
     def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None, accumulations=1):
         """One sync step over the whole gradient set. Returns the per-span stats tensor
-        when ``stats`` is set.
+        when ``stats`` is set (True / "full": rows of 4 + K sums; "similarity": the four sums of the halves
+        and of the aggregate, per-VSW slots zero).
 
         Without ``clip_norm``: one fused launch. With it (global-norm clipping as
         examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
@@ -139,7 +140,9 @@ class VSWFlatSync:
             return out
         if self._plan_agg is None:
             self._build_clip_plans()
-        rows = self._plan_agg.run(self.step_args(stats=True, with_opt=False, accumulations=accumulations), stream=stream)
+        # the norm needs the similarity sums only; a caller that asked for full rows gets them
+        level = stats if stats else "similarity"
+        rows = self._plan_agg.run(self.step_args(stats=level, with_opt=False, accumulations=accumulations), stream=stream)
         coef = clip_coef(rows, clip_norm, out=self._coef, stream=stream)
         args = make_step_args((1,), torch.float32, stats=False, opt=self.opt, step=self.step_count + 1,
                               first_step=self.step_count == 0, lr_scale=lr_scale, grad_scale=coef)

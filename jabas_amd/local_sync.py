@@ -71,12 +71,16 @@ class LocalBucketSync:
     """
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
-                 optimizer=None):
+                 optimizer=None, stats_level="similarity"):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
         (one ramp-up and drain: 0.68 ms against 0.9 ms wall for the 14 buckets of ViT-B/16) and less host
         time, and the buckets hold the aggregate only after ``finish_step``.
+
+        stats_level: what a statistic step computes per bucket: "similarity" (the four sums the cosine between
+        the halves and norm clipping read: all the reference's adaptive batching consumes,
+        jabas/train/trainer.py:470-483) or "full" (plus the squared norm of every VSW's gradient).
 
         stream: the stream the fused launches are queued on (the reference's dedicated optimizer
         stream, jabas/train/trainer.py:328); default: the stream VSW 0's hooks run on.
@@ -89,6 +93,7 @@ class LocalBucketSync:
         if deferred and launcher is not None:
             raise ValueError("the deferred mode drives the C ABI itself: no launcher can be injected")
         self.deferred = bool(deferred)
+        self.stats_level = sync.stats_level(stats_level) or L.STATS_SIMILARITY
         self._ready = {}                       # deferred mode: bucket index -> complete _Slot of this step
         self._vsw_streams = {}                 # VSW index -> the stream its hooks ran on in this step
         self._plan = self._plan_key = None
@@ -317,7 +322,7 @@ class LocalBucketSync:
                     self._refresh_hyperparameters()
                     self._args_cache_fresh = True
                 hit = self._args_cache[key] = sync.make_step_args(
-                    self.batches if batches is None else batches, dtype, stats=want_stats,
+                    self.batches if batches is None else batches, dtype, stats=self.stats_level if want_stats else 0,
                     opt=self.opt if with_opt else None, step=self.step_count + 1,
                     first_step=not self._momentum_ready, lr_scale=self.lr_scale,
                     accumulations=self.accumulations if batches is None else 1, grad_scale=grad_scale)

@@ -65,6 +65,19 @@ def opt_kind(opt):
     return _KIND[kind]
 
 
+def stats_level(stats):
+    """JABAS_STATS_* level of a launch: False / None / 0 none; True / 1 / 'full' the full row (4 + K sums);
+    2 / 'similarity' the four sums of the halves and of the aggregate only (what the cosine similarity and
+    global-norm clipping read; the per-VSW norm slots of the row are 0)."""
+    if stats is None or stats is False or stats == 0:
+        return L.STATS_NONE
+    if stats is True or stats == 1 or stats == "full":
+        return L.STATS_FULL
+    if stats == 2 or stats == "similarity":
+        return L.STATS_SIMILARITY
+    raise ValueError(f"unknown statistics level {stats!r}")
+
+
 def grad_dtype_code(dtype):
     if dtype == torch.float32:
         return L.F32
@@ -89,7 +102,7 @@ def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_ste
         a.weight[k] = float(w[k])
         a.half_id[k] = int(hid[k])
         a.half_weight[k] = float(hw[k])
-    a.stats = 1 if stats else 0
+    a.stats = stats_level(stats)
     a.opt_kind = opt_kind(opt)
     if opt is not None and a.opt_kind != L.OPT_NONE:
         groups = opt["groups"]
@@ -234,7 +247,8 @@ class SyncPlan:
                                       self.K, grad_dtype_code(gdt), opt_kind_code,
                                       self._host.ctypes.data, nbytes), "jabas_plan_encode")
         self.n_chunks = int(lib.jabas_plan_chunks(self._host.ctypes.data, 0))            # workgroups of a plain launch
-        self.n_chunks_stats = int(lib.jabas_plan_chunks(self._host.ctypes.data, 1))      # of a launch with statistics
+        self.n_chunks_stats = int(lib.jabas_plan_chunks(self._host.ctypes.data, 1))      # of a launch with full statistics rows
+        self.n_chunks_similarity = int(lib.jabas_plan_chunks(self._host.ctypes.data, 2)) # of a launch with similarity sums
         self._dev = torch.from_numpy(self._host.view(np.int64)).to(dev)
         self.ws = Workspace(lib.jabas_plan_workspace_bytes(self._host.ctypes.data), n_span, dev)
         self.n_span = n_span

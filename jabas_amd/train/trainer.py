@@ -416,7 +416,8 @@ class VSWSyncTrainer:
         st = self.similarity_state
         want = st.step % st.interval == 0
         self._refresh_hyperparameters()
-        rows = self.engine.step(stats=want, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm,
+        # the cosine (and the clipping norm) read the four similarity sums only
+        rows = self.engine.step(stats="similarity" if want else False, lr_scale=self.global_lr_modifier, clip_norm=self.clip_norm,
                                 accumulations=max(1, self.accumulated))
         self.accumulated = 0
         self.sync_step += 1

@@ -297,9 +297,10 @@ def test_plan_encode_rejects_overlapping_written_buffers():
 
 
 def test_launch_shape_follows_what_the_plan_is_encoded_for():
-    """Launches with statistics run 256-thread workgroups of 2 tiles (K <= 4) or 4 tiles; plain launches
-    512 threads x 1 tile for K > 4, 128 threads x 2 tiles for SGD with fp32 gradients and K <= 4, else
-    256 x 2. A plan holds a chunk table per shape and serves launches of its own optimizer class only."""
+    """Launches with full statistics rows run 256-thread workgroups of 2 tiles (K <= 4) or 4 tiles, with
+    similarity sums only 2 tiles for every K; plain launches 512 threads x 1 tile for K > 4, 128 threads x
+    2 tiles for SGD with fp32 gradients and K <= 4, else 256 x 2. A plan holds a chunk table per shape and
+    serves launches of its own optimizer class only."""
     lib = L.lib()
     n = 10 * 4096
     def chunks(K, dtype, opt, gs=4):
@@ -314,6 +315,10 @@ def test_launch_shape_follows_what_the_plan_is_encoded_for():
     assert chunks(8, L.BF16, L.OPT_ADAMW, gs=2)[0] == (n // 2048, n // 4096)
     assert chunks(2, L.F32, L.OPT_NONE)[0] == (n // 2048, n // 2048)
     assert chunks(8, L.F32, L.OPT_NONE)[0] == (n // 4096, n // 4096)
+    _, blob8 = chunks(8, L.BF16, L.OPT_ADAMW, gs=2)
+    assert lib.jabas_plan_chunks(blob8.ctypes.data, L.STATS_SIMILARITY) == n // 2048
+    _, blob2 = chunks(2, L.F32, L.OPT_SGD)
+    assert lib.jabas_plan_chunks(blob2.ctypes.data, L.STATS_SIMILARITY) == n // 2048
     _, blob = chunks(2, L.F32, L.OPT_SGD)
     assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (n // 2048 + 1) * L.STATS_STRIDE * 8
     args = L.JabasStepArgs()
@@ -389,7 +394,7 @@ def _shape_model(K, dtype, opt_class, stats):
     else:
         block = 128 if (opt_class == 1 and dtype == L.F32) else 256
     if K > 4:
-        tiles = 4 if (stats or opt_class == 0) else 1
+        tiles = 2 if stats == 2 else (4 if (stats or opt_class == 0) else 1)
     else:
         tiles = 2
     return block, tiles
@@ -409,7 +414,7 @@ def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
     opt_class = {L.OPT_NONE: 0, L.OPT_SGD: 1, L.OPT_ADAM: 2, L.OPT_ADAMW: 2}[opt]
     gs = 2 if dtype == L.BF16 else 4
     n_span = int(rng.randint(1, 12))
-    spans, want_chunks, want_rc = [], [0, 0], L.OK
+    spans, want_chunks, want_rc = [], [0, 0, 0], L.OK
     stride = 1 << 36
     for i in range(n_span):
         numel = int(rng.choice([0, 1, 3, 500, 1023, 1024, 1025, 4096, 4097, 70000, 1 << 20])) + int(rng.randint(0, 3))
@@ -443,7 +448,7 @@ def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
             want_rc = L.ERR_ALIGN
             continue
         skew = used[0] if len(set(used)) == 1 else used[0] % 4
-        for v, stats in enumerate((False, True)):
+        for v, stats in enumerate((0, 1, 2)):                           # statistics level of the launch
             block, tiles = _shape_model(K, dtype, opt_class, stats)
             te = block * 4
             want_chunks[v] += -(-(-(-(skew + numel) // te)) // tiles)
@@ -457,3 +462,5 @@ def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
     assert rc == L.OK, rc
     assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == want_chunks[0]
     assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == want_chunks[1]
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 2) == want_chunks[2]
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 3) == L.ERR_OPT

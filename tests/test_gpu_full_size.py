@@ -119,12 +119,14 @@ def test_full_size_configuration(gpu, name):
     assert abs(got_sum - want_sum) <= 1e-6 * g_abs + 1e-12
 
     # ---- statistics
+    # fp32 gradients: fp64 sums throughout; bf16 gradients: fp32 partial sums per thread and chunk (bar 1e-2)
+    stat_rel = 1e-10 if cfg.grad_dtype != "bf16" else 1e-5
     whole = rows1.sum(0)
     for k in range(cfg.K):
-        assert whole[4 + k].item() == pytest.approx(norms[k], rel=1e-10)
-    assert whole[3].item() == pytest.approx((eng.agg.double() ** 2).sum().item(), rel=1e-10)
+        assert whole[4 + k].item() == pytest.approx(norms[k], rel=stat_rel)
+    assert whole[3].item() == pytest.approx((eng.agg.double() ** 2).sum().item(), rel=stat_rel)
     one_span = sync.gradient_stats(g_before, cfg.batches).cpu()          # one span over the whole arena
-    assert torch.allclose(whole[:4 + cfg.K], one_span[:4 + cfg.K], rtol=1e-11, atol=0.0)
+    assert torch.allclose(whole[:4 + cfg.K], one_span[:4 + cfg.K], rtol=stat_rel / 10, atol=0.0)
     cos = sync.cosine_from_stats(rows1)
     assert -1.0 <= cos <= 1.0
 

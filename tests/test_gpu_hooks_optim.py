@@ -116,7 +116,7 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
             return self._t
 
     K, batches, sizes = 3, (4, 2, 2), [40001, 7, 250000]
-    local = LocalBucketSync(batches, deferred=deferred)
+    local = LocalBucketSync(batches, deferred=deferred, stats_level="full")
     st = H.GradientSimilarityState(None, 4, None, [], 1).attach_local(local)
     main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
     streams = [torch.cuda.Stream(gpu) for _ in range(K)]
