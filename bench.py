@@ -2,19 +2,25 @@
 """Benchmark of the fused per-GPU gradient-sync step on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-all] [--no-cpu]
+                    [--cpu-seconds S] [--calibrate-copy]
 
 A step is one fused sync step (batch-weighted aggregate of the K VSW gradient buckets
-+ gradient statistics where the configuration asks for them + optimizer update) over
-one full synthetic gradient set. The headline workload is the ViT-B/16 configuration;
-the other four configurations are timed too and reported under "workloads" in the
-same JSON line. Inputs are resident in HBM before the timed region starts. Small
-configurations rotate over several copies of their buffers so that the working set
-stays far above the 256 MB last-level cache.
++ the similarity statistics where the configuration asks for them + optimizer update) over
+one full synthetic gradient set. The headline workload is the largest configuration that
+fits one GPU, ViT-L/16 (304 M parameters, K = 8 bf16 gradient sets, AdamW); the other four
+configurations are timed too and reported under "workloads" in the same JSON line. Inputs
+are resident in HBM before the timed region starts. Small configurations rotate over
+several copies of their buffers so that the working set stays far above the 256 MB
+last-level cache.
 
 Prints ONE JSON line: metric sync_step_GBps = algorithmic bytes per step / time per step,
-with a "roofline" object (HBM-bound; achieved = algorithmic bytes per launch / mean
-launch duration from HIP events on the launching stream) and a "cpu_baseline" object
-(the reference's unfused PyTorch structure timed on this box's host cores, rank 0 only).
+with a "roofline" object (HBM-bound; achieved = algorithmic bytes per launch / mean launch
+duration = HIP-event time of the timed region on the launching stream / its launches) and a
+"cpu_baseline" object (the reference's unfused PyTorch structure timed on this box's host
+cores, rank 0 only, a bounded number of whole steps). Every entry of "workloads" carries
+its own figures of both, the step as the reference's calling convention reaches it (one
+hook call per bucket and VSW, per bucket and deferred), and the neighbouring launches
+(without statistics, with full statistics rows).
 """
 import argparse
 import json
@@ -29,11 +35,18 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published peak
 ROTATE_TARGET_BYTES = 1.5e9   # minimum total working set per configuration
+TRAFFIC_FILE = os.path.join("profiles", "fused_kernel_hbm_traffic.json")
 
-# HBM bytes per launch of the fused kernel measured with rocprofv3 --pmc (FETCH_SIZE and
-# WRITE_SIZE runs, scaled by a copy kernel of known size; profiles/fused_kernel_hbm_traffic_pmc.md).
-MEASURED_TRAFFIC_BYTES = {"vit_b16": 3816.9e6, "resnet50": 718.9e6, "faster_rcnn_r50_fpn": 1345.5e6,
-                          "gnmt": 7083.6e6, "vit_l16": 13405.5e6}
+
+def measured_traffic(name):
+    """HBM bytes per launch of the fused kernel from rocprofv3 counters, read from the tracked summary
+    next to the profile it came from (None when that file does not cover the workload)."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            table = json.load(f)
+        return table["workloads"].get(name, {}).get("hbm_bytes_per_launch")
+    except (OSError, ValueError, KeyError):
+        return None
 
 
 def algorithmic_bytes_per_elem(cfg):
@@ -42,9 +55,29 @@ def algorithmic_bytes_per_elem(cfg):
     return cfg.K * s_g + 4 + state
 
 
-def build_engines(cfg, device, torch):
-    from jabas_amd.engine import VSWFlatSync
+def fill_engine(eng, cfg, device, torch, seed, independent_masks=False):
     from jabas_amd import workloads as W
+    gdt = eng.grad_dtype
+    gen = torch.Generator(device=device).manual_seed(seed)
+    for k in range(cfg.K):
+        tmp = torch.randn(eng.layout.total, generator=gen, device=device, dtype=torch.float32) * cfg.grad_std
+        eng.grads[k].copy_(tmp.to(gdt))
+        del tmp
+    eng.param.copy_(torch.randn(eng.layout.total, generator=gen, device=device) * 0.05)
+    if cfg.name == "gnmt":
+        # embedding gradient: a fixed random 10 % of the rows non-zero; the same rows for every VSW, or
+        # (second variant) rows drawn independently per VSW
+        i = [s.name for s in cfg.specs].index(W.GNMT_EMBEDDING)
+        rows, cols = W.GNMT_EMBEDDING_ROWS, W.GNMT_EMBEDDING_COLS
+        for k in range(cfg.K):
+            mask_seed = k + 1 if independent_masks else 0
+            keep = (torch.rand(rows, generator=torch.Generator().manual_seed(mask_seed)) < 0.1).to(device)
+            v = eng.grad_view(k, i).view(rows, cols)
+            v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=device, dtype=v.dtype)))
+
+
+def build_engines(cfg, device, torch, independent_masks=False):
+    from jabas_amd.engine import VSWFlatSync
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
     numel = sum(s.numel for s in cfg.specs)
     ws = numel * algorithmic_bytes_per_elem(cfg)
@@ -52,81 +85,173 @@ def build_engines(cfg, device, torch):
     engines = []
     for c in range(copies):
         eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device)
-        gen = torch.Generator(device=device).manual_seed(1234 + 17 * c)
-        for k in range(cfg.K):
-            tmp = torch.randn(eng.layout.total, generator=gen, device=device, dtype=torch.float32) * cfg.grad_std
-            eng.grads[k].copy_(tmp.to(gdt))
-            del tmp
-        eng.param.copy_(torch.randn(eng.layout.total, generator=gen, device=device) * 0.05)
-        if cfg.name == "gnmt":
-            # embedding gradient: a fixed random 10 % of the rows non-zero, same rows for every VSW
-            i = [s.name for s in cfg.specs].index(W.GNMT_EMBEDDING)
-            rows, cols = W.GNMT_EMBEDDING_ROWS, W.GNMT_EMBEDDING_COLS
-            keep = (torch.rand(rows, generator=torch.Generator().manual_seed(0)) < 0.1).to(device)
-            for k in range(cfg.K):
-                v = eng.grad_view(k, i).view(rows, cols)
-                v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=device, dtype=v.dtype)))
+        fill_engine(eng, cfg, device, torch, 1234 + 17 * c, independent_masks)
         engines.append(eng)
     return engines, numel, copies
 
 
-def time_config(cfg, device, steps, warmup, torch):
-    engines, numel, copies = build_engines(cfg, device, torch)
-    bytes_per_step = numel * algorithmic_bytes_per_elem(cfg)
-    n = len(engines)
+def timed_region(fn, steps, warmup, torch):
+    """ms per call of fn(i) over exactly `steps` calls, HIP events on the current stream."""
     for i in range(warmup):
-        engines[i % n].step(stats=cfg.stats)
+        fn(i)
     torch.cuda.synchronize()
-    # timed region: exactly `steps` steps
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for i in range(steps):
-        engines[i % n].step(stats=cfg.stats)
+        fn(i)
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    region_ms = e0.elapsed_time(e1)
-    ms_per_step = max(region_ms, 1e-6) / steps
-    # per-launch durations (instrumentation pass, outside the timed region)
+    return max(e0.elapsed_time(e1), 1e-6) / steps, wall_ms / steps
+
+
+def rate(bytes_per_step, ms):
+    gbps = bytes_per_step / 1e9 / (ms / 1e3)
+    return dict(ms_per_step=ms, GBps=gbps, pct_hbm_peak=100.0 * gbps / HBM_PEAK_GBPS)
+
+
+class _Bucket:
+    """The part of a DDP GradBucket the hooks read."""
+
+    def __init__(self, i, t):
+        self._i, self._t = i, t
+
+    def index(self):
+        return self._i
+
+    def buffer(self):
+        return self._t
+
+
+def hook_path(cfg, eng, device, steps, warmup, torch, deferred):
+    """The same step as the reference's calling convention reaches it: per bucket, VSW 0's similarity
+    hook (with the optimizer bound: the overlap weight-sync mode) and K - 1 dummy hooks, each handing
+    over its bucket view; one fused launch per bucket (or one per step, deferred) on a launch stream
+    of its own. One host thread plays all K VSWs. Returns ms per step (HIP events around the steps)."""
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    pbs, bucket_slices = {}, []
+    for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
+        sl = slice(off, off + numel)
+        bucket_slices.append(sl)
+        pbs[b] = dict(param=eng.param[sl], state1=None if eng.state1 is None else eng.state1[sl],
+                      state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds,
+                      agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
+    stream = torch.cuda.Stream(device)
+    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, deferred=deferred, stream=stream)
+    local.step_count = eng.step_count
+    local._momentum_ready = eng.step_count > 0
+    state = H.GradientSimilarityState(None, cfg.K + cfg.K % 2, None, [], 1 if cfg.stats else 10 ** 9).attach_local(local)
+    main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
+    peers = [H.VSWPeerState(local, k) for k in range(1, cfg.K)]
+    buckets = [[_Bucket(b, eng.grads[k][sl]) for k in range(cfg.K)] for b, sl in enumerate(bucket_slices)]
+    cur = torch.cuda.current_stream(device)
+
+    def one_step(_):
+        for per_vsw in buckets:
+            main_hook(state, per_vsw[0])
+            for k in range(1, cfg.K):
+                H.dummy_hook(peers[k - 1], per_vsw[k])
+        local.finish_step((cur,))
+        state.grad_placeholder.clear()
+
+    ms, wall = timed_region(one_step, steps, warmup, torch)
+    eng.step_count = local.step_count
+    return dict(ms_per_step=ms, wall_ms_per_step=wall, launches_per_step=1 if deferred else len(buckets))
+
+
+def time_config(cfg, device, steps, warmup, torch, extras=True):
+    engines, numel, copies = build_engines(cfg, device, torch)
+    bytes_per_step = numel * algorithmic_bytes_per_elem(cfg)
+    n = len(engines)
+    level = "similarity" if cfg.stats else False
+    # timed region: exactly `steps` steps, back to back on one stream
+    ms_per_step, wall_ms = timed_region(lambda i: engines[i % n].step(stats=level), steps, warmup, torch)
+    # per-launch durations (instrumentation pass, outside the timed region): one event pair per step
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i, (a, b) in enumerate(evs):
         a.record()
-        engines[i % n].step(stats=cfg.stats)
+        engines[i % n].step(stats=level)
         b.record()
     torch.cuda.synchronize()
     launch_ms = sorted(a.elapsed_time(b) for a, b in evs)
-    mean_launch_ms = sum(launch_ms) / len(launch_ms)
-    # the step between statistic steps (statistics run every `interval` steps in training): same
-    # bytes, no fp64 sums, the launch shape of the plain kernels
-    plain = None
-    if cfg.stats:
-        for i in range(warmup):
-            engines[i % n].step(stats=False)
-        p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        p0.record()
-        for i in range(steps):
-            engines[i % n].step(stats=False)
-        p1.record()
-        torch.cuda.synchronize()
-        plain_ms = max(p0.elapsed_time(p1), 1e-6) / steps
-        plain = dict(ms_per_step=plain_ms, GBps=bytes_per_step / 1e9 / (plain_ms / 1e3),
-                     pct_hbm_peak=100.0 * bytes_per_step / 1e9 / (plain_ms / 1e3) / HBM_PEAK_GBPS)
-    stats_rows = engines[0].step(stats=True) if cfg.stats else None
-    cos = engines[0].cosine(stats_rows) if stats_rows is not None else None
-    finite = bool(torch.isfinite(engines[0].param).all())
     res = dict(
         workload=cfg.name, elements=numel, K=cfg.K, batches=list(cfg.batches), grad_dtype=cfg.grad_dtype,
-        optimizer=cfg.opt["kind"], stats=cfg.stats, spans=engines[0].plan.n_span,
+        optimizer=cfg.opt["kind"], stats="similarity" if cfg.stats else "none", spans=engines[0].plan.n_span,
         bytes_per_elem=algorithmic_bytes_per_elem(cfg), GB_per_step=bytes_per_step / 1e9,
-        ms_per_step=ms_per_step, wall_ms_per_step=wall_ms / steps, GBps=bytes_per_step / 1e9 / (ms_per_step / 1e3),
-        launch_ms_mean=mean_launch_ms, launch_ms_median=launch_ms[len(launch_ms) // 2], launch_ms_min=launch_ms[0],
-        GBps_launch=bytes_per_step / 1e9 / (mean_launch_ms / 1e3),
-        pct_hbm_peak=100.0 * bytes_per_step / 1e9 / (mean_launch_ms / 1e3) / HBM_PEAK_GBPS,
-        buffer_copies=copies, cosine=cos, finite=finite, step_without_statistics=plain)
+        wall_ms_per_step=wall_ms, buffer_copies=copies,
+        launch_ms_mean=sum(launch_ms) / len(launch_ms), launch_ms_median=launch_ms[len(launch_ms) // 2],
+        launch_ms_min=launch_ms[0])
+    res.update(rate(bytes_per_step, ms_per_step))
+    if cfg.stats and extras:
+        # the step between statistic steps (statistics run every `interval` steps in training), and the
+        # step that also forms the squared norm of every VSW's gradient
+        ms, _ = timed_region(lambda i: engines[i % n].step(stats=False), steps, warmup, torch)
+        res["step_without_statistics"] = rate(bytes_per_step, ms)
+        ms, _ = timed_region(lambda i: engines[i % n].step(stats="full"), steps, warmup, torch)
+        res["step_with_per_vsw_norms"] = rate(bytes_per_step, ms)
+    if extras:
+        hsteps, hwarm = max(5, steps // 2), max(2, warmup // 2)
+        res["hook_path_per_bucket_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False)
+        res["hook_path_deferred_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, True)
+    if cfg.name == "gnmt" and extras:
+        # global-norm clipping (examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
+        # coefficient on the device, then the update over the scaled aggregate
+        ms, _ = timed_region(lambda i: engines[i % n].step(stats=level, clip_norm=5.0), steps, warmup, torch)
+        res["clipped_step_ms"] = ms
+    stats_rows = engines[0].step(stats=level) if cfg.stats else None
+    res["cosine"] = engines[0].cosine(stats_rows) if stats_rows is not None else None
+    res["finite"] = bool(torch.isfinite(engines[0].param).all())
     del engines
     torch.cuda.empty_cache()
+    if cfg.name == "gnmt" and extras:
+        engines, _, _ = build_engines(cfg, device, torch, independent_masks=True)
+        ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
+        res["independent_row_masks"] = rate(bytes_per_step, ms)
+        del engines
+        torch.cuda.empty_cache()
     return res
+
+
+def copy_rate(device, steps, torch):
+    """The library's own plain copy (K = 1, weight 1 aggregate: the same 16-byte nontemporal loads and
+    stores as every other instantiation) over 1 GiB: what this box's memory system gives a 1:1
+    read/write stream."""
+    from jabas_amd import sync
+    src = torch.ones(1 << 28, dtype=torch.float32, device=device)
+    dst = torch.empty_like(src)
+    ms, _ = timed_region(lambda i: sync.aggregate([src], (1,), out=dst), max(5, steps // 5), 2, torch)
+    del src, dst
+    torch.cuda.empty_cache()
+    return 2 * (1 << 30) / 1e9 / (ms / 1e3)
+
+
+def statistics_launches(device, steps, torch):
+    """The similarity hook on a step without weight update (the sequential weight-sync mode): aggregate +
+    statistics over a 64 Mi-element bucket set, and the statistics alone, K = 4 and 8, fp32 and bf16."""
+    from jabas_amd import sync
+    n = 1 << 26
+    out = []
+    for K in (4, 8):
+        for gdt, name, sg in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
+            grads = [(torch.randn(n, device=device) * 1e-3).to(gdt) for _ in range(K)]
+            agg = torch.empty(n, device=device)
+            batches = tuple(range(K, 0, -1))
+            entry = dict(K=K, grad_dtype=name, elements=n)
+            for level in ("similarity", "full"):
+                args = sync.make_step_args(batches, gdt, stats=level)
+                ws = sync.Workspace.for_span(n, gdt, device)
+                span = sync.SpanSpec(grads, agg_out=agg)
+                ms, _ = timed_region(lambda i: sync.sync_bucket(span, args, workspace=ws), max(5, steps // 2), 3, torch)
+                entry[f"aggregate_and_{level}"] = rate(n * (K * sg + 4), ms)
+                span = sync.SpanSpec(grads)
+                ms, _ = timed_region(lambda i: sync.sync_bucket(span, args, workspace=ws), max(5, steps // 2), 3, torch)
+                entry[f"{level}_only"] = rate(n * K * sg, ms)
+            out.append(entry)
+            del grads, agg
+            torch.cuda.empty_cache()
+    return out
 
 
 def launch_modes(cfg, device, steps, torch):
@@ -137,41 +262,30 @@ def launch_modes(cfg, device, steps, torch):
     from jabas_amd.sync import SyncPlan
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
     out = {}
-
-    def timed(fn, n):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(n):
-            fn()
-        b.record()
-        torch.cuda.synchronize()
-        return a.elapsed_time(b) / n
-
     for label, per_tensor in (("one_launch_bucket_spans", False), ("one_launch_tensor_spans", True)):
         eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, per_tensor_spans=per_tensor)
         for g in eng.grads:
             g.normal_(0, cfg.grad_std)
         eng.param.normal_(0, 0.05)
         eng.step()
-        out[label] = dict(launches=1, spans=eng.plan.n_span, ms=timed(lambda: eng.step(), steps))
+        out[label] = dict(launches=1, spans=eng.plan.n_span, ms=timed_region(lambda i: eng.step(), steps, 3, torch)[0])
         plans = [SyncPlan([sp], eng.plan.opt_kind) for sp in eng.plan.spans]
         args = eng.step_args()
 
-        def many():
+        def many(_):
             for p in plans:
                 p.run(args)
         key = "one_launch_per_tensor" if per_tensor else "one_launch_per_bucket"
-        out[key] = dict(launches=len(plans), spans=len(plans), ms=timed(many, max(3, steps // 5)))
+        out[key] = dict(launches=len(plans), spans=len(plans), ms=timed_region(many, max(3, steps // 5), 3, torch)[0])
         del eng, plans
         torch.cuda.empty_cache()
     return out
 
 
-def cpu_baseline(cfg, torch, budget_s=25.0):
-    """Reference-structured unfused step on the host cores, bounded to about budget_s."""
+def cpu_baseline(cfg, torch, budget_s):
+    """Reference-structured unfused step on the host cores: 1 warm-up step (allocates the optimizer state),
+    then at least 3 whole steps and as many more as fit about budget_s, all threads; then the same step
+    on one thread (bounded)."""
     from jabas_amd.layout import FlatLayout
     from oracle.unfused_baseline import UnfusedStep
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
@@ -179,9 +293,9 @@ def cpu_baseline(cfg, torch, budget_s=25.0):
     numel = sum(s.numel for s in cfg.specs)
     st = UnfusedStep(layout, cfg.batches, gdt, cfg.grad_std, cfg.opt)
     t0 = time.perf_counter()
-    st.step(cfg.stats)                                 # warm-up (allocates optimizer state)
+    st.step(cfg.stats)
     first = time.perf_counter() - t0
-    iters = int(max(2, min(8, (budget_s - first) / max(first, 1e-3))))
+    iters = int(max(3, min(8, (budget_s - first) / max(first, 1e-3))))
     times = []
     for _ in range(iters):
         t0 = time.perf_counter()
@@ -190,13 +304,12 @@ def cpu_baseline(cfg, torch, budget_s=25.0):
     times.sort()
     med = times[len(times) // 2]
     bytes_per_step = numel * algorithmic_bytes_per_elem(cfg)
-    # the same step on one host thread (bounded: at most 3 steps or ~10 s)
     threads = torch.get_num_threads()
     torch.set_num_threads(1)
     one = []
     try:
         t_begin = time.perf_counter()
-        while len(one) < 3 and (not one or time.perf_counter() - t_begin + one[-1] < 10.0):
+        while len(one) < 2 and (not one or time.perf_counter() - t_begin + one[-1] < budget_s / 3):
             t0 = time.perf_counter()
             st.step(cfg.stats)
             one.append(time.perf_counter() - t0)
@@ -204,12 +317,12 @@ def cpu_baseline(cfg, torch, budget_s=25.0):
         torch.set_num_threads(threads)
     one_best = min(one)
     return dict(value=bytes_per_step / 1e9 / med, unit="GB/s", cores=threads, kind="port",
-                ms_per_step=med * 1e3,
+                ms_per_step=med * 1e3, steps=iters,
                 one_thread=dict(value=bytes_per_step / 1e9 / one_best, unit="GB/s", cores=1,
                                 ms_per_step=one_best * 1e3, steps=len(one)),
                 sample=f"{cfg.name} full gradient set ({numel} elements), unfused torch CPU ops "
                        f"(K in-place aggregate passes, per-bucket clone+scale, cat + cosine_similarity, "
-                       f"torch.optim single-tensor loop), median of {iters} steps after 1 warm-up")
+                       f"torch.optim single-tensor loop), median of {iters} whole steps after 1 warm-up")
 
 
 def main():
@@ -217,13 +330,15 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="vit_b16")
+    ap.add_argument("--workload", default="vit_l16")
     ap.add_argument("--no-all", action="store_true", help="time only the headline workload")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0,
+                    help="CPU time the headline's baseline may take; the other workloads get a third each")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 1 GiB copy 5 times (the K=1, weight-1 aggregate: same 16-byte "
-                         "nontemporal loads and stores as the fused kernel, known traffic) for scaling "
-                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
+                    help="also run a plain 1 GiB copy 5 times before anything else (the K=1, weight-1 aggregate: "
+                         "same 16-byte nontemporal loads and stores as the fused kernel, known traffic) for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures the one-GPU share of the gradient-sync path; "
@@ -249,37 +364,53 @@ def main():
     results = {}
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
     for cfg in order:
-        results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch)
-        r = results[cfg.name]
+        r = results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch)
+        r["hbm_traffic_bytes_per_launch"] = measured_traffic(cfg.name)
         extra = ""
-        if r["step_without_statistics"]:
-            extra = (f"; without statistics {r['step_without_statistics']['ms_per_step']:.4f} ms/step, "
-                     f"{r['step_without_statistics']['pct_hbm_peak']:.1f} %")
+        if r.get("step_without_statistics"):
+            extra = (f"; without statistics {r['step_without_statistics']['ms_per_step']:.4f} ms "
+                     f"{r['step_without_statistics']['pct_hbm_peak']:.1f} %; per-VSW norms too "
+                     f"{r['step_with_per_vsw_norms']['pct_hbm_peak']:.1f} %")
         print(f"# {cfg.name}: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s, "
-              f"{r['pct_hbm_peak']:.1f} % of HBM peak{extra}", file=sys.stderr, flush=True)
+              f"{r['pct_hbm_peak']:.1f} % of HBM peak{extra}; hooks per bucket "
+              f"{r['hook_path_per_bucket_ms']['ms_per_step']:.4f} ms, deferred "
+              f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms", file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
                                                                       args.steps, torch)
+    copy_gbps = copy_rate(device, args.steps, torch)
+    stat_launches = None if args.no_all else statistics_launches(device, args.steps, torch)
     head = results[head_cfg.name]
+    if not args.no_cpu:
+        for cfg in order:
+            budget = args.cpu_seconds if cfg.name == head_cfg.name else args.cpu_seconds / 3.0
+            results[cfg.name]["cpu_baseline"] = cpu_baseline(cfg, torch, budget)
+            c = results[cfg.name]["cpu_baseline"]
+            print(f"# cpu {cfg.name}: {c['ms_per_step']:.1f} ms/step on {c['cores']} threads ({c['steps']} steps), "
+                  f"{c['one_thread']['ms_per_step']:.1f} ms on one", file=sys.stderr, flush=True)
     bytes_per_launch = head["GB_per_step"] * 1e9
-    roofline = dict(bound="hbm", achieved=head["GBps_launch"], peak=HBM_PEAK_GBPS, unit="GB/s",
-                    frac=head["GBps_launch"] / HBM_PEAK_GBPS,
-                    traffic=MEASURED_TRAFFIC_BYTES.get(head_cfg.name),
+    # one fused-kernel launch per step (plus the statistics' finalize launch, about 1 % of it): the mean
+    # launch duration is the HIP-event time of the timed region over its steps
+    roofline = dict(bound="hbm", achieved=head["GBps"], peak=HBM_PEAK_GBPS, unit="GB/s",
+                    frac=head["GBps"] / HBM_PEAK_GBPS, traffic=head["hbm_traffic_bytes_per_launch"],
+                    traffic_source=TRAFFIC_FILE if head["hbm_traffic_bytes_per_launch"] is not None else None,
                     kernel="jabas::fused_kernel", algorithmic_bytes_per_launch=bytes_per_launch,
-                    launch_ms=head["launch_ms_mean"])
-    cpu = None if args.no_cpu else cpu_baseline(head_cfg, torch)
+                    launch_ms=head["ms_per_step"], launch_ms_isolated=head["launch_ms_mean"],
+                    copy_GBps=copy_gbps)
     out = {
         "metric": "sync_step_GBps", "value": head["GBps"], "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
         "config": {"workload": head_cfg.name, "elements": head["elements"], "K": head["K"],
                    "batches": head["batches"], "grad_dtype": head["grad_dtype"], "optimizer": head["optimizer"],
                    "stats": head["stats"], "bytes_per_elem": head["bytes_per_elem"]},
         "pct_hbm_peak": head["pct_hbm_peak"],
         "roofline": roofline,
-        "cpu_baseline": cpu,
+        "cpu_baseline": head.get("cpu_baseline"),
+        "copy_GBps": copy_gbps,
         "workloads": list(results.values()),
+        "statistics_launches": stat_launches,
     }
     print(json.dumps(out))
 

@@ -115,6 +115,7 @@ class LocalBucketSync:
         self._args_cache = {}
         self._launch_streams = set()           # streams that carry launches of the current step
         self._errors = []
+        self._events = {}                      # (bucket index, VSW) -> ordering event, reused every step
         self._momentum_ready = False           # SGD: the momentum buffers hold a first step
         self._bound_steps = []                 # optimizer.state dictionaries whose 'step' follows step_count
         self.launched = 0                      # fused launches queued so far
@@ -261,12 +262,18 @@ class LocalBucketSync:
         if tensor.is_cuda:
             stream = torch.cuda.current_stream(tensor.device)
             if not self.deferred and (k != 0 or self._sync_stream is not None):
-                event = torch.cuda.Event()     # VSW 0's own stream needs none when the launch is queued on it
+                # VSW 0's own stream needs none when the launch is queued on it. One event per (bucket, VSW),
+                # recorded anew every step: its last use (the launch stream's wait of the step before) is over
+                event = self._events.get((bucket_index, k))
+                if event is None:
+                    event = self._events[(bucket_index, k)] = torch.cuda.Event()
                 event.record(stream)
         with self._lock:
             if stream is not None:
                 self._vsw_streams[k] = stream  # deferred mode orders once per VSW stream in finish_step
-            slot = self._slots.setdefault(bucket_index, _Slot(self.K))
+            slot = self._slots.get(bucket_index)
+            if slot is None:
+                slot = self._slots[bucket_index] = _Slot(self.K)
             if slot.tensors[k] is not None:
                 raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
             slot.tensors[k], slot.events[k], slot.buckets[k] = tensor, event, bucket
