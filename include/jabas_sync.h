@@ -38,8 +38,8 @@ extern "C" {
 #define JABAS_MAX_K 16          /* VSWs aggregated by one launch                      */
 #define JABAS_MAX_GROUPS 16     /* optimizer parameter groups per launch              */
 #define JABAS_STATS_STRIDE 20   /* doubles per span in stats_out: 4 + JABAS_MAX_K     */
-#define JABAS_GRAM_MAX_K 8      /* VSWs of one jabas_gram call                        */
-#define JABAS_GRAM_STRIDE 64    /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
+#define JABAS_GRAM_MAX_K 16     /* VSWs of one jabas_gram call                        */
+#define JABAS_GRAM_STRIDE 256   /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
 #define JABAS_STATIC_MAX_NUMEL (1ull << 26)  /* largest span of jabas_sync_bucket_static  */
 
 typedef void* jabas_stream_t;   /* hipStream_t */
@@ -249,8 +249,8 @@ int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype,
 /* K x K Gram matrix of the worker gradients, gram_out[a*JABAS_GRAM_MAX_K + b] = sum g_a*g_b
  * (fp64 products and sums), symmetric, JABAS_GRAM_STRIDE doubles. The "between
  * workers" statistics; no reference counterpart beyond the pairwise cosine of
- * jabas/train/trainer.py:478. K <= JABAS_GRAM_MAX_K (the K(K+1)/2 running sums live in
- * registers); JABAS_ERR_K above that. */
+ * jabas/train/trainer.py:478. K <= JABAS_GRAM_MAX_K. workspace: at least
+ * 1024 * JABAS_GRAM_STRIDE doubles (one tile of partial sums per workgroup). */
 int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype,
                uint64_t numel, double* gram_out,
                void* workspace, size_t workspace_bytes, jabas_stream_t stream);

@@ -14,8 +14,8 @@ LIB_PATH = os.environ.get("JABAS_SYNC_LIB") or os.path.join(_HERE, "csrc", "libj
 MAX_K = 16
 MAX_GROUPS = 16
 STATS_STRIDE = 20
-GRAM_MAX_K = 8
-GRAM_STRIDE = 64
+GRAM_MAX_K = 16
+GRAM_STRIDE = 256
 STATIC_MAX_NUMEL = 1 << 26
 
 F32, BF16 = 0, 1

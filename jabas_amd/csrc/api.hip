@@ -386,7 +386,7 @@ JABAS_API const char* jabas_status_string(int status) {
     switch (status) {
         case JABAS_OK: return "ok";
         case JABAS_ERR_NULL: return "a required pointer is NULL";
-        case JABAS_ERR_K: return "K outside 1..16 (1..8 for jabas_gram) or half_id not 0/1";
+        case JABAS_ERR_K: return "K outside 1..16 or half_id not 0/1";
         case JABAS_ERR_ALIGN: return "buffers of a span are not mutually congruent modulo 16 bytes";
         case JABAS_ERR_DTYPE: return "unsupported gradient dtype";
         case JABAS_ERR_OPT: return "unknown optimizer kind or inconsistent optimizer arguments";

@@ -1,12 +1,25 @@
 // K x K Gram matrix of the K worker gradients of one span: gram[a][b] = sum_e g_a[e]*g_b[e].
-// fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums. Grid-stride over 4-element
-// vectors, K(K+1)/2 accumulators per thread, wave64 shuffle tree -> LDS -> one packed
-// partial row per workgroup, then a single-workgroup finalize that sums the rows in a fixed
-// order and mirrors the lower triangle.
+// fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums, fixed order: bit-identical run to run.
+//   K <= 8   grid-stride over 4-element vectors, K(K+1)/2 fp64 accumulators per thread on the vector
+//            ALU, wave64 shuffle tree -> LDS -> one packed partial row per workgroup;
+//   K >= 9   the Gram matrix is a contraction over the elements, X X^T with X the K x N matrix of the
+//            workers' gradients: v_mfma_f64_16x16x4 with the SAME register as A and B operand (lane l
+//            holds X[l % 16][l / 16] of a 16 x 4 slice, which is both A[i][k] and B[k][j] = A[j][k]).
+//            The 256 running sums of the 16 x 16 tile take 8 registers per lane instead of K(K+1)/2
+//            register pairs per thread, which is what limited the vector-ALU form to K <= 8. For K <= 8
+//            the 16 rows hold two (K <= 4: four ...) element groups of the K workers, and the diagonal
+//            blocks of the tile are added up at the end.
+// Then a single-workgroup finalize that sums the workgroup rows in a fixed order.
 #include "jabas_internal.h"
+
+#ifndef JABAS_GRAM_VALU_MAX_K
+#define JABAS_GRAM_VALU_MAX_K 8
+#endif
 
 namespace jabas {
 namespace {
+
+constexpr int kGramValuMaxK = JABAS_GRAM_VALU_MAX_K;   // up to here the vector-ALU kernel, beyond it the matrix cores
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -124,6 +137,99 @@ __global__ void __launch_bounds__(kGramFinalizeBlock) gram_finalize_kernel(int K
     }
 }
 
+
+// ---- K >= 9: fp64 matrix cores -------------------------------------------------------------------------
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+constexpr int kGramRunBlocks = 4;                // element blocks a wave loads before it multiplies
+
+// Rows of the 16 x 16 tile: row r = group * Kp + worker, Kp = K rounded up to a power of two, 16 / Kp
+// element groups. A block is 16 * (16 / Kp) consecutive elements: lane (r, ks) reads the four elements at
+// group * 16 + ks * 4 of its worker, so every worker's part of a block is one contiguous stretch of 64 to
+// 256 bytes and a run of blocks a contiguous kilobyte or more. Four MFMAs per load: the j-th takes element
+// j of every lane's vector (which element sits in which k slot does not matter as long as A and B agree,
+// and they are the same register).
+template <int DT>
+__global__ void __launch_bounds__(kBlock) gram_mfma_kernel(const SpanDev sp, int K, int log_kp, double* partials) {
+    using L = GramLoad<DT>;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, ks = lane >> 4;
+    const int kp = 1 << log_kp;
+    const int worker = r & (kp - 1), group = r >> log_kp;
+    const int groups = 16 >> log_kp;
+    const uint64_t block_elems = 16ull * groups;
+    const uint64_t n_blocks = (sp.hi + block_elems - 1) / block_elems;
+    const bool row_live = worker < K;
+    const void* base = sp.g[row_live ? worker : 0];
+    const uint32_t lane_off = static_cast<uint32_t>(group) * 16u + static_cast<uint32_t>(ks) * 4u;
+    f64x4 acc = {0.0, 0.0, 0.0, 0.0}, acc1 = {0.0, 0.0, 0.0, 0.0};     // two chains: a multiply need not wait for the one before
+    const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWaves;
+    const uint64_t n_runs = (n_blocks + kGramRunBlocks - 1) / kGramRunBlocks;
+    for (uint64_t run = static_cast<uint64_t>(blockIdx.x) * kWaves + wave; run < n_runs; run += n_waves) {
+        float x[kGramRunBlocks][4];
+#pragma unroll
+        for (int u = 0; u < kGramRunBlocks; ++u) {
+            const uint64_t e = (run * kGramRunBlocks + u) * block_elems + lane_off;
+            if (row_live && e >= sp.lo && e + 4 <= sp.hi) {
+                L::vec(base, e, x[u]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    x[u][i] = (row_live && e + i >= sp.lo && e + i < sp.hi) ? L::one(base, e + i) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGramRunBlocks; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; i += 2) {
+                const double d0 = static_cast<double>(x[u][i]), d1 = static_cast<double>(x[u][i + 1]);
+                acc = __builtin_amdgcn_mfma_f64_16x16x4f64(d0, d0, acc, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f64_16x16x4f64(d1, d1, acc1, 0, 0, 0);
+            }
+    }
+    acc += acc1;
+    // the four waves' tiles, added in wave order: entry t = v * 64 + lane of the tile is register v of lane
+    __shared__ double red[kWaves][256];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][v * 64 + lane] = acc[v];
+    __syncthreads();
+    const int t = threadIdx.x;
+    double s = red[0][t];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) s += red[w][t];
+    partials[static_cast<uint64_t>(blockIdx.x) * JABAS_GRAM_STRIDE + t] = s;
+}
+
+// Sums the workgroup tiles (1024 threads: thread (entry, part) adds rows part, part + 4, ... in order, the
+// four parts in order), then folds the diagonal blocks: gram[a][b] = sum over groups of
+// tile[group * Kp + a][group * Kp + b]. Register v of lane l holds tile[4 * v + l / 16][l % 16].
+constexpr int kGramMfmaFinalizeBlock = 1024;
+__global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_kernel(int K, int log_kp, const double* partials,
+                                                                                    unsigned grid, double* gram_out) {
+    __shared__ double part_sum[4][256];
+    __shared__ double tile[256];
+    const int t = threadIdx.x, e = t & 255, part = t >> 8;
+    double s = 0.0;
+#pragma unroll 8
+    for (unsigned b = part; b < grid; b += 4) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + e];
+    part_sum[part][e] = s;
+    __syncthreads();
+    if (t < 256) tile[t] = ((part_sum[0][t] + part_sum[1][t]) + part_sum[2][t]) + part_sum[3][t];
+    __syncthreads();
+    if (t < JABAS_GRAM_STRIDE) {
+        const int a = t / JABAS_GRAM_MAX_K, b = t % JABAS_GRAM_MAX_K;
+        double out = 0.0;
+        if (a < K && b < K) {
+            const int lo = a < b ? a : b, hi = a < b ? b : a;      // one triangle, mirrored: symmetric bit for bit
+            const int kp = 1 << log_kp;
+            for (int g = 0; g < (16 >> log_kp); ++g) {
+                const int i = g * kp + lo, j = g * kp + hi;
+                out += tile[(i >> 2) * 64 + (i & 3) * 16 + j];
+            }
+        }
+        gram_out[t] = out;
+    }
+}
+
 template <int K>
 int launch_gram_k(int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
     if (grad_dtype == JABAS_BF16)
@@ -134,20 +240,35 @@ int launch_gram_k(int grad_dtype, const SpanDev& sp, double* partials, unsigned 
 }  // namespace
 
 int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
+    if (K > kGramValuMaxK) {
+        int log_kp = 0;
+        while ((1 << log_kp) < K) ++log_kp;
+        if (grad_dtype == JABAS_BF16)
+            return static_cast<int>(launch_kernel(gram_mfma_kernel<JABAS_BF16>, dim3(grid), dim3(kBlock), 0, stream, sp, K, log_kp, partials));
+        return static_cast<int>(launch_kernel(gram_mfma_kernel<JABAS_F32>, dim3(grid), dim3(kBlock), 0, stream, sp, K, log_kp, partials));
+    }
     switch (K) {
         case 1: return launch_gram_k<1>(grad_dtype, sp, partials, grid, stream);
         case 2: return launch_gram_k<2>(grad_dtype, sp, partials, grid, stream);
         case 3: return launch_gram_k<3>(grad_dtype, sp, partials, grid, stream);
         case 4: return launch_gram_k<4>(grad_dtype, sp, partials, grid, stream);
+#if JABAS_GRAM_VALU_MAX_K > 4
         case 5: return launch_gram_k<5>(grad_dtype, sp, partials, grid, stream);
         case 6: return launch_gram_k<6>(grad_dtype, sp, partials, grid, stream);
         case 7: return launch_gram_k<7>(grad_dtype, sp, partials, grid, stream);
         case 8: return launch_gram_k<8>(grad_dtype, sp, partials, grid, stream);
+#endif
         default: return -1;
     }
 }
 
 int launch_gram_finalize(int K, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
+    if (K > kGramValuMaxK) {
+        int log_kp = 0;
+        while ((1 << log_kp) < K) ++log_kp;
+        return static_cast<int>(launch_kernel(gram_mfma_finalize_kernel, dim3(1), dim3(kGramMfmaFinalizeBlock), 0, stream, K, log_kp,
+                                              partials, grid, gram_out));
+    }
     return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(kGramFinalizeBlock), 0, stream, K, partials, grid, gram_out));
 }
 

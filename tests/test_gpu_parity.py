@@ -174,24 +174,37 @@ def test_stats_cosine_identities(gpu):
     assert sync.cosine_from_stats(sync.gradient_stats([z, z], (1, 1))) == 0.0
 
 
-@pytest.mark.parametrize("K", [1, 2, 5, 8])
+@pytest.mark.parametrize("K", list(range(1, 17)))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gram(gpu, K, dtype):
+    """K <= 4: fp64 on the vector ALU; K >= 5: fp64 matrix cores over a 16 x 16 tile whose rows are the
+    workers (twice over for K <= 8). Either way exact fp64 products, 1e-11 against the float64 oracle."""
     from jabas_amd import sync
-    for n, skew in ((7, 0), (100003, 2), (1 << 20, 0), (100003, 61)):
+    for n, skew in ((7, 0), (100003, 2), (1 << 20, 0), (100003, 61), (3_000_001, 5)):
         hg = _host_grads(K, n, 30 + K, dtype=dtype)
         G = sync.gram([_dev(t, gpu, skew) for t in hg]).cpu()
         want = O.gram(hg)
-        assert _close(G, want, 1e-11, 1e-30)[0], f"K={K} n={n}"
+        # off-diagonal entries cancel: their error is measured against |g_a| |g_b|
+        scale = torch.sqrt(torch.outer(torch.diagonal(want), torch.diagonal(want)))
+        assert bool(((G - want).abs() <= 1e-12 * scale + 1e-30).all()), f"K={K} n={n}"
+        assert _close(torch.diagonal(G), torch.diagonal(want), 1e-11, 1e-30)[0], f"K={K} n={n}"
         assert torch.equal(G, G.t())
 
 
-def test_gram_is_limited_to_eight_workers(gpu):
+def test_gram_limits_and_determinism(gpu):
     from jabas_amd import sync, _lib as L
-    g = [torch.zeros(4096, device=gpu) for _ in range(9)]
+    g = [torch.zeros(4096, device=gpu) for _ in range(17)]
     with pytest.raises(L.JabasSyncError) as e:
         sync.gram(g)
     assert e.value.status == L.ERR_K
+    hg = _host_grads(11, 2_000_003, 77)
+    dg = [_dev(t, gpu, 3) for t in hg]
+    a = sync.gram(dg).cpu().clone()
+    for _ in range(3):
+        assert torch.equal(sync.gram(dg).cpu().view(torch.int64), a.view(torch.int64))
+    # the diagonal is the per-worker norm row of the statistics kernel's full level
+    row = sync.gradient_stats(dg, BATCHES[11]).cpu()
+    assert torch.allclose(torch.diagonal(a), row[4:4 + 11], rtol=1e-12, atol=0.0)
 
 
 # ---------------------------------------------------------------------------- optimizer
