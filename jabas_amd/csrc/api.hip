@@ -17,7 +17,10 @@ int launch_gram_finalize(int K, const double* partials, unsigned grid, double* g
 
 namespace {
 
-constexpr uint64_t kGramGrid = 1024;     // persistent workgroups of the Gram kernel
+#ifndef JABAS_GRAM_GRID
+#define JABAS_GRAM_GRID 1024
+#endif
+constexpr uint64_t kGramGrid = JABAS_GRAM_GRID;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
 constexpr uint32_t kPlanVersion = 7;
 

@@ -140,7 +140,10 @@ __global__ void __launch_bounds__(kGramFinalizeBlock) gram_finalize_kernel(int K
 
 // ---- K >= 9: fp64 matrix cores -------------------------------------------------------------------------
 typedef double f64x4 __attribute__((ext_vector_type(4)));
-constexpr int kGramRunBlocks = 4;                // element blocks a wave loads before it multiplies
+#ifndef JABAS_GRAM_RUN
+#define JABAS_GRAM_RUN 4
+#endif
+constexpr int kGramRunBlocks = JABAS_GRAM_RUN;   // element blocks a wave loads before it multiplies
 
 // Rows of the 16 x 16 tile: row r = group * Kp + worker, Kp = K rounded up to a power of two, 16 / Kp
 // element groups. A block is 16 * (16 / Kp) consecutive elements: lane (r, ks) reads the four elements at

@@ -402,7 +402,7 @@ def gram(grads, stream=None):
     span = SpanSpec(grads)
     n, dev, gdt = span.validate()
     K = len(grads)
-    ws = torch.empty(1024 * L.GRAM_STRIDE, dtype=torch.float64, device=dev)
+    ws = torch.empty(2048 * L.GRAM_STRIDE, dtype=torch.float64, device=dev)
     out = torch.empty(L.GRAM_STRIDE, dtype=torch.float64, device=dev)
     L.check(L.lib().jabas_gram(_ptr_array(grads), K, grad_dtype_code(gdt), n, out.data_ptr(), ws.data_ptr(),
                                ws.numel() * 8, _stream_ptr(stream)), "jabas_gram")
