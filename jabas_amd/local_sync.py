@@ -117,7 +117,7 @@ class LocalBucketSync:
         self._errors = []
         self._events = {}                      # (bucket index, VSW) -> ordering event, reused every step
         self._momentum_ready = False           # SGD: the momentum buffers hold a first step
-        self._bound_steps = []                 # optimizer.state dictionaries whose 'step' follows step_count
+        self._bound_steps = {}                 # id -> optimizer.state dictionary whose 'step' follows step_count
         self.launched = 0                      # fused launches queued so far
         self.launched_with_opt = 0             # of them, launches that updated weights
         if optimizer is not None:
@@ -207,7 +207,7 @@ class LocalBucketSync:
                             raise RuntimeError("a parameter's Adam step count differs from the steps taken here")
                         self.step_count = int(float(st["step"]))        # state carried in from earlier steps
                     st["step"] = self.step_count
-                    self._bound_steps.append(st)
+                    self._bound_steps[id(st)] = st
             if sgd and had_state:
                 if had_state != len(params) and self.opt.get("dampening", 0.0) != 0.0:
                     raise RuntimeError("some parameters of a bucket hold a momentum buffer and some do not: "
@@ -495,5 +495,5 @@ class LocalBucketSync:
         self.step_count += 1
         if self.launched_with_opt:
             self._momentum_ready = True
-        for st in self._bound_steps:
+        for st in self._bound_steps.values():
             st["step"] = self.step_count

@@ -263,3 +263,43 @@ def test_shard_optimizer_constructors_validate_like_torch():
     g = torch.ones(4)
     with pytest.raises(ValueError, match="index"):
         optim.ShardSGD(p, lr=0.1).step([g])
+
+
+def test_statistics_levels_and_their_names():
+    from jabas_amd import sync, _lib as L
+    assert [sync.stats_level(x) for x in (None, False, 0)] == [L.STATS_NONE] * 3
+    assert [sync.stats_level(x) for x in (True, 1, "full")] == [L.STATS_FULL] * 3
+    assert [sync.stats_level(x) for x in (2, "similarity")] == [L.STATS_SIMILARITY] * 2
+    with pytest.raises(ValueError):
+        sync.stats_level("everything")
+    assert LocalBucketSync([1, 1], launcher=Recorder()).stats_level == L.STATS_SIMILARITY
+    assert LocalBucketSync([1, 1], launcher=Recorder(), stats_level="full").stats_level == L.STATS_FULL
+    args = sync.make_step_args((3, 1), torch.float32, stats="similarity")
+    assert args.stats == L.STATS_SIMILARITY and args.K == 2
+
+
+def test_optimizer_hook_needs_the_rendezvous_when_there_are_several_workers():
+    """With K > 1 workers the update belongs to the launch the rendezvous queues; a hook that stepped the
+    optimizer on its own would read VSW 0's bucket before the other VSWs' gradients are in it."""
+    opt = torch.optim.SGD([torch.nn.Parameter(torch.zeros(3))], lr=0.1)
+    hook = create_optimizer_hook(H.iidp_allreduce_hook, opt)
+    with pytest.raises(RuntimeError, match="LocalBucketSync"):
+        hook(H.IIDPState(None, 4), NewBucket(0, torch.ones(3)))
+    # with a rendezvous attached the optimizer is bound to it and the hook is the plain hook
+    local = LocalBucketSync([2, 2], launcher=Recorder())
+    state = H.IIDPState(None, 2).attach_local(local)
+    fut = hook(state, NewBucket(0, torch.ones(3)))
+    assert fut.done() and local.optimizer is opt and local.opt["kind"] == "sgd"
+    with pytest.raises(RuntimeError, match="already bound"):
+        local.bind_optimizer(torch.optim.SGD([torch.nn.Parameter(torch.zeros(3))], lr=0.1))
+
+
+def test_shard_gnmt_adam_constructor_follows_the_reference():
+    p = [torch.nn.Parameter(torch.zeros(4)), torch.nn.Parameter(torch.zeros(2))]
+    o = optim.ShardGNMTAdam(p, lr=2e-3, grad_clip=5.0)
+    assert o.grad_clip == 5.0 and o.defaults["weight_decay"] == 0 and len(o.param_groups) == 1
+    assert optim.ShardGNMTAdam(p).grad_clip == float("inf")
+    with pytest.raises(ValueError, match="param_groups"):
+        optim.ShardGNMTAdam([{"params": p[:1]}, {"params": p[1:]}], grad_clip=1.0)
+    with pytest.raises(ValueError):
+        optim.ShardGNMTAdam(p, betas=(0.9, 1.0))
