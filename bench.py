@@ -19,7 +19,7 @@ duration = HIP-event time of the timed region on the launching stream / its laun
 "cpu_baseline" object (the reference's unfused PyTorch structure timed on this box's host
 cores, rank 0 only, a bounded number of whole steps). Every entry of "workloads" carries
 its own figures of both, the step as the reference's calling convention reaches it (one
-hook call per bucket and VSW, per bucket and deferred), and the neighbouring launches
+hook call per bucket and VSW: one launch per bucket, per 64 MiB of buckets, per step), and the neighbouring launches
 (without statistics, with full statistics rows).
 """
 import argparse
@@ -124,7 +124,7 @@ class _Bucket:
         return self._t
 
 
-def hook_path(cfg, eng, device, steps, warmup, torch, deferred):
+def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0):
     """The same step as the reference's calling convention reaches it: per bucket, VSW 0's similarity
     hook (with the optimizer bound: the overlap weight-sync mode) and K - 1 dummy hooks, each handing
     over its bucket view; one fused launch per bucket (or one per step, deferred) on a launch stream
@@ -139,7 +139,8 @@ def hook_path(cfg, eng, device, steps, warmup, torch, deferred):
                       state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds,
                       agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
     stream = torch.cuda.Stream(device)
-    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, deferred=deferred, stream=stream)
+    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, deferred=deferred, stream=stream,
+                            batch_bytes=batch_bytes)
     local.step_count = eng.step_count
     local._momentum_ready = eng.step_count > 0
     state = H.GradientSimilarityState(None, cfg.K + cfg.K % 2, None, [], 1 if cfg.stats else 10 ** 9).attach_local(local)
@@ -156,9 +157,12 @@ def hook_path(cfg, eng, device, steps, warmup, torch, deferred):
         local.finish_step((cur,))
         state.grad_placeholder.clear()
 
-    ms, wall = timed_region(one_step, steps, warmup, torch)
+    for i in range(warmup):                         # the first steps create streams' and events' pools
+        one_step(i)
+    launched_before = local.launched
+    ms, wall = timed_region(one_step, steps, 0, torch)
     eng.step_count = local.step_count
-    return dict(ms_per_step=ms, wall_ms_per_step=wall, launches_per_step=1 if deferred else len(buckets))
+    return dict(ms_per_step=ms, wall_ms_per_step=wall, launches_per_step=(local.launched - launched_before) / steps)
 
 
 def time_config(cfg, device, steps, warmup, torch, extras=True):
@@ -192,8 +196,9 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         ms, _ = timed_region(lambda i: engines[i % n].step(stats="full"), steps, warmup, torch)
         res["step_with_per_vsw_norms"] = rate(bytes_per_step, ms)
     if extras:
-        hsteps, hwarm = max(5, steps // 2), max(2, warmup // 2)
+        hsteps, hwarm = max(5, steps // 2), max(10, warmup)
         res["hook_path_per_bucket_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False)
+        res["hook_path_batched_64MiB_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False, 64 << 20)
         res["hook_path_deferred_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, True)
     if cfg.name == "gnmt" and extras:
         # global-norm clipping (examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
@@ -373,7 +378,8 @@ def main():
                      f"{r['step_with_per_vsw_norms']['pct_hbm_peak']:.1f} %")
         print(f"# {cfg.name}: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s, "
               f"{r['pct_hbm_peak']:.1f} % of HBM peak{extra}; hooks per bucket "
-              f"{r['hook_path_per_bucket_ms']['ms_per_step']:.4f} ms, deferred "
+              f"{r['hook_path_per_bucket_ms']['ms_per_step']:.4f} ms, batched "
+              f"{r['hook_path_batched_64MiB_ms']['ms_per_step']:.4f} ms, deferred "
               f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms", file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,

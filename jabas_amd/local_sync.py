@@ -46,6 +46,7 @@ class _Slot:
         self.tensors = [None] * K
         self.buckets = [None] * K
         self.events = [None] * K
+        self.seq = [0] * K
         self.want_stats = False
         self.on_done = None
         self.count = 0
@@ -71,12 +72,19 @@ class LocalBucketSync:
     """
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
-                 optimizer=None, stats_level="similarity"):
+                 optimizer=None, stats_level="similarity", batch_bytes=0):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
         (one ramp-up and drain: 0.68 ms against 0.9 ms wall for the 14 buckets of ViT-B/16) and less host
         time, and the buckets hold the aggregate only after ``finish_step``.
+
+        batch_bytes: between the two: complete buckets are held back until this many bytes of them (size of
+        one VSW's buffers) are ready, then go out as ONE planned launch behind one event wait per VSW
+        (what remains at the end of the step goes out in ``finish_step``). The sync still overlaps the
+        backward passes, in coarser steps; every launch costs the host K stream waits and the GPU a ramp-up
+        and drain, which is what batching divides (14 x 25 MB buckets of ViT-B/16 in batches of 64 MB: five
+        launches instead of fourteen). 0: one launch per bucket.
 
         stats_level: what a statistic step computes per bucket: "similarity" (the four sums the cosine between
         the halves and norm clipping read: all the reference's adaptive batching consumes,
@@ -93,10 +101,17 @@ class LocalBucketSync:
         if deferred and launcher is not None:
             raise ValueError("the deferred mode drives the C ABI itself: no launcher can be injected")
         self.deferred = bool(deferred)
+        self.batch_bytes = 0 if deferred else int(batch_bytes)
+        if self.batch_bytes and launcher is not None:
+            raise ValueError("batched launches drive the C ABI themselves: no launcher can be injected")
+        self._ready_bytes = 0
+        self._seq = [0] * len(tuple(batches))  # per VSW: buckets published so far (orders its events)
+        self._plans = {}                       # batched mode: group of buckets -> its plan
+        self._stream_cache = {}
         self.stats_level = sync.stats_level(stats_level) or L.STATS_SIMILARITY
-        self._ready = {}                       # deferred mode: bucket index -> complete _Slot of this step
+        self._ready = {}                       # deferred / batched mode: bucket index -> complete _Slot not launched yet
         self._vsw_streams = {}                 # VSW index -> the stream its hooks ran on in this step
-        self._plan = self._plan_key = None
+        self._plan = None                      # the planned launch used last (deferred / batched mode)
         self.batches = tuple(batches)
         self.K = len(self.batches)
         self.opt = opt
@@ -115,7 +130,6 @@ class LocalBucketSync:
         self._args_cache = {}
         self._launch_streams = set()           # streams that carry launches of the current step
         self._errors = []
-        self._events = {}                      # (bucket index, VSW) -> ordering event, reused every step
         self._momentum_ready = False           # SGD: the momentum buffers hold a first step
         self._bound_steps = {}                 # id -> optimizer.state dictionary whose 'step' follows step_count
         self.launched = 0                      # fused launches queued so far
@@ -240,7 +254,7 @@ class LocalBucketSync:
         self.param_buckets[bucket_index] = new
         with self._lock:
             self._calls.pop(bucket_index, None)
-            self._plan_key = None
+            self._plans.clear()
         return new
 
     def aggregate_of(self, bucket_index):
@@ -260,14 +274,14 @@ class LocalBucketSync:
         fut.set_result(tensor if value is None else value)
         event = stream = None
         if tensor.is_cuda:
-            stream = torch.cuda.current_stream(tensor.device)
+            stream = self._current_stream(tensor)
             if not self.deferred and (k != 0 or self._sync_stream is not None):
-                # VSW 0's own stream needs none when the launch is queued on it. One event per (bucket, VSW),
-                # recorded anew every step: its last use (the launch stream's wait of the step before) is over
-                event = self._events.get((bucket_index, k))
-                if event is None:
-                    event = self._events[(bucket_index, k)] = torch.cuda.Event()
+                # VSW 0's own stream needs none when the launch is queued on it. A fresh event every time:
+                # recording one event again step after step (to save its creation) made the waits on it
+                # three times as expensive on this runtime
+                event = torch.cuda.Event()
                 event.record(stream)
+        batch = None
         with self._lock:
             if stream is not None:
                 self._vsw_streams[k] = stream  # deferred mode orders once per VSW stream in finish_step
@@ -277,6 +291,8 @@ class LocalBucketSync:
             if slot.tensors[k] is not None:
                 raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
             slot.tensors[k], slot.events[k], slot.buckets[k] = tensor, event, bucket
+            self._seq[k] += 1
+            slot.seq[k] = self._seq[k]
             slot.count += 1
             if k == 0:
                 slot.want_stats, slot.on_done = want_stats, on_done
@@ -284,11 +300,26 @@ class LocalBucketSync:
             ready = slot.count == self.K
             if ready:
                 del self._slots[bucket_index]
-                if self.deferred:
+                if self.deferred or (self.batch_bytes and stream is not None):
                     self._ready[bucket_index] = slot
-        if ready and not self.deferred:
+                    self._ready_bytes += tensor.numel() * tensor.element_size()
+                    if not self.deferred and self._ready_bytes >= self.batch_bytes:
+                        batch, self._ready, self._ready_bytes = self._ready, {}, 0
+                    ready = False
+        if ready:
             self._fire(bucket_index, slot)
+        elif batch is not None:
+            self._fire_group(batch, per_publish_events=True)
         return fut
+
+    def _current_stream(self, tensor):
+        """torch.cuda.current_stream(tensor.device) without its per-call device bookkeeping (4.6 us a call,
+        as much as the rest of a publish): the Stream object of a raw stream is made once and kept."""
+        raw = torch._C._cuda_getCurrentStream(tensor.get_device())
+        stream = self._stream_cache.get(raw)
+        if stream is None:
+            stream = self._stream_cache[raw] = torch.cuda.Stream(stream_id=raw[0], device_index=raw[1], device_type=raw[2])
+        return stream
 
     def _launch_stream(self):
         return self._sync_stream if self._sync_stream is not None else self._main_stream
@@ -389,10 +420,10 @@ class LocalBucketSync:
                              bounds=(pb or {}).get("bounds", ()) if opt else ())
         return span, opt is not None
 
-    def _fire_all(self):
-        """Deferred mode: one planned launch over every bucket of the step, in bucket order."""
+    def _fire_group(self, ready, per_publish_events):
+        """One planned launch over a group of complete buckets, in bucket order: all buckets of the step
+        (deferred mode, from ``finish_step``) or a batch of them (batched mode)."""
         with self._lock:
-            ready, self._ready = self._ready, {}
             vsw_streams = sorted(self._vsw_streams.items())
         order = sorted(ready)
         slots = [ready[i] for i in order]
@@ -401,15 +432,25 @@ class LocalBucketSync:
             for i, slot in zip(order, slots):          # host tensors (protocol tests)
                 self._fire(i, slot)
             return
+        if len(order) == 1 and per_publish_events:
+            self._fire(order[0], slots[0])
+            return
         try:
-            # everything the VSWs queued up to now (their whole backward) precedes the launch: one
-            # event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
-            # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
-            for k, stream in vsw_streams:
-                if stream != main:
-                    ev = torch.cuda.Event()
-                    ev.record(stream)
-                    main.wait_event(ev)
+            if per_publish_events:
+                # per VSW, the event of the bucket it handed over last covers its earlier ones
+                for k in range(self.K):
+                    last = max(slots, key=lambda sl: sl.seq[k])
+                    if last.events[k] is not None:
+                        main.wait_event(last.events[k])
+            else:
+                # everything the VSWs queued up to now (their whole backward) precedes the launch: one
+                # event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
+                # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
+                for k, stream in vsw_streams:
+                    if stream != main:
+                        ev = torch.cuda.Event()
+                        ev.record(stream)
+                        main.wait_event(ev)
             for i, slot in zip(order, slots):
                 self._bind_bucket(i, slot)
         except Exception as exc:
@@ -425,19 +466,25 @@ class LocalBucketSync:
         try:
             key = tuple((i, slot.tensors[0].numel()) + tuple(t.data_ptr() for t in slot.tensors)
                         for i, slot in zip(order, slots))
-            if key != self._plan_key:                   # DDP hands over the same buffers every step: built once
+            with self._lock:
+                plan = self._plans.get(key)
+            if plan is None:                            # DDP hands over the same buffers every step: built once
                 spans = [self._span_of(i, slot.tensors)[0] for i, slot in zip(order, slots)]
-                self._plan = sync.SyncPlan(spans, sync.opt_kind(self.opt) if with_opt[0] else L.OPT_NONE)
-                self._plan_key = key
+                plan = sync.SyncPlan(spans, sync.opt_kind(self.opt) if with_opt[0] else L.OPT_NONE)
+                with self._lock:
+                    if len(self._plans) >= 256:
+                        self._plans.clear()
+                    self._plans[key] = plan
+            self._plan = plan
             want = any(slot.want_stats for slot in slots)
             args = self._step_args(slots[0].tensors[0].dtype, want, with_opt[0])
-            rows = self._plan.run(args, stream=main)
-            if with_opt[0]:
-                self.launched_with_opt += 1
+            rows = plan.run(args, stream=main)
             if rows is not None:
                 with torch.cuda.stream(main):
                     rows = rows.clone()                 # the plan's own rows are overwritten by its next launch
             with self._lock:
+                if with_opt[0]:
+                    self.launched_with_opt += 1
                 self._launch_streams.add(main)
         except Exception as exc:
             with self._lock:
@@ -459,6 +506,7 @@ class LocalBucketSync:
         with self._lock:
             self._slots.clear()
             self._ready.clear()
+            self._ready_bytes = 0
             self._launch_streams = set()
             self._vsw_streams = {}
             self._errors = []
@@ -472,8 +520,10 @@ class LocalBucketSync:
         if left:
             self.reset()
             raise RuntimeError(f"buckets {left} were not published by every VSW")
-        if self._ready:
-            self._fire_all()
+        with self._lock:
+            ready, self._ready, self._ready_bytes = self._ready, {}, 0
+        if ready:
+            self._fire_group(ready, per_publish_events=not self.deferred)
         # the launches of a step sit on one stream in order: one event behind the last of them orders
         # every VSW stream behind all of them
         with self._lock:
