@@ -1,25 +1,27 @@
 // K x K Gram matrix of the K worker gradients of one span: gram[a][b] = sum_e g_a[e]*g_b[e].
 // fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums, fixed order: bit-identical run to run.
-//   K <= 8   grid-stride over 4-element vectors, K(K+1)/2 fp64 accumulators per thread on the vector
-//            ALU, wave64 shuffle tree -> LDS -> one packed partial row per workgroup;
-//   K >= 9   the Gram matrix is a contraction over the elements, X X^T with X the K x N matrix of the
-//            workers' gradients: v_mfma_f64_16x16x4 with the SAME register as A and B operand (lane l
-//            holds X[l % 16][l / 16] of a 16 x 4 slice, which is both A[i][k] and B[k][j] = A[j][k]).
-//            The 256 running sums of the 16 x 16 tile take 8 registers per lane instead of K(K+1)/2
-//            register pairs per thread, which is what limited the vector-ALU form to K <= 8. For K <= 8
-//            the 16 rows hold two (K <= 4: four ...) element groups of the K workers, and the diagonal
-//            blocks of the tile are added up at the end.
+//   few workers    grid-stride over 4-element vectors, K(K+1)/2 fp64 accumulators per thread on the vector
+//                  ALU, wave64 shuffle tree -> LDS -> one packed partial row per workgroup (K <= 5 for fp32
+//                  gradients, K <= 8 for bf16);
+//   more, to 16    fp64 matrix cores: v_mfma_f64_4x4x4 over 4 x 4 blocks of worker pairs, fed from registers
+//                  (gram_mfma_kernel below).
 // Then a single-workgroup finalize that sums the workgroup rows in a fixed order.
 #include "jabas_internal.h"
 
 #ifndef JABAS_GRAM_VALU_MAX_K
-#define JABAS_GRAM_VALU_MAX_K 8
+#define JABAS_GRAM_VALU_MAX_K 5
 #endif
 
 namespace jabas {
 namespace {
 
-constexpr int kGramValuMaxK = JABAS_GRAM_VALU_MAX_K;   // up to here the vector-ALU kernel, beyond it the matrix cores
+#ifndef JABAS_GRAM_VALU_MAX_K_BF16
+#define JABAS_GRAM_VALU_MAX_K_BF16 8
+#endif
+// Up to here the vector-ALU kernel, beyond it the matrix cores. Measured on 86.6 M elements: fp32 K = 5: 5.95
+// against 4.96 TB/s, K = 6: 5.54 against 5.94, K = 8: 5.45 against 6.01; bf16 gradients (half the bytes for the same
+// arithmetic) K = 8: 5.45 against 4.15.
+constexpr int gram_valu_max_k(int grad_dtype) { return grad_dtype == JABAS_BF16 ? JABAS_GRAM_VALU_MAX_K_BF16 : JABAS_GRAM_VALU_MAX_K; }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -29,6 +31,12 @@ __device__ __forceinline__ float bits_to_float(uint32_t u) { return __builtin_bi
 template <int DT> struct GramLoad;
 template <> struct GramLoad<JABAS_F32> {
     static constexpr int EPT = 4;
+    using Raw = f32x4;
+    static __device__ __forceinline__ Raw raw(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + e));
+    }
+    static __device__ __forceinline__ float elem(const Raw& r, int i) { return r[i]; }
+    static __device__ __forceinline__ Raw from(const float (&x)[4]) { return Raw{x[0], x[1], x[2], x[3]}; }
     static __device__ __forceinline__ void vec(const void* base, uint64_t e, float (&x)[4]) {
         const f32x4 r = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + e));
         x[0] = r.x; x[1] = r.y; x[2] = r.z; x[3] = r.w;
@@ -37,6 +45,18 @@ template <> struct GramLoad<JABAS_F32> {
 };
 template <> struct GramLoad<JABAS_BF16> {
     static constexpr int EPT = 4;
+    using Raw = u32x2;
+    static __device__ __forceinline__ Raw raw(const void* base, uint64_t e) {
+        return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(base) + e));
+    }
+    static __device__ __forceinline__ float elem(const Raw& r, int i) {
+        const uint32_t w = i < 2 ? r.x : r.y;
+        return bits_to_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+    }
+    static __device__ __forceinline__ Raw from(const float (&x)[4]) {       // values that came from bf16: exact
+        return Raw{(__builtin_bit_cast(uint32_t, x[0]) >> 16) | (__builtin_bit_cast(uint32_t, x[1]) & 0xffff0000u),
+                   (__builtin_bit_cast(uint32_t, x[2]) >> 16) | (__builtin_bit_cast(uint32_t, x[3]) & 0xffff0000u)};
+    }
     static __device__ __forceinline__ void vec(const void* base, uint64_t e, float (&x)[4]) {
         const u32x2 r = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(base) + e));
         x[0] = bits_to_float(r.x << 16); x[1] = bits_to_float(r.x & 0xffff0000u);
@@ -138,82 +158,119 @@ __global__ void __launch_bounds__(kGramFinalizeBlock) gram_finalize_kernel(int K
 }
 
 
-// ---- K >= 9: fp64 matrix cores -------------------------------------------------------------------------
-typedef double f64x4 __attribute__((ext_vector_type(4)));
-#ifndef JABAS_GRAM_RUN
-#define JABAS_GRAM_RUN 4
+// ---- K >= 5: fp64 matrix cores, 4 x 4 blocks ----------------------------------------------------------
+// The Gram matrix is a contraction over the elements, X X^T with X the K x N matrix of the workers'
+// gradients. The workers are cut into G = ceil(K / 4) groups of four; v_mfma_f64_4x4x4 (four independent
+// 4 x 4 x 4 products per instruction) forms, for one pair of groups (ga <= gb), the 4 x 4 block of products
+// over four elements in each of its four products. Lane l is
+// worker l % 4 of every group and vector l / 4 of a 64-element block: it loads ONE 16-byte vector per group
+// (a wave reads 256 contiguous bytes of each worker) and feeds round r of every pair from registers,
+// A = element r of its vector of group ga, B = element r of its vector of group gb: no LDS, no shuffles,
+// G(G+1)/2 running sums per lane instead of K(K+1)/2 register pairs per thread (which is what limits the
+// vector-ALU form to K <= 8). Products of widened fp32 values are exact in fp64 and the order is fixed.
+// Per 64 elements: 4 G(G+1)/2 MFMAs and 4 G conversions per wave, against 36 fp64 multiply-adds and 8
+// conversions PER ELEMENT AND THREAD at K = 8 on the vector ALU.
+#ifndef JABAS_GRAM_RUN_F32
+#define JABAS_GRAM_RUN_F32 2
 #endif
-constexpr int kGramRunBlocks = JABAS_GRAM_RUN;   // element blocks a wave loads before it multiplies
+#ifndef JABAS_GRAM_RUN_BF16
+#define JABAS_GRAM_RUN_BF16 4
+#endif
+// 64-element blocks a wave loads before it multiplies (bf16 vectors are half as long: twice as many in flight)
+template <int DT> struct GramRun { static constexpr int value = DT == JABAS_BF16 ? JABAS_GRAM_RUN_BF16 : JABAS_GRAM_RUN_F32; };
 
-// Rows of the 16 x 16 tile: row r = group * Kp + worker, Kp = K rounded up to a power of two, 16 / Kp
-// element groups. A block is 16 * (16 / Kp) consecutive elements: lane (r, ks) reads the four elements at
-// group * 16 + ks * 4 of its worker, so every worker's part of a block is one contiguous stretch of 64 to
-// 256 bytes and a run of blocks a contiguous kilobyte or more. Four MFMAs per load: the j-th takes element
-// j of every lane's vector (which element sits in which k slot does not matter as long as A and B agree,
-// and they are the same register).
-template <int DT>
-__global__ void __launch_bounds__(kBlock) gram_mfma_kernel(const SpanDev sp, int K, int log_kp, double* partials) {
+template <int DT, int G>
+__global__ void __launch_bounds__(kBlock) gram_mfma_kernel(const SpanDev sp, int K, double* partials) {
     using L = GramLoad<DT>;
+    constexpr int P = G * (G + 1) / 2;
+    constexpr int kGramRunBlocks = GramRun<DT>::value;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = lane & 15, ks = lane >> 4;
-    const int kp = 1 << log_kp;
-    const int worker = r & (kp - 1), group = r >> log_kp;
-    const int groups = 16 >> log_kp;
-    const uint64_t block_elems = 16ull * groups;
-    const uint64_t n_blocks = (sp.hi + block_elems - 1) / block_elems;
-    const bool row_live = worker < K;
-    const void* base = sp.g[row_live ? worker : 0];
-    const uint32_t lane_off = static_cast<uint32_t>(group) * 16u + static_cast<uint32_t>(ks) * 4u;
-    f64x4 acc = {0.0, 0.0, 0.0, 0.0}, acc1 = {0.0, 0.0, 0.0, 0.0};     // two chains: a multiply need not wait for the one before
-    const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWaves;
+    const int wi = lane & 3;                           // worker inside its group
+    const uint32_t lane_off = static_cast<uint32_t>(lane >> 2) * 4u;
+    const void* base[G];
+    bool live[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        live[g] = g * 4 + wi < K;
+        base[g] = sp.g[live[g] ? g * 4 + wi : 0];
+    }
+    double acc[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) acc[p] = 0.0;
+    const uint64_t n_blocks = (sp.hi + 63) / 64;
     const uint64_t n_runs = (n_blocks + kGramRunBlocks - 1) / kGramRunBlocks;
+    const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWaves;
     for (uint64_t run = static_cast<uint64_t>(blockIdx.x) * kWaves + wave; run < n_runs; run += n_waves) {
-        float x[kGramRunBlocks][4];
+        typename L::Raw x[kGramRunBlocks][G];
 #pragma unroll
         for (int u = 0; u < kGramRunBlocks; ++u) {
-            const uint64_t e = (run * kGramRunBlocks + u) * block_elems + lane_off;
-            if (row_live && e >= sp.lo && e + 4 <= sp.hi) {
-                L::vec(base, e, x[u]);
-            } else {
+            const uint64_t e = (run * kGramRunBlocks + u) * 64 + lane_off;
+            const bool whole = e >= sp.lo && e + 4 <= sp.hi;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    x[u][i] = (row_live && e + i >= sp.lo && e + i < sp.hi) ? L::one(base, e + i) : 0.0f;
+            for (int g = 0; g < G; ++g) {
+                if (whole) {
+                    // a lane beyond the last worker reads worker 0's vector (the same line another lane of the
+                    // wave reads anyway) and drops it when it multiplies: the wave stays on one path and no
+                    // load waits for another
+                    x[u][g] = L::raw(base[g], e);
+                } else {                             // a vector across the span's first or last element
+                    float y[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        y[i] = (live[g] && e + i >= sp.lo && e + i < sp.hi) ? L::one(base[g], e + i) : 0.0f;
+                    x[u][g] = L::from(y);
+                }
             }
         }
 #pragma unroll
         for (int u = 0; u < kGramRunBlocks; ++u)
 #pragma unroll
-            for (int i = 0; i < 4; i += 2) {
-                const double d0 = static_cast<double>(x[u][i]), d1 = static_cast<double>(x[u][i + 1]);
-                acc = __builtin_amdgcn_mfma_f64_16x16x4f64(d0, d0, acc, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f64_16x16x4f64(d1, d1, acc1, 0, 0, 0);
+            for (int r = 0; r < 4; ++r) {
+                double d[G];
+#pragma unroll
+                for (int g = 0; g < G; ++g) d[g] = live[g] ? static_cast<double>(L::elem(x[u][g], r)) : 0.0;
+                int p = 0;
+#pragma unroll
+                for (int ga = 0; ga < G; ++ga)
+#pragma unroll
+                    for (int gb = ga; gb < G; ++gb, ++p)
+                        acc[p] = __builtin_amdgcn_mfma_f64_4x4x4f64(d[ga], d[gb], acc[p], 0, 0, 0);
             }
     }
-    acc += acc1;
-    // the four waves' tiles, added in wave order: entry t = v * 64 + lane of the tile is register v of lane
-    __shared__ double red[kWaves][256];
+    // The instruction's contraction index is lane / 16 and its four independent products are indexed by
+    // (lane / 4) % 4; entry (i, j) of product b sits in lane j + 4 b + 16 i. Which of a lane's elements meets
+    // which is therefore fixed by the lanes alone (A and B come from the same lane), and the four products
+    // are partial sums over different elements of the same 4 x 4 block. Row of the workgroup: entry
+    // [p][4 i + j] is the sum over the four products and the four waves (in that order) for pair p.
+    __shared__ double red[kWaves][P][64];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][v * 64 + lane] = acc[v];
+    for (int p = 0; p < P; ++p) red[wave][p][lane] = acc[p];
     __syncthreads();
-    const int t = threadIdx.x;
-    double s = red[0][t];
+    for (int t = threadIdx.x; t < P * 16; t += kBlock) {
+        const int p = t >> 4, i = (t >> 2) & 3, j = t & 3;
+        const int l0 = j + 16 * i;
+        double s = 0.0;
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) s += red[w][t];
-    partials[static_cast<uint64_t>(blockIdx.x) * JABAS_GRAM_STRIDE + t] = s;
+        for (int w = 0; w < kWaves; ++w) s += ((red[w][p][l0] + red[w][p][l0 + 4]) + red[w][p][l0 + 8]) + red[w][p][l0 + 12];
+        partials[static_cast<uint64_t>(blockIdx.x) * JABAS_GRAM_STRIDE + t] = s;
+    }
 }
 
-// Sums the workgroup tiles (1024 threads: thread (entry, part) adds rows part, part + 4, ... in order, the
-// four parts in order), then folds the diagonal blocks: gram[a][b] = sum over groups of
-// tile[group * Kp + a][group * Kp + b]. Register v of lane l holds tile[4 * v + l / 16][l % 16].
+// Sums the workgroup rows (1024 threads: thread (entry, part) adds rows part, part + 4, ... in order, then
+// the four parts in order) and unfolds the blocks: entry [p][4 i + j] of pair p = (ga, gb) is the product sum
+// of workers 4 ga + i and 4 gb + j.
 constexpr int kGramMfmaFinalizeBlock = 1024;
-__global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_kernel(int K, int log_kp, const double* partials,
-                                                                                    unsigned grid, double* gram_out) {
+__global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_kernel(int K, const double* partials, unsigned grid,
+                                                                                    double* gram_out) {
     __shared__ double part_sum[4][256];
     __shared__ double tile[256];
     const int t = threadIdx.x, e = t & 255, part = t >> 8;
+    const int G = (K + 3) / 4, P = G * (G + 1) / 2;
     double s = 0.0;
+    if (e < P * 16) {
 #pragma unroll 8
-    for (unsigned b = part; b < grid; b += 4) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + e];
+        for (unsigned b = part; b < grid; b += 4) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + e];
+    }
     part_sum[part][e] = s;
     __syncthreads();
     if (t < 256) tile[t] = ((part_sum[0][t] + part_sum[1][t]) + part_sum[2][t]) + part_sum[3][t];
@@ -223,11 +280,9 @@ __global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_ker
         double out = 0.0;
         if (a < K && b < K) {
             const int lo = a < b ? a : b, hi = a < b ? b : a;      // one triangle, mirrored: symmetric bit for bit
-            const int kp = 1 << log_kp;
-            for (int g = 0; g < (16 >> log_kp); ++g) {
-                const int i = g * kp + lo, j = g * kp + hi;
-                out += tile[(i >> 2) * 64 + (i & 3) * 16 + j];
-            }
+            const int ga = lo >> 2, gb = hi >> 2;
+            const int p = ga * G - ga * (ga - 1) / 2 + (gb - ga);  // index of pair (ga, gb), ga <= gb
+            out = tile[p * 16 + 4 * (lo & 3) + (hi & 3)];
         }
         gram_out[t] = out;
     }
@@ -240,38 +295,40 @@ int launch_gram_k(int grad_dtype, const SpanDev& sp, double* partials, unsigned 
     return static_cast<int>(launch_kernel(gram_kernel<K, JABAS_F32>, dim3(grid), dim3(kBlock), 0, stream, sp, partials));
 }
 
+template <int DT>
+int launch_gram_mfma(int K, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
+    switch ((K + 3) / 4) {
+        case 1: return static_cast<int>(launch_kernel(gram_mfma_kernel<DT, 1>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 2: return static_cast<int>(launch_kernel(gram_mfma_kernel<DT, 2>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 3: return static_cast<int>(launch_kernel(gram_mfma_kernel<DT, 3>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 4: return static_cast<int>(launch_kernel(gram_mfma_kernel<DT, 4>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        default: return -1;
+    }
+}
+
 }  // namespace
 
 int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
-    if (K > kGramValuMaxK) {
-        int log_kp = 0;
-        while ((1 << log_kp) < K) ++log_kp;
-        if (grad_dtype == JABAS_BF16)
-            return static_cast<int>(launch_kernel(gram_mfma_kernel<JABAS_BF16>, dim3(grid), dim3(kBlock), 0, stream, sp, K, log_kp, partials));
-        return static_cast<int>(launch_kernel(gram_mfma_kernel<JABAS_F32>, dim3(grid), dim3(kBlock), 0, stream, sp, K, log_kp, partials));
-    }
+    if (K > gram_valu_max_k(grad_dtype))
+        return grad_dtype == JABAS_BF16 ? launch_gram_mfma<JABAS_BF16>(K, sp, partials, grid, stream)
+                                        : launch_gram_mfma<JABAS_F32>(K, sp, partials, grid, stream);
     switch (K) {
         case 1: return launch_gram_k<1>(grad_dtype, sp, partials, grid, stream);
         case 2: return launch_gram_k<2>(grad_dtype, sp, partials, grid, stream);
         case 3: return launch_gram_k<3>(grad_dtype, sp, partials, grid, stream);
         case 4: return launch_gram_k<4>(grad_dtype, sp, partials, grid, stream);
-#if JABAS_GRAM_VALU_MAX_K > 4
         case 5: return launch_gram_k<5>(grad_dtype, sp, partials, grid, stream);
         case 6: return launch_gram_k<6>(grad_dtype, sp, partials, grid, stream);
         case 7: return launch_gram_k<7>(grad_dtype, sp, partials, grid, stream);
         case 8: return launch_gram_k<8>(grad_dtype, sp, partials, grid, stream);
-#endif
         default: return -1;
     }
 }
 
-int launch_gram_finalize(int K, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
-    if (K > kGramValuMaxK) {
-        int log_kp = 0;
-        while ((1 << log_kp) < K) ++log_kp;
-        return static_cast<int>(launch_kernel(gram_mfma_finalize_kernel, dim3(1), dim3(kGramMfmaFinalizeBlock), 0, stream, K, log_kp,
+int launch_gram_finalize(int K, int grad_dtype, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
+    if (K > gram_valu_max_k(grad_dtype))
+        return static_cast<int>(launch_kernel(gram_mfma_finalize_kernel, dim3(1), dim3(kGramMfmaFinalizeBlock), 0, stream, K,
                                               partials, grid, gram_out));
-    }
     return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(kGramFinalizeBlock), 0, stream, K, partials, grid, gram_out));
 }
 
