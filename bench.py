@@ -259,6 +259,22 @@ def statistics_launches(device, steps, torch):
     return out
 
 
+def gram_launches(device, steps, torch):
+    """The worker x worker Gram matrix ("between workers" statistics; both launches, Gram and finalize)
+    over 64 Mi elements: bytes read = K x element size per element."""
+    from jabas_amd import sync
+    n = 1 << 26
+    out = []
+    for gdt, name, sg in ((torch.float32, "f32", 4), (torch.bfloat16, "bf16", 2)):
+        grads = [(torch.randn(n, device=device) * 1e-3).to(gdt) for _ in range(16)]
+        for K in (4, 8, 12, 16):
+            ms, _ = timed_region(lambda i: sync.gram(grads[:K]), max(5, steps // 2), 3, torch)
+            out.append(dict(K=K, grad_dtype=name, elements=n, **rate(n * K * sg, ms)))
+        del grads
+        torch.cuda.empty_cache()
+    return out
+
+
 def launch_modes(cfg, device, steps, torch):
     """Small-span launch overhead (the Faster R-CNN configuration's point): the same step as
     one launch over bucket spans, one launch over one span per tensor, one launch per
@@ -386,6 +402,7 @@ def main():
                                                                       args.steps, torch)
     copy_gbps = copy_rate(device, args.steps, torch)
     stat_launches = None if args.no_all else statistics_launches(device, args.steps, torch)
+    gram = None if args.no_all else gram_launches(device, args.steps, torch)
     head = results[head_cfg.name]
     if not args.no_cpu:
         for cfg in order:
@@ -417,6 +434,7 @@ def main():
         "copy_GBps": copy_gbps,
         "workloads": list(results.values()),
         "statistics_launches": stat_launches,
+        "gram_launches": gram,
     }
     print(json.dumps(out))
 
