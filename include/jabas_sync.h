@@ -247,7 +247,10 @@ int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype,
                 void* workspace, size_t workspace_bytes, jabas_stream_t stream);
 
 /* K x K Gram matrix of the worker gradients, gram_out[a*JABAS_GRAM_MAX_K + b] = sum g_a*g_b
- * (fp64 products and sums), symmetric, JABAS_GRAM_STRIDE doubles. The "between
+ * symmetric, JABAS_GRAM_STRIDE doubles. fp32 gradients, and bf16 gradients of up to 7 workers:
+ * exact fp64 products and fp64 sums; bf16 gradients of 8 or more workers: exact fp32 products,
+ * fp32 running sums over at most 4096 elements, then fp64 (about 1e-6 of |g_a||g_b|). The order of
+ * operations is fixed: the same call gives the same bits. The "between
  * workers" statistics; no reference counterpart beyond the pairwise cosine of
  * jabas/train/trainer.py:478. K <= JABAS_GRAM_MAX_K. workspace: at least
  * 1024 * JABAS_GRAM_STRIDE doubles (one tile of partial sums per workgroup). */

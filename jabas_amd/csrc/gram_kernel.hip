@@ -1,10 +1,12 @@
 // K x K Gram matrix of the K worker gradients of one span: gram[a][b] = sum_e g_a[e]*g_b[e].
-// fp32 (or widened bf16) inputs, exact fp64 products, fp64 sums, fixed order: bit-identical run to run.
-//   few workers    grid-stride over 4-element vectors, K(K+1)/2 fp64 accumulators per thread on the vector
-//                  ALU, wave64 shuffle tree -> LDS -> one packed partial row per workgroup (K <= 5 for fp32
-//                  gradients, K <= 8 for bf16);
-//   more, to 16    fp64 matrix cores: v_mfma_f64_4x4x4 over 4 x 4 blocks of worker pairs, fed from registers
-//                  (gram_mfma_kernel below).
+// Fixed order of operations: bit-identical run to run.
+//   few workers    grid-stride over 4-element vectors, exact fp64 products of the fp32 (or widened bf16) values,
+//                  K(K+1)/2 fp64 accumulators per thread on the vector ALU, wave64 shuffle tree -> LDS -> one
+//                  packed partial row per workgroup (K <= 5 for fp32 gradients, K <= 7 for bf16);
+//   more, to 16    fp32 gradients: fp64 matrix cores, v_mfma_f64_4x4x4 over 4 x 4 blocks of worker pairs, fed
+//                  from registers (gram_mfma_kernel below), still exact products and fp64 sums;
+//                  bf16 gradients: bf16 matrix cores, exact fp32 products, fp32 running sums over short runs,
+//                  then fp64 (gram_bf16_mfma_kernel).
 // Then a single-workgroup finalize that sums the workgroup rows in a fixed order.
 #include "jabas_internal.h"
 
@@ -16,11 +18,11 @@ namespace jabas {
 namespace {
 
 #ifndef JABAS_GRAM_VALU_MAX_K_BF16
-#define JABAS_GRAM_VALU_MAX_K_BF16 8
+#define JABAS_GRAM_VALU_MAX_K_BF16 7
 #endif
 // Up to here the vector-ALU kernel, beyond it the matrix cores. Measured on 86.6 M elements: fp32 K = 5: 5.95
-// against 4.96 TB/s, K = 6: 5.54 against 5.94, K = 8: 5.45 against 6.01; bf16 gradients (half the bytes for the same
-// arithmetic) K = 8: 5.45 against 4.15.
+// against 4.96 TB/s, K = 6: 5.54 against 5.94, K = 8: 5.45 against 6.01; bf16 gradients K = 6: 5.83 against 5.81,
+// K = 8: 5.45 against 6.0.
 constexpr int gram_valu_max_k(int grad_dtype) { return grad_dtype == JABAS_BF16 ? JABAS_GRAM_VALU_MAX_K_BF16 : JABAS_GRAM_VALU_MAX_K; }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -288,6 +290,139 @@ __global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_ker
     }
 }
 
+// ---- bf16 gradients: bf16 matrix cores ------------------------------------------------------------------
+// v_mfma_f32_4x4x4_16b_bf16 multiplies, in each of its 16 independent products, a 4 x 4 operand by a 4 x 4
+// operand whose contraction index runs over the four bf16 values ONE lane supplies in a register pair. With the lane
+// layout above (lane l = worker l % 4 of its group, vector l / 4 of the block) the raw loaded registers ARE
+// the operands: no widening, no conversion, one instruction per pair of groups and four elements of every
+// lane. A lane loads 16 bytes (two operands) per group; a wave reads 256 contiguous bytes of each worker.
+// Products of bf16 values are exact in fp32; the instruction adds four of them to an fp32 running sum, which
+// is moved into fp64 sums (LDS, per wave) after at most kGramBf16FlushRuns runs, i.e. after at most
+// 4 * 2 * RUN * kGramBf16FlushRuns elements: fp32 rounding stays near 1e-6 of |g_a| |g_b|, the order is fixed.
+// Lanes beyond the last worker multiply worker 0's values into entries the finalize never reads.
+template <int CTRL> __device__ __forceinline__ float gram_dpp_f32(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 __attribute__((aligned(8))) u32x4_a8;     // element 0 of a bf16 buffer is 8-byte aligned, not more
+
+// 128-element blocks a wave loads before it multiplies, by number of groups
+#ifndef JABAS_GRAM_RUN_BF16_G1
+#define JABAS_GRAM_RUN_BF16_G1 2
+#endif
+#ifndef JABAS_GRAM_RUN_BF16_G2
+#define JABAS_GRAM_RUN_BF16_G2 2
+#endif
+#ifndef JABAS_GRAM_RUN_BF16_G3
+#define JABAS_GRAM_RUN_BF16_G3 2
+#endif
+#ifndef JABAS_GRAM_RUN_BF16_G4
+#define JABAS_GRAM_RUN_BF16_G4 4
+#endif
+constexpr int gram_bf16_run(int G) {
+    return G == 1 ? JABAS_GRAM_RUN_BF16_G1 : G == 2 ? JABAS_GRAM_RUN_BF16_G2 : G == 3 ? JABAS_GRAM_RUN_BF16_G3 : JABAS_GRAM_RUN_BF16_G4;
+}
+constexpr int kGramBf16FlushRuns = 128;
+
+template <int G>
+__global__ void __launch_bounds__(kBlock) gram_bf16_mfma_kernel(const SpanDev sp, int K, double* partials) {
+    constexpr int P = G * (G + 1) / 2;
+    constexpr int U = gram_bf16_run(G);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wi = lane & 3;
+    const uint32_t lane_off = static_cast<uint32_t>(lane >> 2) * 8u;
+    const uint16_t* base[G];
+    bool live[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        live[g] = g * 4 + wi < K;
+        base[g] = static_cast<const uint16_t*>(sp.g[live[g] ? g * 4 + wi : 0]);
+    }
+    // fp64 sums of the wave: [pair * 4 + i][16-lane row * 4 + j]
+    __shared__ double sums[kWaves][P * 4][16];
+    for (int i = lane; i < P * 64; i += 64) (&sums[wave][0][0])[i] = 0.0;
+    f32x4 acc[P];
+#pragma unroll
+    for (int p = 0; p < P; ++p) acc[p] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // entry (i, j) of a product sits in register i of lane j + 4 * product: a rotation by 4 and by 8 inside the
+    // 16-lane row adds the row's four products; lanes 0..3 of every row then own one fp64 sum each per register
+    const bool owner = ((lane >> 2) & 3) == 0;
+    const int col = (lane >> 4) * 4 + wi;
+    auto flush = [&]() {
+#pragma unroll
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = acc[p][i];
+                v += gram_dpp_f32<0x124>(v);        // row_ror:4
+                v += gram_dpp_f32<0x128>(v);        // row_ror:8
+                if (owner) sums[wave][p * 4 + i][col] += static_cast<double>(v);
+                acc[p][i] = 0.0f;
+            }
+    };
+    const uint64_t n_blocks = (sp.hi + 127) / 128;
+    const uint64_t n_runs = (n_blocks + U - 1) / U;
+    const uint64_t n_waves = static_cast<uint64_t>(gridDim.x) * kWaves;
+    int pending = 0;
+    for (uint64_t run = static_cast<uint64_t>(blockIdx.x) * kWaves + wave; run < n_runs; run += n_waves) {
+        u32x4 x[U][G];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint64_t e = (run * U + u) * 128 + lane_off;
+            const bool whole = e >= sp.lo && e + 8 <= sp.hi;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                if (whole) {
+                    x[u][g] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_a8*>(base[g] + e));
+                } else {                             // a vector across the span's first or last element
+                    uint32_t h[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) h[i] = (e + i >= sp.lo && e + i < sp.hi) ? base[g][e + i] : 0u;
+                    x[u][g] = u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                s16x4 d[G];
+#pragma unroll
+                for (int g = 0; g < G; ++g)
+                    d[g] = __builtin_bit_cast(s16x4, half ? u32x2{x[u][g].z, x[u][g].w} : u32x2{x[u][g].x, x[u][g].y});
+                int p = 0;
+#pragma unroll
+                for (int ga = 0; ga < G; ++ga)
+#pragma unroll
+                    for (int gb = ga; gb < G; ++gb, ++p)
+                        acc[p] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(d[ga], d[gb], acc[p], 0, 0, 0);
+            }
+        if (++pending == kGramBf16FlushRuns) { flush(); pending = 0; }
+    }
+    flush();
+    __syncthreads();
+    // row of the workgroup, the format of gram_mfma_kernel: entry [p][4 i + j], rows then waves in order
+    for (int t = threadIdx.x; t < P * 16; t += kBlock) {
+        const int p = t >> 4, i = (t >> 2) & 3, j = t & 3;
+        double s = 0.0;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w)
+            s += ((sums[w][p * 4 + i][j] + sums[w][p * 4 + i][4 + j]) + sums[w][p * 4 + i][8 + j]) + sums[w][p * 4 + i][12 + j];
+        partials[static_cast<uint64_t>(blockIdx.x) * JABAS_GRAM_STRIDE + t] = s;
+    }
+}
+
+int launch_gram_bf16_mfma(int K, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
+    switch ((K + 3) / 4) {
+        case 1: return static_cast<int>(launch_kernel(gram_bf16_mfma_kernel<1>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 2: return static_cast<int>(launch_kernel(gram_bf16_mfma_kernel<2>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 3: return static_cast<int>(launch_kernel(gram_bf16_mfma_kernel<3>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        case 4: return static_cast<int>(launch_kernel(gram_bf16_mfma_kernel<4>, dim3(grid), dim3(kBlock), 0, stream, sp, K, partials));
+        default: return -1;
+    }
+}
+
 template <int K>
 int launch_gram_k(int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
     if (grad_dtype == JABAS_BF16)
@@ -310,7 +445,7 @@ int launch_gram_mfma(int K, const SpanDev& sp, double* partials, unsigned grid, 
 
 int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream) {
     if (K > gram_valu_max_k(grad_dtype))
-        return grad_dtype == JABAS_BF16 ? launch_gram_mfma<JABAS_BF16>(K, sp, partials, grid, stream)
+        return grad_dtype == JABAS_BF16 ? launch_gram_bf16_mfma(K, sp, partials, grid, stream)
                                         : launch_gram_mfma<JABAS_F32>(K, sp, partials, grid, stream);
     switch (K) {
         case 1: return launch_gram_k<1>(grad_dtype, sp, partials, grid, stream);

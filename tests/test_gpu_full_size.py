@@ -224,3 +224,29 @@ def test_gnmt_embedding_rows_with_independent_masks(gpu):
     assert torch.allclose(row.cpu()[:4 + K], rows_h[0][:4 + K], rtol=1e-6, atol=0.0)
     for k in range(K):                                                      # per-worker norms: only that worker's rows count
         assert row[4 + k].item() == pytest.approx((hg[k].double() ** 2).sum().item(), rel=1e-10)
+
+
+@pytest.mark.parametrize("K", [8, 13])
+def test_gram_bf16_long_span(gpu, K):
+    """bf16 Gram over a span long enough (2^28 + 77 elements) that every wave moves its fp32 running sums
+    into the fp64 sums several times before the last one. The K workers point at three distinct buffers
+    (the kernel only reads), so every entry is one of six dot products, which a float64 library reduction gives."""
+    from jabas_amd import sync
+    n = (1 << 28) + 77
+    gen = torch.Generator(device=gpu).manual_seed(99)
+    bufs = [(torch.randn(n + 8, generator=gen, device=gpu) * 1e-2).to(torch.bfloat16) for _ in range(3)]
+    views = [b[s:s + n] for b, s in zip(bufs, (0, 4, 0))]
+    which = [(k * 7 + k // 3) % 3 for k in range(K)]
+    G = sync.gram([views[w] for w in which]).cpu()
+    dots = torch.zeros(3, 3, dtype=torch.float64)
+    for a in range(3):
+        for b in range(a, 3):
+            s = 0.0
+            for c in range(0, n, 1 << 26):                                  # chunks: bounded float64 temporaries
+                s += (views[a][c:c + (1 << 26)].double() * views[b][c:c + (1 << 26)].double()).sum().item()
+            dots[a, b] = dots[b, a] = s
+    for a in range(K):
+        for b in range(K):
+            scale = (dots[which[a], which[a]] * dots[which[b], which[b]]).sqrt().item()
+            assert abs(G[a, b].item() - dots[which[a], which[b]].item()) <= 5e-6 * scale, (a, b)
+    assert torch.equal(G, G.t())
