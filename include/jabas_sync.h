@@ -253,7 +253,9 @@ int jabas_stats(const void* const* grads, int32_t K, int32_t grad_dtype,
  * operations is fixed: the same call gives the same bits. The "between
  * workers" statistics; no reference counterpart beyond the pairwise cosine of
  * jabas/train/trainer.py:478. K <= JABAS_GRAM_MAX_K. workspace: at least
- * 1024 * JABAS_GRAM_STRIDE doubles (one tile of partial sums per workgroup). */
+ * 1024 * JABAS_GRAM_STRIDE doubles (one row of partial sums per workgroup); with 32 rows more
+ * (1056 * JABAS_GRAM_STRIDE doubles) the rows are summed in two stages, which is faster and, since the
+ * order of additions differs, may differ from the one-stage result in the last bits. */
 int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype,
                uint64_t numel, double* gram_out,
                void* workspace, size_t workspace_bytes, jabas_stream_t stream);

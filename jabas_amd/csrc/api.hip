@@ -13,7 +13,8 @@
 namespace jabas {
 
 int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsigned grid, hipStream_t stream);
-int launch_gram_finalize(int K, int grad_dtype, const double* partials, unsigned grid, double* gram_out, hipStream_t stream);
+int launch_gram_finalize(int K, int grad_dtype, double* partials, unsigned grid, unsigned spare_rows, double* gram_out,
+                         hipStream_t stream);
 
 namespace {
 
@@ -738,7 +739,9 @@ JABAS_API int jabas_gram(const void* const* grads, int32_t K, int32_t grad_dtype
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (launch_gram(K, grad_dtype, sd, static_cast<double*>(workspace), static_cast<unsigned>(g), st) != 0)
         return JABAS_ERR_LAUNCH;
-    if (launch_gram_finalize(K, grad_dtype, static_cast<const double*>(workspace), static_cast<unsigned>(g), gram_out, st) != 0)
+    const size_t spare = workspace_bytes / (JABAS_GRAM_STRIDE * sizeof(double)) - g;
+    if (launch_gram_finalize(K, grad_dtype, static_cast<double*>(workspace), static_cast<unsigned>(g),
+                             static_cast<unsigned>(spare > 0xffffffffu ? 0xffffffffu : spare), gram_out, st) != 0)
         return JABAS_ERR_LAUNCH;
     return JABAS_OK;
 }

@@ -290,6 +290,22 @@ __global__ void __launch_bounds__(kGramMfmaFinalizeBlock) gram_mfma_finalize_ker
     }
 }
 
+// One workgroup on one compute unit pulls 1024 rows of up to 160 doubles (1.3 MB) in 12-29 us, a tenth of the
+// bf16 K = 8 Gram launch itself. When the workspace has room for kGramFoldRows more rows, kGramFoldRows
+// workgroups first fold rows j, j + kGramFoldRows, ... (in that order) into row j of that room and the finalize
+// sums those. Which of the two forms runs depends on the sizes the caller passes only: same call, same bits.
+constexpr unsigned kGramFoldRows = 32;
+__global__ void __launch_bounds__(JABAS_GRAM_STRIDE) gram_mfma_fold_kernel(int K, const double* partials, unsigned grid, double* folded) {
+    const int G = (K + 3) / 4, E = G * (G + 1) / 2 * 16;
+    const int e = threadIdx.x;
+    double s = 0.0;
+    if (e < E) {
+#pragma unroll 8
+        for (unsigned b = blockIdx.x; b < grid; b += kGramFoldRows) s += partials[static_cast<uint64_t>(b) * JABAS_GRAM_STRIDE + e];
+    }
+    folded[static_cast<uint64_t>(blockIdx.x) * JABAS_GRAM_STRIDE + e] = s;
+}
+
 // ---- bf16 gradients: bf16 matrix cores ------------------------------------------------------------------
 // v_mfma_f32_4x4x4_16b_bf16 multiplies, in each of its 16 independent products, a 4 x 4 operand by a 4 x 4
 // operand whose contraction index runs over the four bf16 values ONE lane supplies in a register pair. With the lane
@@ -460,11 +476,25 @@ int launch_gram(int K, int grad_dtype, const SpanDev& sp, double* partials, unsi
     }
 }
 
-int launch_gram_finalize(int K, int grad_dtype, const double* partials, unsigned grid, double* gram_out, hipStream_t stream) {
-    if (K > gram_valu_max_k(grad_dtype))
+unsigned gram_fold_rows() { return kGramFoldRows; }
+
+// spare_rows: rows of JABAS_GRAM_STRIDE doubles the workspace holds beyond the `grid` partial rows
+int launch_gram_finalize(int K, int grad_dtype, double* partials, unsigned grid, unsigned spare_rows, double* gram_out,
+                         hipStream_t stream) {
+    if (K > gram_valu_max_k(grad_dtype)) {
+        if (grid > 4 * kGramFoldRows && spare_rows >= kGramFoldRows) {
+            double* folded = partials + static_cast<uint64_t>(grid) * JABAS_GRAM_STRIDE;
+            if (launch_kernel(gram_mfma_fold_kernel, dim3(kGramFoldRows), dim3(JABAS_GRAM_STRIDE), 0, stream, K,
+                              static_cast<const double*>(partials), grid, folded) != 0)
+                return -1;
+            return static_cast<int>(launch_kernel(gram_mfma_finalize_kernel, dim3(1), dim3(kGramMfmaFinalizeBlock), 0, stream, K,
+                                                  static_cast<const double*>(folded), kGramFoldRows, gram_out));
+        }
         return static_cast<int>(launch_kernel(gram_mfma_finalize_kernel, dim3(1), dim3(kGramMfmaFinalizeBlock), 0, stream, K,
-                                              partials, grid, gram_out));
-    return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(kGramFinalizeBlock), 0, stream, K, partials, grid, gram_out));
+                                              static_cast<const double*>(partials), grid, gram_out));
+    }
+    return static_cast<int>(launch_kernel(gram_finalize_kernel, dim3(1), dim3(kGramFinalizeBlock), 0, stream, K,
+                                          static_cast<const double*>(partials), grid, gram_out));
 }
 
 }  // namespace jabas

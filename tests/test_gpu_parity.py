@@ -207,6 +207,13 @@ def test_gram_limits_and_determinism(gpu):
     # the diagonal is the per-worker norm row of the statistics kernel's full level
     row = sync.gradient_stats(dg, BATCHES[11]).cpu()
     assert torch.allclose(torch.diagonal(a), row[4:4 + 11], rtol=1e-12, atol=0.0)
+    # a workspace without room for the two-stage sum of the partial rows: same values within rounding
+    small = torch.empty(1024 * L.GRAM_STRIDE, dtype=torch.float64, device=gpu)
+    b = sync.gram(dg, workspace=small).cpu()
+    assert torch.allclose(a, b, rtol=1e-13, atol=1e-24)
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.gram(dg, workspace=small[:1000 * L.GRAM_STRIDE])
+    assert e.value.status == L.ERR_WORKSPACE
     hb = _host_grads(13, 1_000_003, 78, dtype=torch.bfloat16)
     db = [_dev(t, gpu, 1) for t in hb]
     a = sync.gram(db).cpu().clone()
