@@ -429,8 +429,8 @@ class VSWSyncTrainer:
         if want:
             self._compute_cosine_similarity(rows)
         if self.grad_dtype == torch.float32:            # backward accumulates into the fp32 buckets; reduced-precision
-            for k in range(self.num_models):            # buckets are overwritten by the first compute() of the next step
-                self.engine.grads[k].zero_()
+            # buckets are overwritten by the first compute() of the next step. One multi-tensor launch for the K arenas.
+            torch._foreach_zero_(self.engine.grads[:self.num_models])
         for s in self.model_streams:
             s.wait_stream(cur)
         if want and self.controller is not None:
