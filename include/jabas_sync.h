@@ -16,7 +16,9 @@
  *     on the stream passed in (jabas_stream_t is a hipStream_t);
  *   - the library keeps no mutable global state (jabas_sync_bucket_static apart, which says
  *     so), so calls from different threads on different streams do not interfere as long
- *     as they use different workspaces;
+ *     as they use different workspaces; the jabas_rdv_* calls work on a host object the caller
+ *     creates (it and its HIP events are the only things the library ever allocates), under
+ *     that object's own mutex;
  *   - return value: JABAS_OK (0) or a negative JabasStatus; nothing is launched when a
  *     negative status is returned (except JABAS_ERR_LAUNCH, reported after the fact).
  *     JABAS_ERR_LAUNCH is the return value of this call's own hipLaunchKernel: a HIP
@@ -56,7 +58,9 @@ typedef enum JabasStatus {
     JABAS_ERR_PLAN = -8,        /* plan blob malformed or too small                    */
     JABAS_ERR_SIZE = -9,        /* numel / span count out of range                     */
     JABAS_ERR_LAUNCH = -10,     /* the HIP runtime refused the launch                  */
-    JABAS_ERR_ALIAS = -11       /* a written buffer overlaps another buffer of the span */
+    JABAS_ERR_ALIAS = -11,      /* a written buffer overlaps another buffer of the span */
+    JABAS_ERR_STATE = -12       /* rendezvous: a VSW handed the same bucket over twice in one step,
+                                   or a bucket was described again in the middle of a step */
 } JabasStatus;
 
 enum { JABAS_F32 = 0, JABAS_BF16 = 1 };
@@ -283,6 +287,54 @@ int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t num
 int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq,
                uint64_t numel, double lr, double weight_decay, double beta1, double beta2,
                double eps, int64_t step, int32_t adamw, jabas_stream_t stream);
+
+/* ---- Rendezvous of the K VSW comm hooks of one GPU --------------------------------------------
+ * In IIDP each VSW has its own DDP reducer, thread and stream, only VSW 0's hook communicates and
+ * the others register dummy_hook (jabas/train/trainer.py:452-468, 494-514); where the K hooks of a
+ * GPU meet is Python inside IIDP (absent from the JABAS repository), so these calls have no
+ * counterpart there: they are the native form of that meeting point for buckets that are handed over
+ * with the same buffers step after step. A hook's hand-over is one call (an event on its stream, a
+ * counter under the object's mutex); the call that completes a bucket queues, on launch_stream, a wait
+ * for every VSW's event and the jabas_sync_bucket launch described by jabas_rdv_set_bucket.
+ * Thread-safe per object. The caller orders the VSW streams behind the launches at the end of the
+ * step (one event on launch_stream) before any VSW hands a bucket over again. */
+typedef struct JabasRendezvous JabasRendezvous;
+
+enum {
+    JABAS_RDV_WAITING = 0,        /* handed over; other VSWs are still missing              */
+    JABAS_RDV_LAUNCHED = 1,       /* this call queued the launch, without statistics          */
+    JABAS_RDV_LAUNCHED_ROW0 = 2,  /* ... with statistics into row 0 of the bucket's two rows  */
+    JABAS_RDV_LAUNCHED_ROW1 = 3,  /* ... into row 1 (the rows alternate)                      */
+    JABAS_RDV_UNKNOWN = 4         /* the bucket is not described: nothing was recorded        */
+};
+
+/* K VSWs; the object belongs to the current device (its events are created there). */
+int jabas_rdv_create(int32_t K, JabasRendezvous** out);
+void jabas_rdv_destroy(JabasRendezvous* r);
+
+/* Describes the launch of bucket `bucket` (everything jabas_sync_bucket takes: the span with the K
+ * gradient buffers the VSWs will hand over, the device bound table or NULL); stats_rows: two rows of
+ * JABAS_STATS_STRIDE doubles and a workspace of jabas_sync_workspace_bytes, or NULL when the bucket
+ * never takes statistics. The struct is copied; the buffers stay the caller's and must outlive the
+ * description. Creates the bucket's K events on first use (the only allocation). */
+int jabas_rdv_set_bucket(JabasRendezvous* r, uint32_t bucket, const JabasSpan* span,
+                         const JabasBound* bounds_dev, double* stats_rows,
+                         void* workspace, size_t workspace_bytes);
+
+/* Forgets the description; returns how many VSWs had handed the bucket over in the running step. */
+int jabas_rdv_drop_bucket(JabasRendezvous* r, uint32_t bucket);
+
+/* VSW k hands bucket `bucket` over on vsw_stream. want_stats counts from VSW 0 only (its hook knows
+ * whether this is a statistics step); args: this step's arguments (args->stats is replaced by
+ * stats_level or JABAS_STATS_NONE accordingly). Returns a JABAS_RDV_* code or a negative JabasStatus
+ * (JABAS_ERR_STATE: handed over twice). */
+int jabas_rdv_publish(JabasRendezvous* r, int32_t k, uint32_t bucket, int32_t want_stats,
+                      jabas_stream_t vsw_stream, jabas_stream_t launch_stream,
+                      const JabasStepArgs* args, int32_t stats_level);
+
+/* End of a step or recovery from an error: clears what was handed over and returns the number of
+ * buckets that were incomplete (0 after a healthy step). */
+int jabas_rdv_reset(JabasRendezvous* r);
 
 #ifdef __cplusplus
 }

@@ -26,7 +26,8 @@ STAT_DOT_AB, STAT_NORM_A, STAT_NORM_B, STAT_NORM_AGG, STAT_NORM_VSW0 = 0, 1, 2, 
 
 OK = 0
 ERR_NULL, ERR_K, ERR_ALIGN, ERR_DTYPE, ERR_OPT, ERR_GROUP = -1, -2, -3, -4, -5, -6
-ERR_WORKSPACE, ERR_PLAN, ERR_SIZE, ERR_LAUNCH, ERR_ALIAS = -7, -8, -9, -10, -11
+ERR_WORKSPACE, ERR_PLAN, ERR_SIZE, ERR_LAUNCH, ERR_ALIAS, ERR_STATE = -7, -8, -9, -10, -11, -12
+RDV_WAITING, RDV_LAUNCHED, RDV_LAUNCHED_ROW0, RDV_LAUNCHED_ROW1, RDV_UNKNOWN = 0, 1, 2, 3, 4
 
 
 class JabasSpan(C.Structure):
@@ -104,6 +105,14 @@ SIGNATURES = {
     "jabas_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double,
                              C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64, C.c_int32,
                              C.c_void_p]),
+    "jabas_rdv_create": (C.c_int, [C.c_int32, C.POINTER(C.c_void_p)]),
+    "jabas_rdv_destroy": (None, [C.c_void_p]),
+    "jabas_rdv_set_bucket": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(JabasSpan), C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.c_size_t]),
+    "jabas_rdv_drop_bucket": (C.c_int, [C.c_void_p, C.c_uint32]),
+    "jabas_rdv_publish": (C.c_int, [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_void_p, C.c_void_p,
+                                    C.POINTER(JabasStepArgs), C.c_int32]),
+    "jabas_rdv_reset": (C.c_int, [C.c_void_p]),
 }
 
 _lib = None

@@ -400,6 +400,7 @@ JABAS_API const char* jabas_status_string(int status) {
         case JABAS_ERR_SIZE: return "element, span or fan-out count out of range (jabas_sync_bucket_static: more than JABAS_STATIC_MAX_NUMEL elements)";
         case JABAS_ERR_LAUNCH: return "HIP runtime refused the kernel launch";
         case JABAS_ERR_ALIAS: return "a written buffer overlaps another buffer of the span (only agg_out == grads[k], fp32, may alias)";
+        case JABAS_ERR_STATE: return "rendezvous: bucket handed over twice by one VSW in a step, or described again in the middle of a step";
         default: return "unknown status";
     }
 }

@@ -20,6 +20,7 @@ of its own) is this class with an optimizer bound (``bind_optimizer``) and a lau
 flat arenas exactly like the bucket, so aggregate, update and the copy of the new weights
 to the other replicas are one launch per bucket.
 """
+import ctypes as C
 import threading
 
 import torch
@@ -134,6 +135,15 @@ class LocalBucketSync:
         self._bound_steps = {}                 # id -> optimizer.state dictionary whose 'step' follows step_count
         self.launched = 0                      # fused launches queued so far
         self.launched_with_opt = 0             # of them, launches that updated weights
+        # Native meeting point (jabas_rdv_*): buckets that come with the same buffers step after step are
+        # described to it after their first launch here; from then on a hook's hand-over is one foreign call.
+        self._native_ok = launcher is None and not self.deferred and not self.batch_bytes
+        self._rdv = None
+        self._native = {}                      # bucket index -> (buffer addresses per VSW, elements, prepared call, dtype)
+        self._native_on_done = {}
+        self._native_args = {}
+        self._main_ptr = None
+        self.native_publishes = 0              # hand-overs that took the native path
         if optimizer is not None:
             self.bind_optimizer(optimizer)
 
@@ -255,6 +265,7 @@ class LocalBucketSync:
         with self._lock:
             self._calls.pop(bucket_index, None)
             self._plans.clear()
+        self._forget_native(bucket_index)
         return new
 
     def aggregate_of(self, bucket_index):
@@ -272,6 +283,12 @@ class LocalBucketSync:
             raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
         fut = torch.futures.Future()
         fut.set_result(tensor if value is None else value)
+        known = self._native.get(bucket_index)
+        if known is not None and tensor.is_cuda:
+            if known[0][k] == tensor.data_ptr() and known[1] == tensor.numel():
+                self._publish_native(k, bucket_index, tensor, want_stats, on_done, known)
+                return fut
+            self._forget_native(bucket_index, k)
         event = stream = None
         if tensor.is_cuda:
             stream = self._current_stream(tensor)
@@ -297,6 +314,7 @@ class LocalBucketSync:
             if k == 0:
                 slot.want_stats, slot.on_done = want_stats, on_done
                 self._main_stream = stream
+                self._main_ptr = None if stream is None else stream.cuda_stream
             ready = slot.count == self.K
             if ready:
                 del self._slots[bucket_index]
@@ -315,11 +333,73 @@ class LocalBucketSync:
     def _current_stream(self, tensor):
         """torch.cuda.current_stream(tensor.device) without its per-call device bookkeeping (4.6 us a call,
         as much as the rest of a publish): the Stream object of a raw stream is made once and kept."""
+        return self._current_stream_and_ptr(tensor)[0]
+
+    def _current_stream_and_ptr(self, tensor):
         raw = torch._C._cuda_getCurrentStream(tensor.get_device())
-        stream = self._stream_cache.get(raw)
-        if stream is None:
-            stream = self._stream_cache[raw] = torch.cuda.Stream(stream_id=raw[0], device_index=raw[1], device_type=raw[2])
-        return stream
+        hit = self._stream_cache.get(raw)
+        if hit is None:
+            stream = torch.cuda.Stream(stream_id=raw[0], device_index=raw[1], device_type=raw[2])
+            hit = self._stream_cache[raw] = (stream, stream.cuda_stream)
+        return hit
+
+    # ------------------------------------------------------------------ native meeting point
+    def _describe_native(self, bucket_index, tensors, call):
+        """Describes a bucket that has just had its first launch from here to the native rendezvous."""
+        dev = tensors[0].device
+        lib = L.lib()
+        with torch.cuda.device(dev), torch.cuda.stream(self._launch_stream()):
+            if self._rdv is None:
+                handle = C.c_void_p()
+                L.check(lib.jabas_rdv_create(self.K, C.byref(handle)), "jabas_rdv_create")
+                self._rdv = handle
+                self._rdv_publish = lib.jabas_rdv_publish
+            call.prepare_stats()
+            L.check(lib.jabas_rdv_set_bucket(self._rdv, bucket_index, C.byref(call.c_span),
+                                             None if call.bounds_dev is None else call.bounds_dev.data_ptr(),
+                                             call._rows.data_ptr(), call.ws.buf.data_ptr(), call.ws.nbytes),
+                    "jabas_rdv_set_bucket")
+        self._native[bucket_index] = (tuple(t.data_ptr() for t in tensors), tensors[0].numel(), call, tensors[0].dtype)
+
+    def _forget_native(self, bucket_index, k=None):
+        known = self._native.pop(bucket_index, None)
+        if known is None or self._rdv is None:
+            return
+        arrived = L.lib().jabas_rdv_drop_bucket(self._rdv, bucket_index)
+        if arrived > 0 and k is not None:
+            raise RuntimeError(f"bucket {bucket_index}: VSW {k} handed over another buffer than in the step before, "
+                               f"after {arrived} other VSW(s) had handed over the same ones as before")
+
+    def _publish_native(self, k, bucket_index, tensor, want_stats, on_done, known):
+        stream, ptr = self._current_stream_and_ptr(tensor)
+        self._vsw_streams[k] = stream
+        if k == 0:
+            self._main_stream, self._main_ptr = stream, ptr
+            self._native_on_done[bucket_index] = on_done
+        main_ptr = self._sync_stream.cuda_stream if self._sync_stream is not None else self._main_ptr
+        call = known[2]
+        stamp = (self.step_count, self.lr_scale, self.accumulations)
+        ent = self._native_args.get((known[3], call.with_opt))
+        if ent is None or ent[0] != stamp:
+            args = self._step_args(known[3], False, call.with_opt)
+            ent = self._native_args[(known[3], call.with_opt)] = (stamp, args, C.byref(args))
+        rc = self._rdv_publish(self._rdv, k, bucket_index, 1 if want_stats else 0, ptr, main_ptr, ent[2], self.stats_level)
+        self.native_publishes += 1
+        if rc == L.RDV_WAITING:
+            return
+        if rc < 0 or rc == L.RDV_UNKNOWN:
+            with self._lock:
+                self._errors.append((bucket_index, L.JabasSyncError(rc if rc < 0 else L.ERR_STATE, "jabas_rdv_publish")))
+            return
+        row = call._rows[rc - L.RDV_LAUNCHED_ROW0] if rc >= L.RDV_LAUNCHED_ROW0 else None
+        with self._lock:
+            self._launch_streams.add(self._launch_stream())
+            self.launched += 1
+            if call.with_opt:
+                self.launched_with_opt += 1
+        done = self._native_on_done.get(bucket_index)
+        if done is not None:
+            done(BucketStats(bucket_index, row) if row is not None else None)
 
     def _launch_stream(self):
         return self._sync_stream if self._sync_stream is not None else self._main_stream
@@ -396,6 +476,8 @@ class LocalBucketSync:
             call.with_opt, call.clipped = with_opt, clipped
             with self._lock:
                 self._calls[bucket_index] = call
+            if self._native_ok and not clipped and main is not None:
+                self._describe_native(bucket_index, tensors, call)
         if call.with_opt:
             with self._lock:
                 self.launched_with_opt += 1
@@ -510,6 +592,19 @@ class LocalBucketSync:
             self._launch_streams = set()
             self._vsw_streams = {}
             self._errors = []
+        self._reset_native()
+
+    def _reset_native(self):
+        """Clears the native meeting point; returns how many of its buckets were incomplete."""
+        return 0 if self._rdv is None else max(0, L.lib().jabas_rdv_reset(self._rdv))
+
+    def __del__(self):
+        rdv, self._rdv = getattr(self, "_rdv", None), None
+        if rdv is not None:
+            try:
+                L.lib().jabas_rdv_destroy(rdv)
+            except Exception:                          # interpreter shutdown
+                pass
 
     def finish_step(self, streams=()):
         """End of a sync step: every VSW stream waits for the fused launches that read its
@@ -517,9 +612,11 @@ class LocalBucketSync:
         first-step flag) advances. ``streams``: the VSW streams; default: the streams the hooks of this
         step ran on."""
         left = self.pending()
-        if left:
+        left_native = self._reset_native()
+        if left or left_native:
             self.reset()
-            raise RuntimeError(f"buckets {left} were not published by every VSW")
+            raise RuntimeError(f"buckets {left} were not published by every VSW" +
+                               (f" ({left_native} more at the native meeting point)" if left_native else ""))
         with self._lock:
             ready, self._ready, self._ready_bytes = self._ready, {}, 0
         if ready:

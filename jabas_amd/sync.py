@@ -332,6 +332,14 @@ class BucketCall:
     def matches(self, grads):
         return self.key == self.key_of(grads)
 
+    def prepare_stats(self):
+        """The statistics workspace and the two rows the launches alternate between (made once)."""
+        if self.ws is None:
+            g0 = self.span.grads[0]
+            self.ws = Workspace.for_span(g0.numel(), g0.dtype, g0.device)
+            self._rows = torch.zeros(2, L.STATS_STRIDE, dtype=torch.float64, device=g0.device)
+            self._flip = 0
+
     def run(self, args, stream=None):
         """Queues the step; returns the statistics row or None. Rows alternate between two device
         buffers, so a returned row stays untouched by this call's next statistics launch and is
@@ -339,11 +347,7 @@ class BucketCall:
         stats_ptr = ws_ptr = row = None
         ws_bytes = 0
         if args.stats:
-            if self.ws is None:
-                g0 = self.span.grads[0]
-                self.ws = Workspace.for_span(g0.numel(), g0.dtype, g0.device)
-                self._rows = torch.zeros(2, L.STATS_STRIDE, dtype=torch.float64, device=g0.device)
-                self._flip = 0
+            self.prepare_stats()
             self._flip ^= 1
             row = self._rows[self._flip]
             stats_ptr, ws_ptr, ws_bytes = row.data_ptr(), self.ws.buf.data_ptr(), self.ws.nbytes

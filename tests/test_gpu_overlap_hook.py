@@ -177,6 +177,9 @@ def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, mode
         assert 3 * 1 <= local.launched <= 3 * len(SHAPES)
     else:
         assert local.launched == 3 * (1 if mode == "deferred" else len(SHAPES))
+    # one launch per bucket: the first step describes the buckets to the native meeting point, the hand-overs of
+    # the second (a statistics step) and third go through it
+    assert local.native_publishes == (2 * K * len(SHAPES) if mode == "per_bucket" else 0)
 
 
 @pytest.mark.parametrize("kind", ["sgd", "adam"])
@@ -216,6 +219,72 @@ def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
         assert _same(bufs[0], agg_h) and _same(p_d, p_h) and _same(s1_d, s1_h) and _same(fan, p_h), step
         if kind != "sgd":
             assert _same(s2_d, s2_h), step
+    assert local.native_publishes == 2 * K * len(sizes) and local.launched == 3 * len(sizes)
+
+
+def test_native_meeting_point_errors_and_new_buffers(gpu):
+    """Hand-overs of buckets the native meeting point knows: a VSW that never comes, one that comes twice, and
+    buffers that change between steps (DDP's bucket rebuild). Every healthy step is bit-exact with the oracle."""
+    from jabas_amd.local_sync import LocalBucketSync
+    K, batches, sizes = 3, (4, 2, 2), [50001, 4099]
+    local = LocalBucketSync(batches)
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+
+    def fresh():
+        return [[torch.zeros(n, device=gpu) for _ in range(K)] for n in sizes]
+
+    def step(bufs, seed, skip=None, twice=None):
+        host = [[torch.randn(n, generator=torch.Generator().manual_seed(seed + 10 * b + k)) * 1e-3 for k in range(K)]
+                for b, n in enumerate(sizes)]
+        for b in range(len(sizes)):
+            for k in (1, 0, 2):                                                  # VSW 0 in the middle
+                if (b, k) == skip:
+                    continue
+                with torch.cuda.stream(streams[k]):
+                    bufs[b][k].copy_(host[b][k].to(gpu, non_blocking=False))
+                    local.publish(k, b, bufs[b][k])
+                    if (b, k) == twice:
+                        local.publish(k, b, bufs[b][k])
+        return host
+
+    def check(bufs, host):
+        torch.cuda.synchronize()
+        for b, n in enumerate(sizes):
+            agg_h, _ = O.sync_step(host[b], batches, [(0, n, ((0, 0),))], None, None, None, None, step=1, first_step=True)
+            assert _same(bufs[b][0], agg_h), b
+
+    bufs = fresh()
+    host = step(bufs, 100)                       # described here
+    local.finish_step()
+    check(bufs, host)
+    assert local.native_publishes == 0
+    host = step(bufs, 200)                       # native
+    local.finish_step()
+    check(bufs, host)
+    assert local.native_publishes == K * len(sizes)
+    step(bufs, 300, skip=(1, 2))                 # VSW 2 never hands bucket 1 over
+    with pytest.raises(RuntimeError, match="not published by every VSW"):
+        local.finish_step()
+    host = step(bufs, 400)                       # the next step starts clean
+    local.finish_step()
+    check(bufs, host)
+    step(bufs, 500, twice=(0, 1))                # bucket 0 from VSW 1 twice: reported at the end of the step
+    with pytest.raises(RuntimeError):
+        local.finish_step()
+    local.reset()
+    host = step(bufs, 600)
+    local.finish_step()
+    check(bufs, host)
+    before = local.native_publishes
+    other = fresh()                              # other buffers: described again, native again the step after
+    host = step(other, 700)
+    local.finish_step()
+    check(other, host)
+    assert local.native_publishes == before
+    host = step(other, 800)
+    local.finish_step()
+    check(other, host)
+    assert local.native_publishes == before + K * len(sizes)
 
 
 def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
