@@ -464,3 +464,20 @@ def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
     assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == want_chunks[1]
     assert lib.jabas_plan_chunks(blob.ctypes.data, 2) == want_chunks[2]
     assert lib.jabas_plan_chunks(blob.ctypes.data, 3) == L.ERR_OPT
+
+
+def test_rendezvous_calls_validate_their_arguments():
+    """The meeting point's argument checks (no GPU: creating the object itself needs a device and is covered by
+    the GPU tests)."""
+    lib = L.lib()
+    h = C.c_void_p()
+    assert lib.jabas_rdv_create(0, C.byref(h)) == L.ERR_K and not h.value
+    assert lib.jabas_rdv_create(L.MAX_K + 1, C.byref(h)) == L.ERR_K
+    assert lib.jabas_rdv_create(2, None) == L.ERR_NULL
+    args, span = L.JabasStepArgs(), L.JabasSpan()
+    assert lib.jabas_rdv_publish(None, 0, 0, 0, None, None, C.byref(args), L.STATS_SIMILARITY) == L.ERR_NULL
+    assert lib.jabas_rdv_set_bucket(None, 0, C.byref(span), None, None, None, 0) == L.ERR_NULL
+    assert lib.jabas_rdv_drop_bucket(None, 0) == L.ERR_NULL
+    assert lib.jabas_rdv_reset(None) == L.ERR_NULL
+    lib.jabas_rdv_destroy(None)
+    assert b"rendezvous" in lib.jabas_status_string(L.ERR_STATE)
