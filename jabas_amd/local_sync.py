@@ -143,7 +143,7 @@ class LocalBucketSync:
         self._native_on_done = {}
         self._native_args = {}
         self._main_ptr = None
-        self.native_publishes = 0              # hand-overs that took the native path
+        self.native_launches = 0               # launches queued by the native meeting point
         if optimizer is not None:
             self.bind_optimizer(optimizer)
 
@@ -384,7 +384,6 @@ class LocalBucketSync:
             args = self._step_args(known[3], False, call.with_opt)
             ent = self._native_args[(known[3], call.with_opt)] = (stamp, args, C.byref(args))
         rc = self._rdv_publish(self._rdv, k, bucket_index, 1 if want_stats else 0, ptr, main_ptr, ent[2], self.stats_level)
-        self.native_publishes += 1
         if rc == L.RDV_WAITING:
             return
         if rc < 0 or rc == L.RDV_UNKNOWN:
@@ -395,6 +394,7 @@ class LocalBucketSync:
         with self._lock:
             self._launch_streams.add(self._launch_stream())
             self.launched += 1
+            self.native_launches += 1
             if call.with_opt:
                 self.launched_with_opt += 1
         done = self._native_on_done.get(bucket_index)

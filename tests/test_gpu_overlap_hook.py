@@ -179,7 +179,7 @@ def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, mode
         assert local.launched == 3 * (1 if mode == "deferred" else len(SHAPES))
     # one launch per bucket: the first step describes the buckets to the native meeting point, the hand-overs of
     # the second (a statistics step) and third go through it
-    assert local.native_publishes == (2 * K * len(SHAPES) if mode == "per_bucket" else 0)
+    assert local.native_launches == (2 * len(SHAPES) if mode == "per_bucket" else 0)
 
 
 @pytest.mark.parametrize("kind", ["sgd", "adam"])
@@ -219,7 +219,7 @@ def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
         assert _same(bufs[0], agg_h) and _same(p_d, p_h) and _same(s1_d, s1_h) and _same(fan, p_h), step
         if kind != "sgd":
             assert _same(s2_d, s2_h), step
-    assert local.native_publishes == 2 * K * len(sizes) and local.launched == 3 * len(sizes)
+    assert local.native_launches == 2 * len(sizes) and local.launched == 3 * len(sizes)
 
 
 def test_native_meeting_point_errors_and_new_buffers(gpu):
@@ -257,11 +257,11 @@ def test_native_meeting_point_errors_and_new_buffers(gpu):
     host = step(bufs, 100)                       # described here
     local.finish_step()
     check(bufs, host)
-    assert local.native_publishes == 0
+    assert local.native_launches == 0
     host = step(bufs, 200)                       # native
     local.finish_step()
     check(bufs, host)
-    assert local.native_publishes == K * len(sizes)
+    assert local.native_launches == len(sizes)
     step(bufs, 300, skip=(1, 2))                 # VSW 2 never hands bucket 1 over
     with pytest.raises(RuntimeError, match="not published by every VSW"):
         local.finish_step()
@@ -275,16 +275,16 @@ def test_native_meeting_point_errors_and_new_buffers(gpu):
     host = step(bufs, 600)
     local.finish_step()
     check(bufs, host)
-    before = local.native_publishes
+    before = local.native_launches
     other = fresh()                              # other buffers: described again, native again the step after
     host = step(other, 700)
     local.finish_step()
     check(other, host)
-    assert local.native_publishes == before
+    assert local.native_launches == before
     host = step(other, 800)
     local.finish_step()
     check(other, host)
-    assert local.native_publishes == before + K * len(sizes)
+    assert local.native_launches == before + len(sizes)
 
 
 def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
