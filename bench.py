@@ -196,6 +196,13 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         ms, _ = timed_region(lambda i: engines[i % n].step(stats="full"), steps, warmup, torch)
         res["step_with_per_vsw_norms"] = rate(bytes_per_step, ms)
     if extras:
+        # the same step recorded once in a HIP graph and replayed with the scalars of the moment in a device
+        # block (Adam's bias correction moves every step): one graph launch per step instead of the step's launches
+        graphed = [e.capture(stats=level) for e in engines]
+        ms, wall = timed_region(lambda i: graphed[i % n].replay(), steps, warmup, torch)
+        res["recorded_step"] = dict(rate(bytes_per_step, ms), wall_ms_per_step=wall)
+        del graphed
+    if extras:
         hsteps, hwarm = max(5, steps // 2), max(10, warmup)
         res["hook_path_per_bucket_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False)
         res["hook_path_batched_64MiB_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False, 64 << 20)
@@ -205,6 +212,9 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         # coefficient on the device, then the update over the scaled aggregate
         ms, _ = timed_region(lambda i: engines[i % n].step(stats=level, clip_norm=5.0), steps, warmup, torch)
         res["clipped_step_ms"] = ms
+        graphed = [e.capture(stats=level, clip_norm=5.0) for e in engines]
+        res["clipped_recorded_step_ms"] = timed_region(lambda i: graphed[i % n].replay(), steps, warmup, torch)[0]
+        del graphed
     stats_rows = engines[0].step(stats=level) if cfg.stats else None
     res["cosine"] = engines[0].cosine(stats_rows) if stats_rows is not None else None
     res["finite"] = bool(torch.isfinite(engines[0].param).all())

@@ -43,6 +43,7 @@ extern "C" {
 #define JABAS_GRAM_MAX_K 16     /* VSWs of one jabas_gram call                        */
 #define JABAS_GRAM_STRIDE 256   /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
 #define JABAS_STATIC_MAX_NUMEL (1ull << 26)  /* largest span of jabas_sync_bucket_static  */
+#define JABAS_STEP_SCALARS_BYTES 688         /* size of a step-scalar block (jabas_step_scalars_encode) */
 
 typedef void* jabas_stream_t;   /* hipStream_t */
 
@@ -146,11 +147,40 @@ typedef struct JabasStepArgs {
     const float* grad_scale;            /* device scalar c or NULL: when c < 1 the aggregate
                                            is multiplied by c (one fp32 product) before it is
                                            written and handed to the optimizer (clipping)  */
+    const void* scalars_dev;            /* NULL, or a device block of JABAS_STEP_SCALARS_BYTES bytes,
+                                           16-byte aligned, written by jabas_step_scalars_encode: the
+                                           launch then reads weight, half_id, half_weight, first_step,
+                                           nesterov, momentum, dampening, beta1, beta2, eps and the
+                                           groups' lr, weight_decay and step from the block as it is
+                                           when the kernel runs, not from this struct (which must
+                                           still be filled in: it is what the call is checked
+                                           against). Optimizer kinds other than NONE only.      */
 } JabasStepArgs;
 
 /* Library identification. No reference counterpart. */
 const char* jabas_sync_version(void);
 const char* jabas_status_string(int status);
+
+/* The per-step scalars of `args` as the kernels read them (fp32 constants derived in double and
+ * rounded once, exactly as a call without a block derives them), written to host_block
+ * (JABAS_STEP_SCALARS_BYTES bytes). Pure host code. The caller moves the bytes to the device block
+ * that JabasStepArgs.scalars_dev names, in stream order before the launch that reads them. What it
+ * is for: a step recorded in a HIP graph has every by-value argument baked in, so an Adam step
+ * (bias correction moves with the step count), an SGD step under a learning-rate schedule or under
+ * the adaptive-batching LR modifier (jabas/train/trainer.py:693-700) could not be replayed; with
+ * the scalars in a device block the recorded launch stays valid and only the block is refreshed
+ * (a copy from pinned host memory recorded in the same graph, or a copy queued before the replay).
+ * K, grad_dtype, stats, opt_kind and n_groups of the recorded call stay what they were; a block
+ * encoded from arguments with another K or optimizer kind is the caller's error, unchecked. The
+ * Adam / AdamW flag is part of the block. No reference counterpart. */
+int jabas_step_scalars_encode(const JabasStepArgs* args, void* host_block, size_t block_bytes);
+
+/* Encodes `args` and queues, on `stream`, a one-wave kernel that writes the bytes to the device block
+ * scalars_dev (JABAS_STEP_SCALARS_BYTES bytes, 16-byte aligned): the refresh ahead of a replay, in stream
+ * order with the launches that read the block, without pinned host memory and without a copy engine in
+ * between. Only a kernel launch: may itself be recorded (its bytes are then baked in, which is what a
+ * recording wants for launches whose scalars never move). No reference counterpart. */
+int jabas_step_scalars_upload(const JabasStepArgs* args, void* scalars_dev, jabas_stream_t stream);
 
 /* Bytes of device workspace a single-span call (jabas_sync_bucket, jabas_stats) over
  * numel elements needs when statistics are requested: one partial row per workgroup of

@@ -17,6 +17,7 @@ STATS_STRIDE = 20
 GRAM_MAX_K = 16
 GRAM_STRIDE = 256
 STATIC_MAX_NUMEL = 1 << 26
+STEP_SCALARS_BYTES = 688
 
 F32, BF16 = 0, 1
 OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW = 0, 1, 2, 3
@@ -73,6 +74,7 @@ class JabasStepArgs(C.Structure):
         ("eps", C.c_double),
         ("groups", JabasGroup * MAX_GROUPS),
         ("grad_scale", C.c_void_p),
+        ("scalars_dev", C.c_void_p),
     ]
 
 
@@ -80,6 +82,8 @@ class JabasStepArgs(C.Structure):
 SIGNATURES = {
     "jabas_sync_version": (C.c_char_p, []),
     "jabas_status_string": (C.c_char_p, [C.c_int]),
+    "jabas_step_scalars_encode": (C.c_int, [C.POINTER(JabasStepArgs), C.c_void_p, C.c_size_t]),
+    "jabas_step_scalars_upload": (C.c_int, [C.POINTER(JabasStepArgs), C.c_void_p, C.c_void_p]),
     "jabas_sync_workspace_bytes": (C.c_size_t, [C.c_uint64, C.c_int32]),
     "jabas_plan_bytes": (C.c_size_t, [C.POINTER(JabasSpan), C.c_uint32, C.c_uint32, C.c_int32]),
     "jabas_plan_encode": (C.c_int, [C.POINTER(JabasSpan), C.c_uint32, C.POINTER(JabasBound), C.c_uint32,

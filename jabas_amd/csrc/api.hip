@@ -192,8 +192,8 @@ int check_bounds_host(const JabasSpan& sp, const JabasBound* bounds, uint32_t n_
     return JABAS_OK;
 }
 
-// StepArgs (doubles, as the Python optimizer holds them) -> fp32 kernel constants.
-int fill_kargs(const JabasStepArgs* s, KArgs* a) {
+// StepArgs (doubles, as the Python optimizer holds them) -> the fp32 scalars the kernels read.
+int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
     if (!s) return JABAS_ERR_NULL;
     if (s->K < 1 || s->K > JABAS_MAX_K) return JABAS_ERR_K;
     if (s->grad_dtype != JABAS_F32 && s->grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
@@ -209,7 +209,6 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
         if (s->half_id[k]) mask |= 1u << k;
     }
     a->half_mask = mask;
-    a->grad_scale = s->grad_scale;
     if (oc == 0) return JABAS_OK;
     if (s->n_groups < 1 || s->n_groups > JABAS_MAX_GROUPS) return JABAS_ERR_GROUP;
     OptDev& o = a->opt;
@@ -244,7 +243,28 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
     return JABAS_OK;
 }
 
-typedef int (*LaunchFn)(int, int, int, const KArgs&, unsigned, hipStream_t);
+// The launch arguments' share of a step: the scalars by value, and the device block when the caller names one
+// (the by-value copy is then what the call was checked against, the kernel reads the block).
+int fill_kargs(const JabasStepArgs* s, KArgs* a) {
+    StepScal sc;
+    const int rc = fill_step_scal(s, &sc);
+    if (rc != JABAS_OK) return rc;
+    memset(a, 0, sizeof(*a));
+    memcpy(a->w, sc.w, sizeof(sc.w));
+    memcpy(a->wh, sc.wh, sizeof(sc.wh));
+    a->half_mask = sc.half_mask;
+    a->opt = sc.opt;
+    memcpy(a->groups, sc.groups, sizeof(sc.groups));
+    a->grad_scale = s->grad_scale;
+    if (s->scalars_dev) {
+        if (opt_class_of(s->opt_kind) == 0) return JABAS_ERR_OPT;      // nothing of an aggregate-only launch moves between steps
+        if (reinterpret_cast<uintptr_t>(s->scalars_dev) % 16) return JABAS_ERR_ALIGN;
+        a->dyn = static_cast<const StepScal*>(s->scalars_dev);
+    }
+    return JABAS_OK;
+}
+
+typedef int (*LaunchFn)(int, int, int, int, const KArgs&, unsigned, hipStream_t);
 const LaunchFn kLaunch[JABAS_MAX_K] = {launch_fused_k1,  launch_fused_k2,  launch_fused_k3,  launch_fused_k4,
                                        launch_fused_k5,  launch_fused_k6,  launch_fused_k7,  launch_fused_k8,
                                        launch_fused_k9,  launch_fused_k10, launch_fused_k11, launch_fused_k12,
@@ -359,7 +379,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
     }
     a.partials = static_cast<double*>(workspace);
     if (a.n_chunks) {
-        const int err = kLaunch[s->K - 1](s->grad_dtype, oc, stats, a, a.n_chunks, stream);
+        const int err = kLaunch[s->K - 1](s->grad_dtype, oc, stats, a.dyn != nullptr, a, a.n_chunks, stream);
         if (err != 0) return JABAS_ERR_LAUNCH;
     }
     if (stats) {
@@ -384,7 +404,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
 
 using namespace jabas;
 
-JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.2 (gfx950)"; }
+JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.3 (gfx950)"; }
 
 JABAS_API const char* jabas_status_string(int status) {
     switch (status) {
@@ -403,6 +423,40 @@ JABAS_API const char* jabas_status_string(int status) {
         case JABAS_ERR_STATE: return "rendezvous: bucket handed over twice by one VSW in a step, or described again in the middle of a step";
         default: return "unknown status";
     }
+}
+
+JABAS_API int jabas_step_scalars_encode(const JabasStepArgs* args, void* host_block, size_t block_bytes) {
+    static_assert(sizeof(StepScal) % 16 == 0, "the block is copied and read in 16-byte pieces");
+    if (!args || !host_block) return JABAS_ERR_NULL;
+    if (block_bytes < sizeof(StepScal)) return JABAS_ERR_SIZE;
+    StepScal sc;
+    const int rc = fill_step_scal(args, &sc);
+    if (rc != JABAS_OK) return rc;
+    if (opt_class_of(args->opt_kind) == 0) return JABAS_ERR_OPT;
+    memcpy(host_block, &sc, sizeof(sc));
+    return JABAS_OK;
+}
+
+namespace {
+// One wave writes a step-scalar block that arrives by value in the kernel arguments: the refresh of the block
+// stays on the compute queue, in stream order with the launches that read it (a host-to-device copy would run
+// on a copy engine and cost a hand-over between engines before every step).
+struct ScalWords { uint32_t v[sizeof(StepScal) / 4]; };
+__global__ void __launch_bounds__(64) store_scalars_kernel(const ScalWords src, uint32_t* dst) {
+    for (uint32_t i = threadIdx.x; i < sizeof(StepScal) / 4; i += 64) dst[i] = src.v[i];
+}
+}  // namespace
+
+JABAS_API int jabas_step_scalars_upload(const JabasStepArgs* args, void* scalars_dev, jabas_stream_t stream) {
+    if (!args || !scalars_dev) return JABAS_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(scalars_dev) % 16) return JABAS_ERR_ALIGN;
+    ScalWords words;
+    static_assert(sizeof(words) == sizeof(StepScal), "same bytes");
+    const int rc = jabas_step_scalars_encode(args, &words, sizeof(words));
+    if (rc != JABAS_OK) return rc;
+    const hipError_t err = launch_kernel(store_scalars_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                                         words, static_cast<uint32_t*>(scalars_dev));
+    return err == hipSuccess ? JABAS_OK : JABAS_ERR_LAUNCH;
 }
 
 JABAS_API size_t jabas_sync_workspace_bytes(uint64_t numel, int32_t grad_dtype) {

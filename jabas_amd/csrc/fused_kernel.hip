@@ -117,6 +117,46 @@ __device__ __forceinline__ double stat_fma(float a, float b, double acc) {
 }
 __device__ __forceinline__ float stat_fma(float a, float b, float acc) { return __builtin_fmaf(a, b, acc); }
 
+// The step's scalars as the arithmetic below names them (a.w[k], a.wh[k], a.half_mask, a.opt, a.groups[i],
+// plus a.bounds and a.grad_scale), backed by a StepScal block in device memory instead of the kernel
+// arguments. The block is read through the constant address space: uniform loads that the compiler may
+// place anywhere, the same instructions a kernel-argument read compiles to, and the block is not written
+// while a launch that names it runs. Every function below takes either KArgs or this view.
+struct DynView {
+    typedef const __attribute__((address_space(4))) StepScal* Block;
+    struct Weights {
+        const __attribute__((address_space(4))) float* p;
+        __device__ __forceinline__ float operator[](int k) const { return p[k]; }
+    };
+    struct Groups {
+        Block b;
+        __device__ __forceinline__ GroupDev operator[](uint32_t i) const {
+            GroupDev g;
+            g.wd = b->groups[i].wd; g.neg_lr = b->groups[i].neg_lr; g.decay = b->groups[i].decay;
+            g.neg_step_size = b->groups[i].neg_step_size; g.sqrt_bc2 = b->groups[i].sqrt_bc2;
+            return g;
+        }
+    };
+    Weights w, wh;
+    Groups groups;
+    OptDev opt;
+    uint32_t half_mask;
+    const BoundDev* bounds;
+    const float* grad_scale;
+    __device__ __forceinline__ explicit DynView(const KArgs& a) {
+        Block b = (Block)a.dyn;
+        w.p = b->w; wh.p = b->wh; groups.b = b;
+        opt.momentum = b->opt.momentum; opt.one_minus_damp = b->opt.one_minus_damp;
+        opt.beta1 = b->opt.beta1; opt.one_minus_beta1 = b->opt.one_minus_beta1;
+        opt.beta2 = b->opt.beta2; opt.one_minus_beta2 = b->opt.one_minus_beta2; opt.eps = b->opt.eps;
+        opt.has_momentum = b->opt.has_momentum; opt.first_step = b->opt.first_step;
+        opt.nesterov = b->opt.nesterov; opt.adamw = b->opt.adamw;
+        half_mask = b->half_mask;
+        bounds = a.bounds;
+        grad_scale = a.grad_scale;
+    }
+};
+
 // One element of the optimizer step. g is the aggregated gradient.
 template <int OPT>
 __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2,
@@ -141,9 +181,9 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
 }
 
 // Aggregate, statistics and optimizer for N consecutive elements held in registers.
-template <int K, int N, int DT, int OPT, int SL, bool HD>
+template <int K, int N, int DT, int OPT, int SL, bool HD, class A>
 __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
-                                        float (&s2)[N], float (&agg)[N], const KArgs& a,
+                                        float (&s2)[N], float (&agg)[N], const A& a,
                                         const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
@@ -224,8 +264,8 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev
 }
 
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
-template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW>
-__device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const KArgs& a,
+template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW, class A>
+__device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const A& a,
                                         const GroupDev& G, float clip, bool use_s1, bool load_s1,
                                         typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
@@ -259,8 +299,8 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 
 // Vector path over nfull consecutive full tiles of one parameter group: groups of U tiles,
 // then U/2, ... down to single tiles.
-template <int K, int DT, int OPT, int SL, bool HD, int U>
-__device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const KArgs& a,
+template <int K, int DT, int OPT, int SL, bool HD, int U, class A>
+__device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const A& a,
                                          const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     constexpr int BS = launch_block(K, DT, OPT, SL);
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
@@ -282,8 +322,8 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
 // vector straddles the span's first or last element or a bound take the slow way, so such a tile costs
 // little more than a full one (ResNet-50's batch-norm tensors and ViT's biases put a group change
 // into roughly every hundredth tile; one span per tensor puts an edge into every tensor).
-template <int K, int DT, int OPT, int SL>
-__device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const KArgs& a, uint32_t j,
+template <int K, int DT, int OPT, int SL, class A>
+__device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const A& a, uint32_t j,
                                              float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
@@ -340,9 +380,9 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 }
 
 // Tiles [lt0, lt1) of one span (tile indices local to the span).
-template <int K, int DT, int OPT, int SL, bool HD>
+template <int K, int DT, int OPT, int SL, bool HD, class A>
 __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
-                                           const KArgs& a, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
+                                           const A& a, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
@@ -386,8 +426,8 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
 
 // Statistics kernels carry two copies of the arithmetic: one with the default halves
 // (even worker -> A, odd -> B) resolved at compile time, one driven by the half mask.
-template <int K, int DT, int OPT, int SL>
-__device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const KArgs& a,
+template <int K, int DT, int OPT, int SL, class A>
+__device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const A& a,
                                           typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     if constexpr (SL) {
         constexpr uint32_t kDefaultMask = 0xAAAAu & ((1u << K) - 1u);
@@ -471,17 +511,14 @@ __device__ __forceinline__ void flush_stats(float (&acc)[NS], double* row) {
     }
 }
 
-template <int K, int DT, int OPT, int SL>
-__global__ void __launch_bounds__(launch_block(K, DT, OPT, SL)) fused_kernel(const KArgs a) {
-    constexpr int NS = NStats<K, SL>::value;
+// The chunk of workgroup b: a names the launch (spans, chunk table), s the step's scalars (a itself, or the
+// view of the device block).
+template <int K, int DT, int OPT, int SL, class A>
+__device__ __forceinline__ void workgroup_chunk(const KArgs& a, const A& s, uint32_t b,
+                                                typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     constexpr int BS = launch_block(K, DT, OPT, SL);
     constexpr uint32_t CT = launch_chunk_tiles(K, DT, OPT, SL);     // the host cuts the chunk table for the same shape
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
-    const uint32_t b = blockIdx.x;
-    typename StatAcc<DT>::type acc[NS];
-#pragma unroll
-    for (int i = 0; i < NS; ++i) acc[i] = 0;
-
     if (a.use_inline) {
         const SpanDev& sp = a.span0;
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
@@ -499,19 +536,37 @@ __global__ void __launch_bounds__(launch_block(K, DT, OPT, SL)) fused_kernel(con
             }
             j0 = lo;
         }
-        run_chunk<K, DT, OPT, SL>(sp, lt0, lt1, j0, a, acc);
+        run_chunk<K, DT, OPT, SL>(sp, lt0, lt1, j0, s, acc);
     } else {
         const ChunkDesc c = a.chunks[b];
         const SpanDev& sp = a.spans[c.span];
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
         const uint32_t lt1 = c.tile0 + CT < tiles ? c.tile0 + CT : tiles;
-        run_chunk<K, DT, OPT, SL>(sp, c.tile0, lt1, c.bound0, a, acc);
+        run_chunk<K, DT, OPT, SL>(sp, c.tile0, lt1, c.bound0, s, acc);
+    }
+}
+
+// DYN: the step's scalars are read from the device block a.dyn names (a launch that a HIP graph replays
+// with another learning rate or Adam step) instead of from the kernel arguments.
+template <int K, int DT, int OPT, int SL, bool DYN>
+__global__ void __launch_bounds__(launch_block(K, DT, OPT, SL)) fused_kernel(const KArgs a) {
+    constexpr int NS = NStats<K, SL>::value;
+    constexpr int BS = launch_block(K, DT, OPT, SL);
+    const uint32_t b = blockIdx.x;
+    typename StatAcc<DT>::type acc[NS];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) acc[i] = 0;
+    if constexpr (DYN) {
+        const DynView s(a);
+        workgroup_chunk<K, DT, OPT, SL>(a, s, b, acc);
+    } else {
+        workgroup_chunk<K, DT, OPT, SL>(a, a, b, acc);
     }
     if constexpr (SL) flush_stats<NS, BS>(acc, a.partials + static_cast<uint64_t>(b) * NS);   // compact rows of 4 + K
 }
 
 template <int K, int DT, int OPT, int SL>
-int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
+int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
     // Residency cap through idle dynamic LDS (160 KB per CU). Fewer resident workgroups keep the
     // streamed window of every buffer more compact, which the memory system rewards on write-heavy
     // mixes as long as the kernel does not need the waves to hide its own arithmetic. Measured (A/B in
@@ -521,8 +576,13 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
 #define JABAS_IDLE_LDS_BYTES 32768u
 #endif
     constexpr unsigned idle = (OPT == OPT_ADAM && !SL && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
-    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL>, dim3(grid), dim3(launch_block(K, DT, OPT, SL)),
-                                          idle, stream, a));
+    const dim3 block(launch_block(K, DT, OPT, SL));
+    if constexpr (OPT != OPT_NONE) {
+        if (dyn) return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, true>, dim3(grid), block, idle, stream, a));
+    } else {
+        if (dyn) return static_cast<int>(hipErrorInvalidValue);     // refused by the front before it gets here
+    }
+    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, false>, dim3(grid), block, idle, stream, a));
 }
 
 }  // namespace
@@ -554,9 +614,9 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream) {
         default: return -1;                                                                  \
     }
 
-int JABAS_CAT(launch_fused_k, JABAS_K)(int grad_dtype, int opt_class, int stats, const KArgs& a,
+int JABAS_CAT(launch_fused_k, JABAS_K)(int grad_dtype, int opt_class, int stats, int dyn, const KArgs& a,
                                        unsigned grid, hipStream_t stream) {
-    JABAS_DISPATCH(launch_one, a, grid, stream)
+    JABAS_DISPATCH(launch_one, a, grid, stream, dyn != 0)
 }
 
 }  // namespace jabas

@@ -154,7 +154,22 @@ struct KArgs {
     float wh[JABAS_MAX_K];
     OptDev opt;
     GroupDev groups[JABAS_MAX_GROUPS];
+    const struct StepScal* dyn;              // device block holding this step's scalars, or NULL (they are the fields above)
 };
+
+// The scalars of a step that change from one step to the next (weights, optimizer constants, per-group
+// constants), as a block in device memory: a launch that names such a block reads them from there instead
+// of from its own arguments, so a launch recorded in a HIP graph can be replayed with the learning rate,
+// the Adam step or the weights of the moment. Same layout on host and device; written by
+// jabas_step_scalars_encode.
+struct StepScal {
+    float w[JABAS_MAX_K];
+    float wh[JABAS_MAX_K];
+    OptDev opt;
+    uint32_t half_mask;
+    GroupDev groups[JABAS_MAX_GROUPS];
+};
+static_assert(sizeof(StepScal) == JABAS_STEP_SCALARS_BYTES, "public size of the step-scalar block");
 
 #if defined(__HIPCC__)
 // Launch through hipLaunchKernel so that the status is the one of THIS launch: hipGetLastError() would
@@ -192,9 +207,10 @@ __device__ __forceinline__ double wave_sum_to_lane63(double v) {
 #endif
 
 // Per-K launchers, one translation unit each (fused_kernel.hip with -DJABAS_K=k).
-// opt_class: 0 none, 1 SGD, 2 Adam/AdamW. Returns hipError_t as int.
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW; dyn: the step's scalars come from a.dyn (optimizer classes only).
+// Returns hipError_t as int.
 #define JABAS_DECLARE_K(k)                                                                   \
-    int launch_fused_k##k(int grad_dtype, int opt_class, int stats, const KArgs& a,          \
+    int launch_fused_k##k(int grad_dtype, int opt_class, int stats, int dyn, const KArgs& a, \
                           unsigned grid, hipStream_t stream);
 JABAS_DECLARE_K(1) JABAS_DECLARE_K(2) JABAS_DECLARE_K(3) JABAS_DECLARE_K(4)
 JABAS_DECLARE_K(5) JABAS_DECLARE_K(6) JABAS_DECLARE_K(7) JABAS_DECLARE_K(8)

@@ -12,7 +12,7 @@ import torch
 
 from . import _lib as L
 from .layout import FlatLayout
-from .sync import SpanSpec, SyncPlan, make_step_args, opt_kind, cosine_from_stats, clip_coef
+from .sync import SpanSpec, SyncPlan, StepScalars, aggregate, make_step_args, opt_kind, cosine_from_stats, clip_coef
 
 
 class VSWFlatSync:
@@ -69,6 +69,7 @@ class VSWFlatSync:
         self.span_bucket = [s[3] for s in self.layout.spans]
         self.plan = SyncPlan(spans, kind)
         self._plan_agg = self._plan_opt = self._coef = None
+        self._generation = getattr(self, "_generation", 0) + 1     # recorded graphs name the old plan's tables
 
     # ---- reconfiguration ---------------------------------------------------------
     def reconfigure(self, batches):
@@ -133,22 +134,44 @@ class VSWFlatSync:
         scaled by it -- the norm has to be known before any weight moves.
 
         ``accumulations``: micro-batches every VSW summed into its buckets since the last step."""
-        if clip_norm is None or self.opt is None:
-            args = self.step_args(stats=stats, lr_scale=lr_scale, accumulations=accumulations)
-            out = self.plan.run(args, stream=stream)
-            self.step_count += 1
-            return out
-        if self._plan_agg is None:
+        out = self._queue(stats, lr_scale, stream, clip_norm, accumulations, None)
+        self.step_count += 1
+        return out
+
+    def _clipped(self, clip_norm):
+        return clip_norm is not None and self.opt is not None
+
+    def _update_args(self, stats, lr_scale, clip_norm, accumulations):
+        """Arguments of the launch that moves the weights in the coming step."""
+        if not self._clipped(clip_norm):
+            return self.step_args(stats=stats, lr_scale=lr_scale, accumulations=accumulations)
+        return make_step_args((1,), torch.float32, stats=False, opt=self.opt, step=self.step_count + 1,
+                              first_step=self.step_count == 0, lr_scale=lr_scale, grad_scale=self._coef)
+
+    def _queue(self, stats, lr_scale, stream, clip_norm, accumulations, scalars):
+        if self._clipped(clip_norm) and self._plan_agg is None:
             self._build_clip_plans()
+        args = self._update_args(stats, lr_scale, clip_norm, accumulations)
+        if scalars is not None:
+            scalars.attach(args)
+        if not self._clipped(clip_norm):
+            return self.plan.run(args, stream=stream)
         # the norm needs the similarity sums only; a caller that asked for full rows gets them
         level = stats if stats else "similarity"
         rows = self._plan_agg.run(self.step_args(stats=level, with_opt=False, accumulations=accumulations), stream=stream)
-        coef = clip_coef(rows, clip_norm, out=self._coef, stream=stream)
-        args = make_step_args((1,), torch.float32, stats=False, opt=self.opt, step=self.step_count + 1,
-                              first_step=self.step_count == 0, lr_scale=lr_scale, grad_scale=coef)
+        clip_coef(rows, clip_norm, out=self._coef, stream=stream)
         self._plan_opt.run(args, stream=stream)
-        self.step_count += 1
         return rows if stats else None
+
+    def capture(self, stats=False, clip_norm=None, accumulations=1):
+        """Records the step in a HIP graph. The returned object's ``replay(lr_scale=...)`` is ``step`` with
+        one graph launch instead of the step's kernel launches; the learning rates, Adam's step count and
+        the first-step flag of the moment reach the recorded launch through a block in device memory
+        (``StepScalars``) that is refreshed ahead of every replay. Statistics level, clipping and
+        ``accumulations`` are fixed by the recording; ``reconfigure`` invalidates it."""
+        if self.opt is None:
+            raise ValueError("nothing moves between the steps of an engine without optimizer: record its launch directly")
+        return GraphedStep(self, stats, clip_norm, accumulations)
 
     def _build_clip_plans(self):
         agg_spans, opt_spans = [], []
@@ -175,3 +198,33 @@ class VSWFlatSync:
     @staticmethod
     def cosine(stats):
         return cosine_from_stats(stats)
+
+
+class GraphedStep:
+    """A sync step of a ``VSWFlatSync`` recorded once in a HIP graph (``VSWFlatSync.capture``)."""
+
+    def __init__(self, engine, stats, clip_norm, accumulations):
+        self.engine, self.stats, self.clip_norm, self.accumulations = engine, stats, clip_norm, accumulations
+        self.scalars = StepScalars(engine.device)
+        self._generation = engine._generation
+        # the first launch out of a code object loads it, which a recording stream must not do: one launch of
+        # the same K over a scratch element first
+        warm = [torch.zeros(4, dtype=engine.grad_dtype, device=engine.device) for _ in range(engine.K)]
+        aggregate(warm, (1,) * engine.K, out=torch.zeros(4, dtype=torch.float32, device=engine.device))
+        if engine._clipped(clip_norm):
+            if engine._plan_agg is None:
+                engine._build_clip_plans()
+            aggregate(warm[:1], (1,), out=torch.zeros(4, dtype=torch.float32, device=engine.device))
+        torch.cuda.synchronize(engine.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.out = engine._queue(stats, 1.0, None, clip_norm, accumulations, self.scalars)
+
+    def replay(self, lr_scale=1.0):
+        eng = self.engine
+        if eng._generation != self._generation:
+            raise RuntimeError("the engine was reconfigured after this step was recorded: record it again")
+        self.scalars.update(eng._update_args(self.stats, lr_scale, self.clip_norm, self.accumulations))
+        self.graph.replay()
+        eng.step_count += 1
+        return self.out

@@ -128,6 +128,27 @@ def make_step_args(batches, grad_dtype, stats=False, opt=None, step=1, first_ste
     return a
 
 
+class StepScalars:
+    """The scalars of a step that move from step to step (weights, learning rates, Adam's bias corrections,
+    the first-step flag) as a block in device memory, for launches recorded in a HIP graph: a recorded launch
+    has its by-value arguments baked in, one that names this block (``attach``) reads the block as it is when
+    the kernel runs. ``update(args)`` encodes the arguments of the coming step on the host (the same
+    double -> fp32 derivation as a plain call) and queues a one-wave kernel that writes them to the block
+    (``jabas_step_scalars_upload``), on the stream the replay follows on."""
+
+    def __init__(self, device):
+        self.dev = torch.zeros(L.STEP_SCALARS_BYTES, dtype=torch.uint8, device=device)
+
+    def attach(self, args):
+        args.scalars_dev = self.dev.data_ptr()
+        args._keep_scalars = self                   # keeps the block alive as long as the args
+        return args
+
+    def update(self, args, stream=None):
+        L.check(L.lib().jabas_step_scalars_upload(C.byref(args), self.dev.data_ptr(), _stream_ptr(stream)),
+                "jabas_step_scalars_upload")
+
+
 # ------------------------------------------------------------------------------- spans
 def _ptr(t):
     return None if t is None else t.data_ptr()

@@ -48,6 +48,7 @@ int main(void) {
     SHOW_OFF(JabasStepArgs, eps);
     SHOW_OFF(JabasStepArgs, groups);
     SHOW_OFF(JabasStepArgs, grad_scale);
+    SHOW_OFF(JabasStepArgs, scalars_dev);
 
     printf("version %s\n", jabas_sync_version());
     printf("status0 %s\n", jabas_status_string(JABAS_OK));

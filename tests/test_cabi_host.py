@@ -37,7 +37,8 @@ def test_struct_layouts_match_the_header():
     assert C.sizeof(L.JabasSpan) == K * 8 + 4 * 8 + (K - 1) * 8 + 8 + 4 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
-    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 4 * K + 4 + K + 4 * K + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8
+    assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 4 * K + 4 + K + 4 * K + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8 + 8
+    assert L.JabasStepArgs.scalars_dev.offset == C.sizeof(L.JabasStepArgs) - 8
     assert L.JabasStepArgs.groups.offset % 8 == 0 and L.JabasStepArgs.momentum.offset % 8 == 0
 
 
@@ -248,7 +249,7 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
             s, f = name.split(".")
             assert getattr(structs[s], f).offset == int(val), name
             checked += 1
-    assert checked == 36
+    assert checked == 37
     # every field of the ctypes mirror was reported by the C side (reserved words aside)
     for sname, st in structs.items():
         for f, _ in st._fields_:
@@ -481,3 +482,63 @@ def test_rendezvous_calls_validate_their_arguments():
     assert lib.jabas_rdv_reset(None) == L.ERR_NULL
     lib.jabas_rdv_destroy(None)
     assert b"rendezvous" in lib.jabas_status_string(L.ERR_STATE)
+
+
+def test_step_scalar_block_holds_the_constants_a_plain_call_derives():
+    """jabas_step_scalars_encode is host code: its block is compared, slot by slot, with the constants derived
+    here in Python doubles and rounded once to fp32 (what a Python float becomes as an fp32 kernel scalar)."""
+    import torch
+    from jabas_amd import sync
+    lib = L.lib()
+    f32 = lambda x: np.float32(x)
+    opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+               groups=[dict(lr=5e-4, weight_decay=0.05, step=7), dict(lr=1e-3, weight_decay=0.0, step=3)])
+    batches = (48, 32, 32, 16, 8)
+    m = 2.5 ** 0.5
+    args = sync.make_step_args(batches, torch.bfloat16, stats="similarity", opt=opt, lr_scale=m,
+                               half_id=[0, 1, 1, 0, 1])
+    block = np.zeros(L.STEP_SCALARS_BYTES, dtype=np.uint8)
+    assert lib.jabas_step_scalars_encode(C.byref(args), block.ctypes.data, block.nbytes) == L.OK
+    fl, u32 = block.view(np.float32), block.view(np.uint32)
+    w, hid, hw = sync.batch_weights(batches, [0, 1, 1, 0, 1])
+    assert np.array_equal(fl[0:5], w) and not fl[5:16].any()
+    assert np.array_equal(fl[16:21], hw) and not fl[21:32].any()
+    o = 32                                                       # OptDev: 7 floats, 4 flags
+    assert fl[o + 2] == f32(0.9) and fl[o + 3] == f32(1.0 - 0.9)
+    assert fl[o + 4] == f32(0.999) and fl[o + 5] == f32(1.0 - 0.999) and fl[o + 6] == f32(1e-8)
+    assert list(u32[o + 7:o + 11]) == [0, 0, 0, 1]               # has_momentum, first_step, nesterov, adamw
+    assert u32[o + 11] == 0b10110                                # half B: workers 1, 2, 4
+    for i, g in enumerate(opt["groups"]):
+        base = 44 + 8 * i
+        lr = g["lr"] * m
+        assert fl[base + 0] == f32(g["weight_decay"])
+        assert fl[base + 1] == f32(-lr)
+        assert fl[base + 2] == f32(1.0 - lr * g["weight_decay"])
+        assert fl[base + 3] == f32(-(lr / (1.0 - 0.9 ** g["step"])))
+        assert fl[base + 4] == f32((1.0 - 0.999 ** g["step"]) ** 0.5)
+    assert not fl[44 + 16:].any()
+    # SGD: momentum, dampening, the first-step flag
+    sgd = dict(kind="sgd", momentum=0.9, dampening=0.1, nesterov=False, groups=[dict(lr=0.1, weight_decay=1e-4)])
+    args = sync.make_step_args((2, 2), torch.float32, opt=sgd, first_step=True)
+    assert lib.jabas_step_scalars_encode(C.byref(args), block.ctypes.data, block.nbytes) == L.OK
+    assert fl[o] == f32(0.9) and fl[o + 1] == f32(1.0 - 0.1) and list(u32[o + 7:o + 11]) == [1, 1, 0, 0]
+    assert fl[44 + 1] == f32(-0.1) and fl[44 + 3] == 0.0 and fl[44 + 4] == 1.0
+    # argument checks
+    assert lib.jabas_step_scalars_encode(None, block.ctypes.data, block.nbytes) == L.ERR_NULL
+    assert lib.jabas_step_scalars_encode(C.byref(args), None, block.nbytes) == L.ERR_NULL
+    assert lib.jabas_step_scalars_encode(C.byref(args), block.ctypes.data, L.STEP_SCALARS_BYTES - 1) == L.ERR_SIZE
+    none = sync.make_step_args((2, 2), torch.float32)
+    assert lib.jabas_step_scalars_encode(C.byref(none), block.ctypes.data, block.nbytes) == L.ERR_OPT
+    adam0 = sync.make_step_args((2, 2), torch.float32, opt=dict(opt, groups=[dict(lr=1e-3, step=0)]))
+    assert lib.jabas_step_scalars_encode(C.byref(adam0), block.ctypes.data, block.nbytes) == L.ERR_OPT
+    assert lib.jabas_step_scalars_upload(None, 0x7f0000001000, None) == L.ERR_NULL
+    assert lib.jabas_step_scalars_upload(C.byref(args), None, None) == L.ERR_NULL
+    assert lib.jabas_step_scalars_upload(C.byref(args), 0x7f0000001004, None) == L.ERR_ALIGN
+    assert lib.jabas_step_scalars_upload(C.byref(none), 0x7f0000001000, None) == L.ERR_OPT
+    # a launch without optimizer has nothing that moves between steps: a block is refused, as is a misaligned one
+    span = _span(5000)
+    none.scalars_dev = 0x7f0000001000
+    assert lib.jabas_sync_bucket(C.byref(span), None, C.byref(none), None, None, 0, None) == L.ERR_OPT
+    span = _span(5000, opt=True)
+    args.scalars_dev = 0x7f0000001008
+    assert lib.jabas_sync_bucket(C.byref(span), None, C.byref(args), None, None, 0, None) == L.ERR_ALIGN

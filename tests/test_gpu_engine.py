@@ -1,10 +1,14 @@
 """GPU tests of the flat-arena engine: multi-bucket plans with parameter groups, in-place
 aggregation, fan-out, per-tensor spans, and global-norm clipping (two launches with a
 device-side coefficient), against the oracle over the same arenas."""
+import ctypes as C
 import math
 
+import numpy as np
 import pytest
 import torch
+
+from jabas_amd import _lib as L
 
 from oracle import oracle as O
 from jabas_amd.workloads import ParamSpec
@@ -201,3 +205,86 @@ def test_parameter_groups_at_different_adam_step_counts(gpu, kind):
     O.sync_step(hg, batches, [(0, n, bounds)], dict(opt, groups=[dict(g, step=5) for g in opt["groups"]]), q_h,
                 m_h.clone(), v_h.clone(), step=1)
     assert not torch.equal(q_h, p_h)
+
+
+ADAMW = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+             groups=[dict(lr=5e-4, weight_decay=0.0), dict(lr=5e-4, weight_decay=0.05)])
+
+
+@pytest.mark.parametrize("opt,dtype,batches,stats", [
+    (ADAMW, torch.float32, (48, 32, 32, 16), "similarity"),
+    (ADAM, torch.bfloat16, (64, 56, 48, 40, 32, 24, 16, 8), "similarity"),
+    (ADAM, torch.float32, (3, 2, 1), True),
+    (SGD, torch.float32, (4, 2, 2), False),
+    (SGD, torch.bfloat16, (2,) * 9, True),
+])
+def test_recorded_step_replays_with_the_scalars_of_the_moment(gpu, opt, dtype, batches, stats):
+    """A step recorded ONCE in a HIP graph, replayed from the very first step on (SGD's first-step flag, Adam's
+    bias corrections and an LR modifier that changes every step all reach the recorded launch through the
+    step-scalar block in device memory): aggregate, weights and optimizer state bit for bit against the oracle
+    at every replay, with fresh gradients, eager work and synchronisations between the replays, and bit for
+    bit against the same steps launched one by one."""
+    K = len(batches)
+    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=1)
+    eager, _, _ = _make(gpu, batches, opt, dtype)
+    adam = opt["kind"] != "sgd"
+    graphed = eng.capture(stats=stats)
+    mods = (1.0, math.sqrt(20 / 8), 0.5, 1.0 / 3.0, 1.0)
+    for step, m in enumerate(mods, 1):
+        gen = torch.Generator().manual_seed(500 + step)
+        for k in range(K):
+            host["g"][k] = (torch.randn(eng.layout.total, generator=gen) * 1e-2).to(dtype)
+            eng.grads[k].copy_(host["g"][k])
+            eager.grads[k].copy_(host["g"][k])
+        scratch = (eng.grads[K - 1].float() * 2.0).sum()           # a library reduction between the replays
+        rows = graphed.replay(lr_scale=m)
+        rows_e = eager.step(stats=stats, lr_scale=m)
+        torch.cuda.synchronize()
+        assert torch.isfinite(scratch) and eng.step_count == step
+        # the block on the device holds what the host encoder gives for this step's arguments
+        eng.step_count -= 1
+        block = np.zeros(L.STEP_SCALARS_BYTES, dtype=np.uint8)
+        L.check(L.lib().jabas_step_scalars_encode(C.byref(eng.step_args(stats=stats, lr_scale=m)), block.ctypes.data,
+                                                  block.nbytes), "encode")
+        eng.step_count += 1
+        assert np.array_equal(graphed.scalars.dev.cpu().numpy(), block)
+        agg_h, rows_h = O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"] if adam else None,
+                                    step=step, first_step=(step == 1), want_stats=bool(stats), lr_scale=m)
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            assert torch.equal(eng.agg[sl].cpu().view(torch.int32), agg_h[sl].view(torch.int32)), (step, m)
+            assert torch.equal(eng.param[sl].cpu().view(torch.int32), host["p"][sl].view(torch.int32)), (step, m)
+            assert torch.equal(eng.state1[sl].cpu().view(torch.int32), host["s1"][sl].view(torch.int32)), (step, m)
+            if adam:
+                assert torch.equal(eng.state2[sl].cpu().view(torch.int32), host["s2"][sl].view(torch.int32)), (step, m)
+            assert torch.equal(eng.fanout[0][sl], eng.param[sl])
+            assert torch.equal(eager.param[sl], eng.param[sl])
+        if stats:
+            assert torch.equal(rows, rows_e)                       # same kernels' arithmetic, same order
+            rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+            width = 4 if stats == "similarity" else 4 + K
+            assert _close(rows[:, :width], rows_h[:, :width], rtol, 1e-30)
+
+
+def test_recorded_clipped_step_and_reconfigure(gpu):
+    """Global-norm clipping inside the recording (aggregate + sums, coefficient on the device, Adam over the
+    scaled aggregate: three launches, one graph), three replays against the oracle; a recording made before
+    ``reconfigure`` refuses to replay."""
+    batches = (128, 128, 64, 64)
+    eng, host, spans = _make(gpu, batches, ADAM, n_fanout=1)
+    graphed = eng.capture(clip_norm=0.05)
+    for step in (1, 2, 3):
+        gen = torch.Generator().manual_seed(700 + step)
+        for k in range(len(batches)):
+            host["g"][k] = torch.randn(eng.layout.total, generator=gen) * 1e-2
+            eng.grads[k].copy_(host["g"][k])
+        graphed.replay(lr_scale=1.0 + 0.25 * step)
+        torch.cuda.synchronize()
+        O.sync_step(host["g"], batches, spans, ADAM, host["p"], host["s1"], host["s2"], step=step,
+                    first_step=(step == 1), lr_scale=1.0 + 0.25 * step, clip_norm=0.05)
+        assert float(eng._coef) < 1.0
+        assert _close(eng.param, host["p"]) and _close(eng.state1, host["s1"], 1e-6, 2e-9)
+        assert _close(eng.state2, host["s2"], 1e-6, 1e-12)
+    eng.reconfigure((4, 4))
+    with pytest.raises(RuntimeError, match="record it again"):
+        graphed.replay()
