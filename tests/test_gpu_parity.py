@@ -582,10 +582,17 @@ def test_random_plans_match_the_oracle(gpu, seed):
                                      fanout=[f[sl] for f in fans], bounds=b))
     plan = sync.SyncPlan(spans_d, kind)
     hg_work = [t.clone() for t in hg]
+    block = sync.StepScalars(gpu) if opt and seed % 2 else None
     for step in (1, 2, 3):
         stats = step != 2
         args = sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=step, first_step=(step == 1),
                                    half_id=half_id)
+        if block is not None:
+            # odd seeds: the step's scalars travel in the device block; the by-value arguments of the call are
+            # those of another step at another learning rate, as in a launch recorded once and replayed
+            block.update(args)
+            args = block.attach(sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=5, first_step=(step != 1),
+                                                    half_id=half_id, lr_scale=3.0))
         rows = plan.run(args)
         torch.cuda.synchronize()
         agg_h, rows_h = O.sync_step(hg_work, batches, spans_h, opt, p_h, s1_h, s2_h if adam else None, step=step,
@@ -645,10 +652,15 @@ def test_random_buckets_through_the_inline_path(gpu, seed):
         span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d if opt else None, state1=s1_d if opt else None,
                              state2=s2_d if adam else None, bounds=b)
         call = sync.BucketCall(span)
+        block = sync.StepScalars(gpu) if opt and (seed + si) % 2 else None
         for step in (1, 2, 3):
             stats = step != 2                  # the plain launch may run another workgroup shape
             args = sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=step, first_step=(step == 1),
                                        half_id=half_id)
+            if block is not None:              # every other bucket: scalars from the device block, stale ones by value
+                block.update(args)
+                args = block.attach(sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=9,
+                                                        first_step=(step != 1), half_id=half_id, lr_scale=0.25))
             row = call.run(args)
             torch.cuda.synchronize()
             agg_h, rows_h = O.sync_step(hg, batches, [(0, n, b)], opt, p_h, s1_h, s2_h if adam else None, step=step,
