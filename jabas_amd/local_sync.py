@@ -47,7 +47,6 @@ class _Slot:
         self.tensors = [None] * K
         self.buckets = [None] * K
         self.events = [None] * K
-        self.seq = [0] * K
         self.want_stats = False
         self.on_done = None
         self.count = 0
@@ -106,7 +105,6 @@ class LocalBucketSync:
         if self.batch_bytes and launcher is not None:
             raise ValueError("batched launches drive the C ABI themselves: no launcher can be injected")
         self._ready_bytes = 0
-        self._seq = [0] * len(tuple(batches))  # per VSW: buckets published so far (orders its events)
         self._plans = {}                       # batched mode: group of buckets -> its plan
         self._stream_cache = {}
         self.stats_level = sync.stats_level(stats_level) or L.STATS_SIMILARITY
@@ -292,10 +290,11 @@ class LocalBucketSync:
         event = stream = None
         if tensor.is_cuda:
             stream = self._current_stream(tensor)
-            if not self.deferred and (k != 0 or self._sync_stream is not None):
+            if not self.deferred and not self.batch_bytes and (k != 0 or self._sync_stream is not None):
                 # VSW 0's own stream needs none when the launch is queued on it. A fresh event every time:
                 # recording one event again step after step (to save its creation) made the waits on it
-                # three times as expensive on this runtime
+                # three times as expensive on this runtime. (Batched and deferred launches order themselves
+                # behind one event per VSW stream, recorded when the launch is queued.)
                 event = torch.cuda.Event()
                 event.record(stream)
         batch = None
@@ -308,8 +307,6 @@ class LocalBucketSync:
             if slot.tensors[k] is not None:
                 raise RuntimeError(f"VSW {k} published bucket {bucket_index} twice in one step")
             slot.tensors[k], slot.events[k], slot.buckets[k] = tensor, event, bucket
-            self._seq[k] += 1
-            slot.seq[k] = self._seq[k]
             slot.count += 1
             if k == 0:
                 slot.want_stats, slot.on_done = want_stats, on_done
@@ -327,7 +324,7 @@ class LocalBucketSync:
         if ready:
             self._fire(bucket_index, slot)
         elif batch is not None:
-            self._fire_group(batch, per_publish_events=True)
+            self._fire_group(batch)
         return fut
 
     def _current_stream(self, tensor):
@@ -502,9 +499,13 @@ class LocalBucketSync:
                              bounds=(pb or {}).get("bounds", ()) if opt else ())
         return span, opt is not None
 
-    def _fire_group(self, ready, per_publish_events):
+    def _fire_group(self, ready):
         """One planned launch over a group of complete buckets, in bucket order: all buckets of the step
-        (deferred mode, from ``finish_step``) or a batch of them (batched mode)."""
+        (deferred mode, from ``finish_step``) or a batch of them (batched mode). The launch is ordered behind
+        one event per VSW stream, recorded here: every VSW has handed over all buckets of the group, so
+        whatever its stream holds by now includes the work that filled them (and at most the few kernels its
+        thread has queued since). A fresh event per hand-over, of which only each VSW's last would be waited
+        for, cost the hooks 5 us each: 1.5 ms of host time per ViT-L/16 step."""
         with self._lock:
             vsw_streams = sorted(self._vsw_streams.items())
         order = sorted(ready)
@@ -514,25 +515,14 @@ class LocalBucketSync:
             for i, slot in zip(order, slots):          # host tensors (protocol tests)
                 self._fire(i, slot)
             return
-        if len(order) == 1 and per_publish_events:
-            self._fire(order[0], slots[0])
-            return
         try:
-            if per_publish_events:
-                # per VSW, the event of the bucket it handed over last covers its earlier ones
-                for k in range(self.K):
-                    last = max(slots, key=lambda sl: sl.seq[k])
-                    if last.events[k] is not None:
-                        main.wait_event(last.events[k])
-            else:
-                # everything the VSWs queued up to now (their whole backward) precedes the launch: one
-                # event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
-                # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
-                for k, stream in vsw_streams:
-                    if stream != main:
-                        ev = torch.cuda.Event()
-                        ev.record(stream)
-                        main.wait_event(ev)
+            # one event per stream instead of one per bucket and VSW, which on the GPU's queue are a barrier
+            # packet each (98 of them per step for 14 buckets x 4 VSWs cost 0.25 ms)
+            for k, stream in vsw_streams:
+                if stream != main:
+                    ev = torch.cuda.Event()
+                    ev.record(stream)
+                    main.wait_event(ev)
             for i, slot in zip(order, slots):
                 self._bind_bucket(i, slot)
         except Exception as exc:
@@ -620,7 +610,7 @@ class LocalBucketSync:
         with self._lock:
             ready, self._ready, self._ready_bytes = self._ready, {}, 0
         if ready:
-            self._fire_group(ready, per_publish_events=not self.deferred)
+            self._fire_group(ready)
         # the launches of a step sit on one stream in order: one event behind the last of them orders
         # every VSW stream behind all of them
         with self._lock:
