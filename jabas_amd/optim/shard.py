@@ -31,6 +31,51 @@ class _ShardOptimizer(torch.optim.Optimizer):
         super().__init__(params, defaults)
         self._plans = {}
         self._recipes = {}          # call signature -> prepared launches (see _signature)
+        self._replicas = {}         # id(parameter) -> the same parameter of the other VSW replicas
+
+    def attach_replicas(self, main_params=(), *replica_params):
+        """``main_params``: the parameters of the model this optimizer updates; ``replica_params``: those of the
+        other VSW replicas on this GPU, one iterable per replica, in the same order (``model.parameters()`` of
+        identically built models). Every update then also writes the new weights into the replicas, in the
+        same launch (4 more bytes written per element and replica, nothing read again), which is the copy of
+        the main VSW's weights to the other VSWs that follows the optimizer step in IIDP
+        (jabas/train/trainer.py:530-534 shows the same copy when VSWs are added). Call again after replacing a
+        replica's tensors; call without arguments to detach."""
+        mine = list(main_params)
+        held = {id(p) for group in self.param_groups for p in group["params"]}
+        if len(replica_params) > L.MAX_K - 1:
+            raise ValueError(f"at most {L.MAX_K - 1} replicas")
+        if replica_params and not held <= {id(p) for p in mine}:
+            raise ValueError("main_params must hold every parameter of the optimizer")
+        table = {}
+        for r, params in enumerate(replica_params):
+            theirs = list(params)
+            if len(theirs) != len(mine):
+                raise ValueError(f"replica {r} has {len(theirs)} parameters, the main model {len(mine)}")
+            for p, q in zip(mine, theirs):
+                if id(p) not in held:
+                    continue
+                if q is p or q.shape != p.shape or q.dtype != torch.float32 or q.device != p.device:
+                    raise ValueError(f"replica {r}: a parameter does not mirror the main model's (shape, dtype, "
+                                     "device, or it is the very same tensor)")
+                if not q.is_contiguous():
+                    raise ValueError(f"replica {r}: parameters must be contiguous")
+                table.setdefault(id(p), []).append(q)
+        self._replicas = table
+        self._plans.clear()
+        self._recipes.clear()
+        return self
+
+    def _fanout(self, p):
+        """Flat views of p's replicas for the launch; a replica that sits at another position of a 16-byte line
+        than p cannot share p's vector accesses and is copied after the launch instead."""
+        views = []
+        for q in self._replicas.get(id(p), ()):
+            if self._congruent(q.data, p):
+                views.append(q.data.view(-1))
+            else:
+                self._late_copies.append((q, p))
+        return views
 
     def load_state_dict(self, state_dict):
         super().load_state_dict(state_dict)
@@ -42,14 +87,23 @@ class _ShardOptimizer(torch.optim.Optimizer):
     # (DDP bucket views keep their addresses). Matching, validating and marshalling ~150 tensors costs
     # more host time than the launch takes on the GPU, so a call that found every state in place is
     # remembered under its signature, and repeated calls only refresh the launch scalars.
-    @staticmethod
-    def _signature(pairs):
-        return tuple([(p.data_ptr(), g.data_ptr(), g.numel()) for _, p, g in pairs])
+    def _signature(self, pairs):
+        rep = self._replicas
+        if not rep:
+            return tuple([(p.data_ptr(), g.data_ptr(), g.numel()) for _, p, g in pairs])
+        return tuple([(p.data_ptr(), g.data_ptr(), g.numel()) + tuple(q.data_ptr() for q in rep.get(id(p), ()))
+                      for _, p, g in pairs])
 
     def _remember(self, sig, launches, copies):
         if len(self._recipes) >= self._max_cached_plans:
             self._recipes.clear()
-        self._recipes[sig] = (launches, copies)
+        self._recipes[sig] = (launches, copies, list(self._late_copies))
+
+    _late_copies = ()
+
+    def _copy_late(self, late):
+        for q, p in late:
+            q.data.copy_(p.data)
 
     # -- matching ---------------------------------------------------------------------
     def _pairs(self, gradients):
@@ -102,7 +156,8 @@ class _ShardOptimizer(torch.optim.Optimizer):
         return g
 
     def _launch(self, spans, args):
-        key = tuple((s.grads[0].data_ptr(), s.param.data_ptr(), s.grads[0].numel(), s.bounds[0][1]) for s in spans)
+        key = tuple((s.grads[0].data_ptr(), s.param.data_ptr(), s.grads[0].numel(), s.bounds[0][1]) +
+                    tuple(f.data_ptr() for f in s.fanout) for s in spans)
         plan = self._plans.get(key)
         if plan is None:
             if len(self._plans) >= self._max_cached_plans:
@@ -144,7 +199,7 @@ class ShardSGD(_ShardOptimizer):
         sig = self._signature(pairs)
         if self._replay(self._recipes.get(sig)):
             return loss
-        self._copies, self._volatile, launches = [], False, []
+        self._copies, self._volatile, launches, self._late_copies = [], False, [], []
         # launches are split by (momentum, dampening, nesterov, first-step): launch-wide scalars
         batches = {}
         for gi, p, g in pairs:
@@ -163,7 +218,7 @@ class ShardSGD(_ShardOptimizer):
                 if slot >= L.MAX_GROUPS:
                     raise RuntimeError(f"more than {L.MAX_GROUPS} parameter groups in one launch")
                 spans.append(sync.SpanSpec([g], param=p.data.view(-1), state1=None if buf is None else buf.view(-1),
-                                           bounds=((0, slot),)))
+                                           fanout=self._fanout(p), bounds=((0, slot),)))
             for gi, slot in slots.items():
                 args.groups[slot].lr = float(self.param_groups[gi]["lr"])
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
@@ -174,6 +229,7 @@ class ShardSGD(_ShardOptimizer):
             plan = self._launch(spans, args)
             launches.append((plan, args, (momentum, dampening, bool(nesterov)), list(slots.items())))
             self._volatile = self._volatile or first
+        self._copy_late(self._late_copies)
         if not self._volatile:
             self._remember(sig, launches, self._copies)
         return loss
@@ -183,7 +239,7 @@ class ShardSGD(_ShardOptimizer):
         nothing done) when a group changed a scalar the launches were split by."""
         if recipe is None:
             return False
-        launches, copies = recipe
+        launches, copies, late = recipe
         for _, _, key, slots in launches:
             for gi, _ in slots:
                 group = self.param_groups[gi]
@@ -196,6 +252,7 @@ class ShardSGD(_ShardOptimizer):
                 args.groups[slot].lr = float(self.param_groups[gi]["lr"])
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
             plan.run(args)
+        self._copy_late(late)
         return True
 
 
@@ -222,7 +279,7 @@ class ShardAdam(_ShardOptimizer):
         sig = self._signature(pairs)
         if self._replay(self._recipes.get(sig)):
             return loss
-        self._copies, self._volatile, launches = [], False, []
+        self._copies, self._volatile, launches, self._late_copies = [], False, [], []
         batches = {}
         for gi, p, g in pairs:
             group = self.param_groups[gi]
@@ -245,7 +302,8 @@ class ShardAdam(_ShardOptimizer):
                 if slot >= L.MAX_GROUPS:
                     raise RuntimeError(f"more than {L.MAX_GROUPS} (group, step) combinations in one launch")
                 spans.append(sync.SpanSpec([g], param=p.data.view(-1), state1=st["exp_avg"].view(-1),
-                                           state2=st["exp_avg_sq"].view(-1), bounds=((0, slot),)))
+                                           state2=st["exp_avg_sq"].view(-1), fanout=self._fanout(p),
+                                           bounds=((0, slot),)))
             for (gi, step), slot in slots.items():
                 args.groups[slot].lr = float(self.param_groups[gi]["lr"])
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
@@ -259,6 +317,7 @@ class ShardAdam(_ShardOptimizer):
                 reps.setdefault(slots[(gi, step)], (gi, st))
             launches.append((plan, args, (betas, eps), sorted(reps.items()),
                              [(st, slots[(gi, step)]) for gi, step, p, g, st in items]))
+        self._copy_late(self._late_copies)
         if not self._volatile:
             self._remember(sig, launches, self._copies)
         return loss
@@ -269,7 +328,7 @@ class ShardAdam(_ShardOptimizer):
         step count no longer do (they were stepped apart in between)."""
         if recipe is None:
             return False
-        launches, copies = recipe
+        launches, copies, late = recipe
         for _, _, key, reps, items in launches:
             for _, (gi, _) in reps:
                 group = self.param_groups[gi]
@@ -289,6 +348,7 @@ class ShardAdam(_ShardOptimizer):
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
                 args.groups[slot].step = int(st["step"])
             plan.run(args)
+        self._copy_late(late)
         return True
 
 

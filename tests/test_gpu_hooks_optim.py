@@ -97,6 +97,72 @@ def test_shard_step_with_bucket_gradients_updates_only_matching_parameters(gpu):
             assert len(opt.state[p]) == 0
 
 
+@pytest.mark.parametrize("kind", ["sgd", "adamw", "gnmt_adam"])
+def test_shard_optimizers_refresh_the_other_replicas_in_the_same_launch(gpu, kind):
+    """``attach_replicas``: the weights of the other VSWs' models follow the main model's bit for bit after
+    every ``step()`` and ``step(bucket gradients)``, through first and remembered calls, for a replica whose
+    tensors sit at another position of a 16-byte line too (copied after the launch); the main model itself
+    steps exactly as it does without replicas; detaching stops the refresh."""
+    from jabas_amd import optim
+    from jabas_amd.train.trainer import tag_parameter_indices
+    main, alone = tag_parameter_indices(_mlp(3).to(gpu)), tag_parameter_indices(_mlp(3).to(gpu))
+    rep1, rep2 = _mlp(3).to(gpu), _mlp(3).to(gpu)
+    # replica 2's parameters are views that start one element into their own buffers: not congruent with the main ones
+    for q in rep2.parameters():
+        buf = torch.zeros(q.numel() + 1, device=gpu)
+        view = buf[1:].view(q.shape)
+        view.copy_(q.data)
+        q.data = view
+
+    def build(model):
+        if kind == "sgd":
+            return optim.ShardSGD(_groups(model), lr=0.1, momentum=0.9)
+        if kind == "adamw":
+            return optim.ShardAdamW(_groups(model), lr=5e-4)
+        return optim.ShardGNMTAdam(list(model.parameters()), lr=2e-3, grad_clip=0.05)
+    mine, ref = build(main), build(alone)
+    assert mine.attach_replicas(main.parameters(), rep1.parameters(), rep2.parameters()) is mine
+    params = list(main.parameters())
+    for step in range(6):
+        gen = torch.Generator().manual_seed(40 + step)
+        grads = [(torch.randn(p.shape, generator=gen) * 1e-2).to(gpu) for p in params]
+        if step % 2 == 0:                                    # every parameter from its .grad
+            for m in (main, alone):
+                for p, g in zip(m.parameters(), grads):
+                    p.grad = g.clone()
+            mine.step()
+            ref.step()
+            touched = range(len(params))
+        else:                                                # one "bucket": parameters 1..3
+            touched = [1, 2, 3]
+            for opt_, m in ((mine, main), (ref, alone)):
+                views = []
+                for i in touched:
+                    v = grads[i].clone()
+                    v.index = i
+                    views.append(v)
+                opt_.step(views)
+        torch.cuda.synchronize()
+        for i, (p, a, q1, q2) in enumerate(zip(params, alone.parameters(), rep1.parameters(), rep2.parameters())):
+            assert torch.equal(p, a), (kind, step, i)                            # replicas change nothing for the main model
+            if i in touched or step > 0:
+                assert torch.equal(q1, p) and torch.equal(q2, p), (kind, step, i)
+    mine.attach_replicas()
+    before = [q.detach().clone() for q in rep1.parameters()]
+    for p in main.parameters():
+        p.grad = torch.ones_like(p) * 1e-2
+    mine.step()
+    torch.cuda.synchronize()
+    assert all(torch.equal(q, b) for q, b in zip(rep1.parameters(), before))
+    assert not torch.equal(params[0], before[0])
+    with pytest.raises(ValueError):
+        mine.attach_replicas(main.parameters(), list(rep1.parameters())[:-1])
+    with pytest.raises(ValueError):
+        mine.attach_replicas(main.parameters(), main.parameters())
+    with pytest.raises(ValueError):
+        mine.attach_replicas(list(main.parameters())[1:], list(rep1.parameters())[1:])
+
+
 @pytest.mark.parametrize("deferred", [False, True])
 def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
     """K hook threads on K streams hand their buckets over in different orders. Per-bucket mode: the
