@@ -140,11 +140,13 @@ def test_stock_ddp_buckets_through_the_hooks(gpu):
     dist.destroy_process_group()
 
 
+@pytest.mark.parametrize("mode", ["per_bucket", "batched", "deferred"])
 @pytest.mark.parametrize("kind", ["sgd", "adamw"])
-def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind):
+def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     """Overlap weight-sync mode end to end with stock DDP (jabas/train/trainer.py:327-333): the optimizer
     hook on VSW 0, a launch stream of its own, the weights of both replicas and the optimizer state
-    bit-exact against the oracle over four steps, across DDP's bucket rebuild after the first."""
+    bit-exact against the oracle over four steps, across DDP's bucket rebuild after the first; one launch
+    per bucket, per batch of buckets, and per step."""
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import prepare_overlap_optimizer_with_ddp
@@ -169,7 +171,7 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind):
     p_h = [p.detach().cpu().clone().reshape(-1) for p in main.parameters()]
     s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
 
-    local = LocalBucketSync(batches)
+    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=150_000 if mode == "batched" else 0)
     state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 2).attach_local(local)
     rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), main)
     prepare_overlap_optimizer_with_ddp(replicas, [state, H.VSWPeerState(local, 1)], [rec.hook, H.dummy_hook], optimizer, local)
@@ -201,6 +203,8 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind):
                 assert int(st["step"]) == step
         state.grad_placeholder.clear()
         state.step += 1
+    if mode == "deferred":
+        assert local.launched == 4
     sd = optimizer.state_dict()                           # the caller's optimizer object checkpoints as usual
     assert len(sd["state"]) == len(p_h)
     del replicas
