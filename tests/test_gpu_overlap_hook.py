@@ -82,11 +82,21 @@ def _layout(shapes):
 @pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("mode", ["per_bucket", "deferred", "batched"])
 def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, mode):
+    _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2))
+
+
+@pytest.mark.parametrize("mode", ["per_bucket", "batched"])
+def test_eight_vsw_threads_with_bf16_buckets(gpu, mode):
+    """The largest configuration's shape: eight VSWs with batches 64..8, bf16 buckets, AdamW."""
+    _hooks_with_optimizer(gpu, "adamw", torch.bfloat16, mode, (64, 56, 48, 40, 32, 24, 16, 8))
+
+
+def _hooks_with_optimizer(gpu, kind, gdt, mode, batches):
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
 
-    K, batches = 3, (4, 2, 2)
+    K = len(batches)
     opt = _opt_dict(kind)
     streams = [torch.cuda.Stream(gpu) for _ in range(K)]
     # K replicas of the "model": one Parameter per tensor, the same initial values
@@ -99,7 +109,7 @@ def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, mode
     # batched: complete buckets wait until 100 kB of them are ready, then go out as one planned launch
     local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=100_000 if mode == "batched" else 0,
                             stream=create_stream_for_optimizer(gpu))
-    st = H.GradientSimilarityState(None, 4, None, [], 2).attach_local(local)
+    st = H.GradientSimilarityState(None, K + K % 2, None, [], 2).attach_local(local)
     main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
     # the oracle's flat state per bucket
     p_h = [torch.cat([t.reshape(-1) for t in bucket]) for bucket in init]
