@@ -76,7 +76,7 @@ def fill_engine(eng, cfg, device, torch, seed, independent_masks=False):
             v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=device, dtype=v.dtype)))
 
 
-def build_engines(cfg, device, torch, independent_masks=False):
+def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0):
     from jabas_amd.engine import VSWFlatSync
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
     numel = sum(s.numel for s in cfg.specs)
@@ -84,7 +84,7 @@ def build_engines(cfg, device, torch, independent_masks=False):
     copies = max(1, math.ceil(ROTATE_TARGET_BYTES / ws))
     engines = []
     for c in range(copies):
-        eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device)
+        eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, n_fanout=n_fanout)
         fill_engine(eng, cfg, device, torch, 1234 + 17 * c, independent_masks)
         engines.append(eng)
     return engines, numel, copies
@@ -220,6 +220,15 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
     res["finite"] = bool(torch.isfinite(engines[0].param).all())
     del engines
     torch.cuda.empty_cache()
+    if extras and cfg.K > 1:
+        # what one weight arena shared by every VSW's model saves: the same step when each of the other K - 1
+        # replicas keeps weights of its own that the launch refreshes (4 (K - 1) more bytes written per element)
+        engines, _, _ = build_engines(cfg, device, torch, n_fanout=cfg.K - 1)
+        ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
+        fan_bytes = numel * (algorithmic_bytes_per_elem(cfg) + 4 * (cfg.K - 1))
+        res["step_with_replica_fanout"] = dict(rate(fan_bytes, ms), bytes_per_elem=fan_bytes // numel)
+        del engines
+        torch.cuda.empty_cache()
     if cfg.name == "gnmt" and extras:
         engines, _, _ = build_engines(cfg, device, torch, independent_masks=True)
         ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)

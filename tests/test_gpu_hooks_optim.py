@@ -232,8 +232,9 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
         assert plans[0] is not None and plans[1] is plans[0] and plans[2] is plans[0]
 
 
+@pytest.mark.parametrize("share", [True, False])
 @pytest.mark.parametrize("kind", ["sgd", "adamw"])
-def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind):
+def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind, share):
     from jabas_amd.train import VSWSyncTrainer
     batches = (6, 2)
     if kind == "sgd":
@@ -243,8 +244,12 @@ def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind):
         opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
                    groups=[dict(lr=1e-3, weight_decay=0.0), dict(lr=1e-3, weight_decay=0.05)])
     crit = torch.nn.MSELoss()
-    trainer = VSWSyncTrainer(gpu, batches, opt, interval=2, param_groups_func=_groups)
+    trainer = VSWSyncTrainer(gpu, batches, opt, interval=2, param_groups_func=_groups, share_weights=share)
     trainer.prepare_stream_parallel(_mlp(3), crit)
+    # one weight arena for every VSW's model, or one per VSW refreshed by the launch
+    assert len(trainer.engine.fanout) == (0 if share else 1)
+    for p, q in zip(trainer.main_model.parameters(), trainer.local_models[1].parameters()):
+        assert (p.data_ptr() == q.data_ptr()) == share and p is not q
     ref_model = _mlp(3).to(gpu)
     groups = _groups(ref_model)
     if kind == "sgd":

@@ -146,7 +146,7 @@ def test_stock_ddp_buckets_through_the_hooks(gpu, batches):
     dist.destroy_process_group()
 
 
-@pytest.mark.parametrize("mode", ["per_bucket", "batched", "deferred"])
+@pytest.mark.parametrize("mode", ["per_bucket", "batched", "deferred", "per_bucket_shared_weights"])
 @pytest.mark.parametrize("kind", ["sgd", "adamw"])
 def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     """Overlap weight-sync mode end to end with stock DDP (jabas/train/trainer.py:327-333): the optimizer
@@ -177,7 +177,9 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     p_h = [p.detach().cpu().clone().reshape(-1) for p in main.parameters()]
     s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
 
-    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=150_000 if mode == "batched" else 0)
+    share = mode.endswith("shared_weights")              # the replica's parameters become views of the main weight arena
+    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=150_000 if mode == "batched" else 0,
+                            share_weights=share)
     state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 2).attach_local(local)
     rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), main)
     prepare_overlap_optimizer_with_ddp(replicas, [state, H.VSWPeerState(local, 1)], [rec.hook, H.dummy_hook], optimizer, local)
@@ -200,6 +202,7 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
             assert torch.equal(_bits(p.grad), _bits(agg)), (step, i, "aggregate")
             assert torch.equal(_bits(p.data), _bits(p_h[i])), (step, i, "weights")
             assert torch.equal(_bits(q.data), _bits(p_h[i])), (step, i, "replica weights")
+            assert (q.data_ptr() == p.data_ptr()) == share and q is not p
             st = optimizer.state[p]
             if kind == "sgd":
                 assert torch.equal(_bits(st["momentum_buffer"]), _bits(s1_h[i])), (step, i)
