@@ -170,6 +170,7 @@ class VSWSyncTrainer:
         self.sync_step = 0
         self.accumulated = 0                      # compute() calls since the last step (IIDP's accum_step + 1 at step time)
         self.engine = None
+        self._bucket_views = {}                   # VSW index -> its bucket views, one per parameter (reduced-precision buckets)
         self._step_tensor = torch.zeros((), dtype=torch.float32)       # Adam's state['step'], shared by all parameters
         self.cos_placeholder = None
         self.grad_placeholders = [[], []]
@@ -267,6 +268,7 @@ class VSWSyncTrainer:
     def _bind_model(self, k, m, copy_weights):
         """Points replica k's parameters and gradients at its arenas."""
         eng = self.engine
+        self._bucket_views.pop(k, None)
         weights = eng.param if k == 0 or self.share_weights else eng.fanout[k - 1]
         with torch.no_grad():
             for i, p in enumerate(m.parameters()):
@@ -289,6 +291,7 @@ class VSWSyncTrainer:
             self.model_streams.append(torch.cuda.Stream(self.gpu))
         del self.local_models[new_num_models:]
         del self.model_streams[new_num_models:]
+        self._bucket_views.clear()
         for k, m in enumerate(self.local_models):
             self._bind_model(k, m, copy_weights=False)
         self.num_models = self.total_num_decoupled_workers = new_num_models
@@ -408,12 +411,19 @@ class VSWSyncTrainer:
                 loss = self.criterion(m(x), y)
                 loss.backward()
                 if self.grad_dtype != torch.float32:
-                    for i, p in enumerate(m.parameters()):
-                        view = self.engine.grad_view(k, i)
-                        if self.accumulated == 0:
-                            view.copy_(p.grad.reshape(-1))
-                        else:
-                            view.add_(p.grad.reshape(-1).to(view.dtype))
+                    # reduced-precision buckets: the fp32 gradients autograd left are rounded into VSW k's
+                    # bucket views, all tensors of the model in one multi-tensor launch
+                    params = list(m.parameters())
+                    views = self._bucket_views.get(k)
+                    if views is None:
+                        views = self._bucket_views[k] = [self.engine.grad_view(k, i).view(p.shape)
+                                                         for i, p in enumerate(params)]
+                    grads = [p.grad for p in params]
+                    if self.accumulated == 0:
+                        torch._foreach_copy_(views, grads)
+                    else:
+                        torch._foreach_add_(views, [g.to(self.grad_dtype) for g in grads])
+                    for p in params:
                         p.grad = None
                 losses.append(loss.detach())
         self.accumulated += 1
