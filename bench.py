@@ -76,7 +76,7 @@ def fill_engine(eng, cfg, device, torch, seed, independent_masks=False):
             v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=device, dtype=v.dtype)))
 
 
-def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0):
+def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0, write_aggregate=True):
     from jabas_amd.engine import VSWFlatSync
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
     numel = sum(s.numel for s in cfg.specs)
@@ -84,7 +84,8 @@ def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0):
     copies = max(1, math.ceil(ROTATE_TARGET_BYTES / ws))
     engines = []
     for c in range(copies):
-        eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, n_fanout=n_fanout)
+        eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, n_fanout=n_fanout,
+                          write_aggregate=write_aggregate)
         fill_engine(eng, cfg, device, torch, 1234 + 17 * c, independent_masks)
         engines.append(eng)
     return engines, numel, copies
@@ -227,6 +228,15 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
         fan_bytes = numel * (algorithmic_bytes_per_elem(cfg) + 4 * (cfg.K - 1))
         res["step_with_replica_fanout"] = dict(rate(fan_bytes, ms), bytes_per_elem=fan_bytes // numel)
+        del engines
+        torch.cuda.empty_cache()
+    if extras:
+        # the step as the trainer runs it: it clears the buckets right after the update, so the launch hands the
+        # aggregate to the optimizer in registers and writes it nowhere (4 bytes per element fewer)
+        engines, _, _ = build_engines(cfg, device, torch, write_aggregate=False)
+        ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
+        res["trainer_step_no_aggregate_write"] = dict(rate(bytes_per_step - 4 * numel, ms),
+                                                      bytes_per_elem=algorithmic_bytes_per_elem(cfg) - 4)
         del engines
         torch.cuda.empty_cache()
     if cfg.name == "gnmt" and extras:

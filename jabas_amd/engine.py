@@ -17,8 +17,13 @@ from .sync import SpanSpec, SyncPlan, StepScalars, aggregate, make_step_args, op
 
 class VSWFlatSync:
     def __init__(self, specs, batches, grad_dtype=torch.float32, opt=None, device="cuda", in_place=None,
-                 n_fanout=0, per_tensor_spans=False, caps=None, keep_clipped_grads=True):
+                 n_fanout=0, per_tensor_spans=False, caps=None, keep_clipped_grads=True, write_aggregate=True):
         self.K = len(batches)
+        # False: the launch hands the aggregate to the optimizer in registers and writes it nowhere (4 of the
+        # 44 bytes per element of an Adam step with four fp32 workers). For owners of the whole step who clear
+        # or overwrite the buckets right after it, as the trainer does; a comm hook has to leave the
+        # synchronised gradient in the main VSW's bucket and cannot use this. Ignored without optimizer.
+        self.write_aggregate = bool(write_aggregate) or opt is None
         # clipped steps: True leaves the clipped aggregate in the gradient arena, as clip_grad_norm_
         # leaves the clipped .grad behind; False saves that write (4 of 52 bytes per element)
         self.keep_clipped_grads = keep_clipped_grads
@@ -36,7 +41,11 @@ class VSWFlatSync:
         if in_place and grad_dtype != torch.float32:
             raise ValueError("in-place aggregation needs fp32 gradient buckets")
         self.grads = [torch.zeros(n, dtype=grad_dtype, device=self.device) for _ in range(self.K)]
-        self.agg = self.grads[0] if in_place else torch.zeros(n, dtype=torch.float32, device=self.device)
+        self.in_place = bool(in_place)
+        if in_place:
+            self.agg = self.grads[0]
+        else:                                    # an arena of its own, unless nothing will ever be written to it
+            self.agg = torch.zeros(n, dtype=torch.float32, device=self.device) if self.write_aggregate else None
         kind = opt_kind(opt)
         self.param = self.state1 = self.state2 = None
         self.fanout = []
@@ -60,7 +69,7 @@ class VSWFlatSync:
         for (off, numel, bounds, _bucket) in self.layout.spans:
             sl = slice(off, off + numel)
             spans.append(SpanSpec(
-                [g[sl] for g in self.grads], agg_out=self.agg[sl],
+                [g[sl] for g in self.grads], agg_out=self.agg[sl] if self.write_aggregate else None,
                 param=None if self.param is None else self.param[sl],
                 state1=None if self.state1 is None else self.state1[sl],
                 state2=None if self.state2 is None else self.state2[sl],
@@ -82,7 +91,7 @@ class VSWFlatSync:
         if not 1 <= new_k <= L.MAX_K:
             raise ValueError(f"number of VSWs must be in 1..{L.MAX_K}")
         n = self.layout.total
-        in_place = self.agg is self.grads[0]
+        in_place = self.in_place
         had_fanout = self._fanout_wanted
         while len(self.grads) < new_k:
             self.grads.append(torch.zeros(n, dtype=self.grad_dtype, device=self.device))
@@ -174,6 +183,8 @@ class VSWFlatSync:
         return GraphedStep(self, stats, clip_norm, accumulations)
 
     def _build_clip_plans(self):
+        if self.agg is None:                     # the clipped step passes the aggregate from its first launch to its second
+            self.agg = torch.zeros(self.layout.total, dtype=torch.float32, device=self.device)
         agg_spans, opt_spans = [], []
         for (off, numel, bounds, _bucket) in self.layout.spans:
             sl = slice(off, off + numel)

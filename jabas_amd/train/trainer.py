@@ -226,11 +226,11 @@ class VSWSyncTrainer:
                 for p in group["params"]:
                     group_of[id(p)] = gi
         specs = [ParamSpec(n, p.numel(), group_of.get(id(p), 0)) for n, p in zip(names, params)]
-        # step() clears the buckets right after the update, so a clipped step need not write the clipped
-        # aggregate back
+        # step() clears the buckets right after the update, so the launch need not write the aggregate (nor a
+        # clipped step the clipped aggregate) back
         self.engine = VSWFlatSync(specs, self.local_batch_sizes, grad_dtype=self.grad_dtype, opt=self.opt,
                                   device=self.gpu, n_fanout=0 if self.share_weights else max(1, self.num_models - 1),
-                                  keep_clipped_grads=False)
+                                  keep_clipped_grads=False, write_aggregate=False)
         if self.num_models == 1 and not self.share_weights:
             self.engine.reconfigure(self.local_batch_sizes)       # keeps the fan-out slot for later replicas
         self.local_models = [model] + [copy.deepcopy(model) for _ in range(self.num_models - 1)]

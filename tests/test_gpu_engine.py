@@ -288,3 +288,44 @@ def test_recorded_clipped_step_and_reconfigure(gpu):
     eng.reconfigure((4, 4))
     with pytest.raises(RuntimeError, match="record it again"):
         graphed.replay()
+
+
+@pytest.mark.parametrize("opt,dtype", [(SGD, torch.float32), (ADAM, torch.bfloat16)])
+def test_step_that_writes_no_aggregate(gpu, opt, dtype):
+    """``write_aggregate=False`` (the trainer's setting: it clears the buckets right after the step): weights,
+    state, replicas and statistics bit for bit those of the step that writes the aggregate; the gradient buckets
+    are left exactly as backward filled them; no aggregate arena exists until a clipped step needs one."""
+    batches = (4, 2, 2)
+    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=1, write_aggregate=False)
+    ref, _, _ = _make(gpu, batches, opt, dtype, n_fanout=1)
+    assert eng.agg is (eng.grads[0] if dtype == torch.float32 else None)
+    adam = opt["kind"] != "sgd"
+    for step in (1, 2, 3):
+        gen = torch.Generator().manual_seed(800 + step)
+        for k in range(len(batches)):
+            host["g"][k] = (torch.randn(eng.layout.total, generator=gen) * 1e-2).to(dtype)
+            eng.grads[k].copy_(host["g"][k])
+            ref.grads[k].copy_(host["g"][k])
+        rows = eng.step(stats="similarity")
+        rows_ref = ref.step(stats="similarity")
+        torch.cuda.synchronize()
+        O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"] if adam else None, step=step,
+                    first_step=(step == 1))
+        assert torch.equal(rows, rows_ref)
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            assert torch.equal(eng.param[sl].cpu().view(torch.int32), host["p"][sl].view(torch.int32)), step
+            assert torch.equal(eng.param[sl], ref.param[sl]) and torch.equal(eng.state1[sl], ref.state1[sl])
+            assert torch.equal(eng.fanout[0][sl], eng.param[sl])
+        for k in range(len(batches)):                              # every bucket as it was handed in, VSW 0's included
+            assert torch.equal(eng.grads[k].cpu().view(torch.int16 if dtype == torch.bfloat16 else torch.int32),
+                               host["g"][k].view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+    # a clipped step passes the aggregate from its first launch to its second: the arena appears then
+    for k in range(len(batches)):                                  # (the other engine's VSW 0 bucket holds its aggregate by now)
+        ref.grads[k].copy_(host["g"][k])
+    eng.step(clip_norm=0.05)
+    ref.step(clip_norm=0.05)
+    torch.cuda.synchronize()
+    assert eng.agg is not None
+    for off, cnt, _ in spans:
+        assert torch.equal(eng.param[off:off + cnt], ref.param[off:off + cnt])
