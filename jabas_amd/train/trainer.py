@@ -15,12 +15,12 @@ its own ``step()`` is never called: the fused launch does the update.
 It is not the reference's trainer: data loading, the configuration solver, elastic
 restarts and the cross-GPU all-reduce are outside this build.
 
-Memory layout (MI355X-first): the weights, their optimizer state, the aggregated gradient
-and every VSW's gradients live in flat arenas with one common bucket layout
-(``VSWFlatSync``); module parameters and their ``.grad`` are views into the arenas, so
-backward writes straight into the buckets (what ``gradient_as_bucket_view=True`` gives
-the reference) and the whole sync step is one fused launch that also refreshes the
-replicas' weights.
+Memory layout (MI355X-first): the weights, their optimizer state and every VSW's gradient
+buckets live in flat arenas with one common bucket layout (``VSWFlatSync``). The parameters
+of every VSW's model are views of ONE weight arena (no copy of the new weights to the other
+VSWs), a VSW's gradients are moved into its buckets by one multi-tensor launch per backward
+pass (no clearing of the buckets between steps), and the whole sync step is one fused launch
+that writes nothing but the weights and the optimizer state.
 """
 import copy
 
@@ -170,7 +170,8 @@ class VSWSyncTrainer:
         self.sync_step = 0
         self.accumulated = 0                      # compute() calls since the last step (IIDP's accum_step + 1 at step time)
         self.engine = None
-        self._bucket_views = {}                   # VSW index -> its bucket views, one per parameter (reduced-precision buckets)
+        self._bucket_views = {}                   # VSW index -> its bucket views, one per parameter
+        self._params = {}                         # VSW index -> the parameters of its model, in order
         self._step_tensor = torch.zeros((), dtype=torch.float32)       # Adam's state['step'], shared by all parameters
         self.cos_placeholder = None
         self.grad_placeholders = [[], []]
@@ -269,6 +270,7 @@ class VSWSyncTrainer:
         """Points replica k's parameters and gradients at its arenas."""
         eng = self.engine
         self._bucket_views.pop(k, None)
+        self._params.pop(k, None)
         weights = eng.param if k == 0 or self.share_weights else eng.fanout[k - 1]
         with torch.no_grad():
             for i, p in enumerate(m.parameters()):
@@ -276,8 +278,7 @@ class VSWSyncTrainer:
                 if copy_weights and (k == 0 or not self.share_weights):
                     view.copy_(p.data)
                 p.data = view
-                if self.grad_dtype == torch.float32:
-                    p.grad = eng.grad_view(k, i).view(p.shape)         # backward accumulates into the bucket
+                p.grad = None
 
     def _change_local_models_state(self, new_num_models, local_batch_size):
         """Adds or removes VSWs (counterpart of jabas/train/trainer.py:485-575): the engine
@@ -292,6 +293,7 @@ class VSWSyncTrainer:
         del self.local_models[new_num_models:]
         del self.model_streams[new_num_models:]
         self._bucket_views.clear()
+        self._params.clear()
         for k, m in enumerate(self.local_models):
             self._bind_model(k, m, copy_weights=False)
         self.num_models = self.total_num_decoupled_workers = new_num_models
@@ -410,21 +412,31 @@ class VSWSyncTrainer:
             with torch.cuda.stream(s):
                 loss = self.criterion(m(x), y)
                 loss.backward()
-                if self.grad_dtype != torch.float32:
-                    # reduced-precision buckets: the fp32 gradients autograd left are rounded into VSW k's
-                    # bucket views, all tensors of the model in one multi-tensor launch
-                    params = list(m.parameters())
-                    views = self._bucket_views.get(k)
-                    if views is None:
-                        views = self._bucket_views[k] = [self.engine.grad_view(k, i).view(p.shape)
-                                                         for i, p in enumerate(params)]
-                    grads = [p.grad for p in params]
+                # The gradients autograd left go into VSW k's bucket views with one multi-tensor launch (rounded
+                # there for reduced-precision buckets), and .grad is dropped again: with .grad unset autograd
+                # hands over the buffer its backward kernel wrote instead of adding it into an existing tensor
+                # with one small kernel per parameter, and the buckets need no clearing between steps (the first
+                # micro-batch of a step overwrites them). Per element and VSW that is one read and one write
+                # instead of a clearing write plus a read-modify-write.
+                params = self._params.get(k)
+                if params is None:
+                    params = self._params[k] = list(m.parameters())
+                    self._bucket_views[k] = [self.engine.grad_view(k, i).view(p.shape) for i, p in enumerate(params)]
+                views = self._bucket_views[k]
+                have = [(v, p.grad) for v, p in zip(views, params) if p.grad is not None]
+                unused = [v for v, p in zip(views, params) if p.grad is None]
+                if have:
+                    dst, src = [v for v, _ in have], [g for _, g in have]
                     if self.accumulated == 0:
-                        torch._foreach_copy_(views, grads)
+                        torch._foreach_copy_(dst, src)
+                    elif self.grad_dtype == torch.float32:
+                        torch._foreach_add_(dst, src)
                     else:
-                        torch._foreach_add_(views, [g.to(self.grad_dtype) for g in grads])
-                    for p in params:
-                        p.grad = None
+                        torch._foreach_add_(dst, [g.to(self.grad_dtype) for g in src])
+                if unused and self.accumulated == 0:       # parameters this micro-batch did not reach
+                    torch._foreach_zero_(unused)
+                for p in params:
+                    p.grad = None
                 losses.append(loss.detach())
         self.accumulated += 1
         return losses
@@ -448,9 +460,6 @@ class VSWSyncTrainer:
                 sched.step()
         if want:
             self._compute_cosine_similarity(rows)
-        if self.grad_dtype == torch.float32:            # backward accumulates into the fp32 buckets; reduced-precision
-            # buckets are overwritten by the first compute() of the next step. One multi-tensor launch for the K arenas.
-            torch._foreach_zero_(self.engine.grads[:self.num_models])
         for s in self.model_streams:
             s.wait_stream(cur)
         if want and self.controller is not None:

@@ -714,3 +714,49 @@ def test_trainer_clips_the_global_gradient_norm(gpu, max_norm):
         for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
             assert _close(p, rp, 2e-6, 1e-7), f"step {step}"
     assert clipped == (3 if max_norm < 1.0 else 0)
+
+
+def test_trainer_parameter_that_no_micro_batch_reaches(gpu):
+    """A parameter outside the graph of a step has no gradient: its bucket slot holds zeros (not what an earlier
+    step left there), so with no weight decay it stays put while the others move, across steps and across
+    accumulated micro-batches."""
+    from jabas_amd.train import VSWSyncTrainer
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            torch.manual_seed(9)
+            self.used = torch.nn.Linear(37, 10)
+            self.idle = torch.nn.Linear(37, 10)
+            self.use_idle = False
+
+        def forward(self, x):
+            return self.used(x) + (self.idle(x) if self.use_idle else 0.0)
+
+    opt = dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False, groups=[dict(lr=0.05, weight_decay=0.0)])
+    trainer = VSWSyncTrainer(gpu, (4, 4), opt, interval=1000)
+    trainer.prepare_stream_parallel(Net(), torch.nn.MSELoss())
+    main = trainer.main_model
+
+    def iteration(micro_batches):
+        for _ in range(micro_batches):
+            trainer.compute([(torch.randn(4, 37, device=gpu), torch.randn(4, 10, device=gpu)) for _ in range(2)])
+        trainer.step()
+        torch.cuda.synchronize()
+
+    for m in trainer.local_models:
+        m.use_idle = True
+    iteration(1)                                               # fills the idle layer's bucket slots with real gradients
+    for m in trainer.local_models:
+        m.use_idle = False
+    idle_before = [p.detach().clone() for p in main.idle.parameters()]
+    used_before = [p.detach().clone() for p in main.used.parameters()]
+    momentum = [trainer.engine._view(trainer.engine.state1, i).clone() for i, (n, _) in enumerate(main.named_parameters())
+                if n.startswith("idle")]
+    iteration(1)
+    iteration(2)
+    assert all(not torch.equal(p, b) for p, b in zip(main.used.parameters(), used_before))
+    # only the momentum of its one real step still moves the idle layer: p -= lr * (0.9 buf), then lr * (0.81 buf)
+    for p, b, buf in zip(main.idle.parameters(), idle_before, momentum):
+        want = b.reshape(-1) - 0.05 * (0.9 * buf) - 0.05 * (0.81 * buf)
+        assert torch.allclose(p.reshape(-1), want, rtol=1e-5, atol=1e-8)
