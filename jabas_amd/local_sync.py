@@ -72,7 +72,7 @@ class LocalBucketSync:
     """
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
-                 optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False):
+                 optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
@@ -99,6 +99,12 @@ class LocalBucketSync:
         in the backward pass, so one copy serves all: 4 (K - 1) fewer bytes written per element and step, K - 1
         fewer copies of the weights in HBM. The replicas take the main model's values when a bucket is bound.
 
+        write_aggregate=False (buckets whose launch runs the optimizer only): the aggregate goes to the update
+        in registers and is written nowhere, neither into VSW 0's fp32 bucket nor into an fp32 arena beside a
+        reduced-precision one: 4 bytes per element fewer. For callers that read no gradient after the step; the
+        default leaves the synchronised gradient in the main VSW's bucket, as the reference's hooks do. Buckets
+        under a norm bound (``grad_clip``) keep the write: their second launch reads the aggregate.
+
         opt + param_buckets: hyperparameter dictionary and, per bucket index, dict(param=, state1=,
         state2=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket; the launch of
         such a bucket also runs the optimizer. ``optimizer=`` (or ``bind_optimizer``) takes a
@@ -108,6 +114,7 @@ class LocalBucketSync:
             raise ValueError("the deferred mode drives the C ABI itself: no launcher can be injected")
         self.deferred = bool(deferred)
         self.share_weights = bool(share_weights)
+        self.write_aggregate = bool(write_aggregate)
         self.batch_bytes = 0 if deferred else int(batch_bytes)
         if self.batch_bytes and launcher is not None:
             raise ValueError("batched launches drive the C ABI themselves: no launcher can be injected")
@@ -213,7 +220,7 @@ class LocalBucketSync:
                 new["state1"] = _arena_like(buf0)
             if not sgd:
                 new["state2"] = _arena_like(buf0)
-            if buf0.dtype != torch.float32:
+            if buf0.dtype != torch.float32 and (self.write_aggregate or self.grad_clip != float("inf")):
                 new["agg_out"] = _arena_like(buf0)
             names = ("momentum_buffer",) if sgd else ("exp_avg", "exp_avg_sq")
             had_state = 0
@@ -504,6 +511,8 @@ class LocalBucketSync:
         agg_out = g0 if g0.dtype == torch.float32 else (pb or {}).get("agg_out")
         if opt is not None and self.grad_clip != float("inf") and agg_out is None:
             raise ValueError("clipping a reduced-precision bucket needs an fp32 agg_out arena")
+        if opt is not None and not self.write_aggregate and self.grad_clip == float("inf"):
+            agg_out = None
         span = sync.SpanSpec(tensors, agg_out=agg_out,
                              param=pb and pb.get("param"), state1=pb and pb.get("state1"),
                              state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
