@@ -12,7 +12,7 @@ import torch
 
 from . import _lib as L
 from .layout import FlatLayout
-from .sync import SpanSpec, SyncPlan, StepScalars, aggregate, make_step_args, opt_kind, cosine_from_stats, clip_coef
+from .sync import SpanSpec, SyncPlan, StepScalars, gradient_stats, make_step_args, opt_kind, cosine_from_stats, clip_coef
 
 
 class VSWFlatSync:
@@ -218,14 +218,16 @@ class GraphedStep:
         self.engine, self.stats, self.clip_norm, self.accumulations = engine, stats, clip_norm, accumulations
         self.scalars = StepScalars(engine.device)
         self._generation = engine._generation
-        # the first launch out of a code object loads it, which a recording stream must not do: one launch of
-        # the same K over a scratch element first
+        # the first launch out of a code object loads it, which a recording stream must not do: one statistics
+        # launch of the same K over a scratch vector first (the per-K kernels, the finalize and coefficient kernels)
         warm = [torch.zeros(4, dtype=engine.grad_dtype, device=engine.device) for _ in range(engine.K)]
-        aggregate(warm, (1,) * engine.K, out=torch.zeros(4, dtype=torch.float32, device=engine.device))
+        rows = gradient_stats(warm, (1,) * engine.K)
         if engine._clipped(clip_norm):
             if engine._plan_agg is None:
                 engine._build_clip_plans()
-            aggregate(warm[:1], (1,), out=torch.zeros(4, dtype=torch.float32, device=engine.device))
+            clip_coef(gradient_stats([torch.zeros(4, device=engine.device)], (1,)).view(1, -1), 1.0)
+        self.scalars.update(engine._update_args(stats, 1.0, clip_norm, accumulations))
+        del rows
         torch.cuda.synchronize(engine.device)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
