@@ -254,8 +254,10 @@ int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev,
  * hipMalloc) and so cannot size a workspace for whatever bucket comes next. No counterpart
  * in the reference. The partial rows of the statistics reduction go to a static device
  * array of 5.25 MB that every GPU the process uses holds until the process ends; its
- * address is looked up once per GPU, on the first call made with that GPU current (the
- * stream must belong to the current device). Calls neither allocate nor free anything.
+ * address is looked up once per GPU, on the first call with statistics made with that GPU
+ * current (the stream must belong to the current device; make that one call outside any
+ * graph capture: the lookup, like the first launch out of a code object, loads device code).
+ * Calls neither allocate nor free anything.
  * span->numel above JABAS_STATIC_MAX_NUMEL (64 Mi elements, a 256 MB fp32 bucket) is refused
  * with JABAS_ERR_SIZE before anything is launched. All calls on one GPU share that GPU's
  * array: calls with statistics that overlap in time on one GPU (different streams or
