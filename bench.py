@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused per-GPU gradient-sync step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-all] [--no-cpu] [--no-extras]
                     [--cpu-seconds S] [--calibrate-copy]
 
 A step is one fused sync step (batch-weighted aggregate of the K VSW gradient buckets
@@ -383,6 +383,9 @@ def main():
     ap.add_argument("--workload", default="vit_l16")
     ap.add_argument("--no-all", action="store_true", help="time only the headline workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="per workload only the timed steps and the instrumented launches (a kernel trace of such a "
+                         "run holds one kind of launch per kernel name and grid)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="CPU time the headline's baseline may take; the other workloads get a third each")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -414,8 +417,12 @@ def main():
     results = {}
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
     for cfg in order:
-        r = results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch)
+        r = results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch, extras=not args.no_extras)
         r["hbm_traffic_bytes_per_launch"] = measured_traffic(cfg.name)
+        if args.no_extras:
+            print(f"# {cfg.name}: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s, {r['pct_hbm_peak']:.1f} % of HBM peak",
+                  file=sys.stderr, flush=True)
+            continue
         extra = ""
         if r.get("step_without_statistics"):
             extra = (f"; without statistics {r['step_without_statistics']['ms_per_step']:.4f} ms "
@@ -426,12 +433,12 @@ def main():
               f"{r['hook_path_per_bucket_ms']['ms_per_step']:.4f} ms, batched "
               f"{r['hook_path_batched_64MiB_ms']['ms_per_step']:.4f} ms, deferred "
               f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms", file=sys.stderr, flush=True)
-    if "faster_rcnn_r50_fpn" in results:
+    if "faster_rcnn_r50_fpn" in results and not args.no_extras:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
                                                                       args.steps, torch)
     copy_gbps = copy_rate(device, args.steps, torch)
-    stat_launches = None if args.no_all else statistics_launches(device, args.steps, torch)
-    gram = None if args.no_all else gram_launches(device, args.steps, torch)
+    stat_launches = None if args.no_all or args.no_extras else statistics_launches(device, args.steps, torch)
+    gram = None if args.no_all or args.no_extras else gram_launches(device, args.steps, torch)
     head = results[head_cfg.name]
     if not args.no_cpu:
         for cfg in order:
