@@ -347,11 +347,14 @@ void jabas_rdv_destroy(JabasRendezvous* r);
 /* Describes the launch of bucket `bucket` (everything jabas_sync_bucket takes: the span with the K
  * gradient buffers the VSWs will hand over, the device bound table or NULL); stats_rows: two rows of
  * JABAS_STATS_STRIDE doubles and a workspace of jabas_sync_workspace_bytes, or NULL when the bucket
- * never takes statistics. The struct is copied; the buffers stay the caller's and must outlive the
+ * never takes statistics. last_row (0 or 1): the row the bucket's statistics were written to last,
+ * by whoever launched it before (0 when nobody did): the launches queued from here go on alternating
+ * from there, so a row handed out earlier stays untouched until the second-next statistics launch.
+ * The struct is copied; the buffers stay the caller's and must outlive the
  * description. Creates the bucket's K events on first use (the only allocation). */
 int jabas_rdv_set_bucket(JabasRendezvous* r, uint32_t bucket, const JabasSpan* span,
                          const JabasBound* bounds_dev, double* stats_rows,
-                         void* workspace, size_t workspace_bytes);
+                         void* workspace, size_t workspace_bytes, int32_t last_row);
 
 /* Forgets the description; returns how many VSWs had handed the bucket over in the running step. */
 int jabas_rdv_drop_bucket(JabasRendezvous* r, uint32_t bucket);

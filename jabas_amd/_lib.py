@@ -112,7 +112,7 @@ SIGNATURES = {
     "jabas_rdv_create": (C.c_int, [C.c_int32, C.POINTER(C.c_void_p)]),
     "jabas_rdv_destroy": (None, [C.c_void_p]),
     "jabas_rdv_set_bucket": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(JabasSpan), C.c_void_p, C.c_void_p,
-                                       C.c_void_p, C.c_size_t]),
+                                       C.c_void_p, C.c_size_t, C.c_int32]),
     "jabas_rdv_drop_bucket": (C.c_int, [C.c_void_p, C.c_uint32]),
     "jabas_rdv_publish": (C.c_int, [C.c_void_p, C.c_int32, C.c_uint32, C.c_int32, C.c_void_p, C.c_void_p,
                                     C.POINTER(JabasStepArgs), C.c_int32]),

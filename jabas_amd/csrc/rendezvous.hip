@@ -74,9 +74,9 @@ JABAS_API void jabas_rdv_destroy(JabasRendezvous* r) {
 }
 
 JABAS_API int jabas_rdv_set_bucket(JabasRendezvous* r, uint32_t bucket, const JabasSpan* span, const JabasBound* bounds_dev,
-                                   double* stats_rows, void* workspace, size_t workspace_bytes) {
+                                   double* stats_rows, void* workspace, size_t workspace_bytes, int32_t last_row) {
     if (!r || !span) return JABAS_ERR_NULL;
-    if (bucket >= kMaxBuckets) return JABAS_ERR_SIZE;
+    if (bucket >= kMaxBuckets || last_row < 0 || last_row > 1) return JABAS_ERR_SIZE;
     if (stats_rows && (!workspace || reinterpret_cast<uintptr_t>(stats_rows) % 8)) return JABAS_ERR_WORKSPACE;
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev != r->device) return JABAS_ERR_LAUNCH;   // events belong to a device
@@ -97,6 +97,7 @@ JABAS_API int jabas_rdv_set_bucket(JabasRendezvous* r, uint32_t bucket, const Ja
     b.workspace_bytes = workspace_bytes;
     b.recorded = 0;
     b.want_stats = 0;
+    b.flip = last_row;                          // the next statistics launch takes the other row
     b.set = true;
     return JABAS_OK;
 }

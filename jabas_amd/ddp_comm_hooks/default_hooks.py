@@ -46,18 +46,29 @@ def _allreduce_sum_fut(group, tensor):
 
 
 class VSWPeerState:
-    """State a non-main VSW registers with ``dummy_hook`` so that its buckets reach the
-    GPU's LocalBucketSync. The reference registers ``state=None``
-    (jabas/train/trainer.py:466-468); that still works and makes the hook a pure
-    pass-through."""
+    """State a non-main VSW may register with ``dummy_hook`` to name its meeting point and VSW index
+    itself. The reference registers ``state=None`` (jabas/train/trainer.py:466-468); ``dummy_hook`` then
+    finds both on its own."""
 
     def __init__(self, local, vsw_index):
         self.local, self.vsw_index = local, vsw_index
 
 
+def installed_local(tensor):
+    """The LocalBucketSync installed for the device ``tensor`` lives on, or None."""
+    from ..local_sync import installed
+    return installed(tensor.device if tensor.is_cuda else None)
+
+
 def dummy_hook(state, bucket):
+    """The hook of every VSW but the first (jabas/train/trainer.py:461-468, registered with ``state=None``):
+    hands the replica's bucket to the GPU's meeting point and returns at once. The meeting point is the one
+    installed for the bucket's device (``LocalBucketSync.install``), the VSW index comes from the bucket's
+    parameters (``register_replicas``) or from the stream the hook runs on. With no meeting point installed
+    (a single VSW, or plain DDP) the hook is the pass-through its name says."""
     tensor = bucket_tensor(bucket)
-    if state is None or getattr(state, "local", None) is None:
+    local = getattr(state, "local", None) if state is not None else installed_local(tensor)
+    if local is None:
         return completed(bucket_value(bucket, tensor))
-    return state.local.publish(state.vsw_index, bucket_index(bucket), tensor, value=bucket_value(bucket, tensor),
-                               bucket=bucket)
+    k = state.vsw_index if state is not None else local.vsw_of(bucket, tensor)
+    return local.publish(k, bucket_index(bucket), tensor, value=bucket_value(bucket, tensor), bucket=bucket)

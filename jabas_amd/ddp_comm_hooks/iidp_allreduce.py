@@ -7,7 +7,7 @@ In the reference the hook all-reduces the main VSW's bucket over the world and d
 publishes VSW 0's bucket to the LocalBucketSync, and the fused kernel writes the
 batch-weighted aggregate (the weights already carry the division) back into that bucket.
 """
-from .default_hooks import bucket_tensor, bucket_value, bucket_index, completed
+from .default_hooks import bucket_tensor, bucket_value, bucket_index, completed, installed_local
 
 
 class IIDPState:
@@ -18,7 +18,10 @@ class IIDPState:
         self.vsw_index = 0
 
     def attach_local(self, local):
-        """Binds the GPU's LocalBucketSync; its K must account for every local VSW."""
+        """Binds the GPU's LocalBucketSync; its K must account for every local VSW. A state nobody
+        attached (the reference builds its states without any handle to IIDP's local machinery,
+        jabas/train/trainer.py:452-458) takes the meeting point installed for the bucket's device at
+        its first hook call."""
         self.local = local
         return self
 
@@ -27,6 +30,10 @@ def iidp_allreduce_hook(state, bucket, want_stats=False, on_done=None):
     tensor = bucket_tensor(bucket)
     value = bucket_value(bucket, tensor)
     local = getattr(state, "local", None)
+    if local is None:
+        local = installed_local(tensor)
+        if local is not None:
+            state.local = local
     if local is None:
         if state.total_num_decoupled_workers != 1:
             raise RuntimeError(

@@ -22,11 +22,35 @@ to the other replicas are one launch per bucket.
 """
 import ctypes as C
 import threading
+import weakref
 
 import torch
 
 from . import sync
 from . import _lib as L
+
+# The meeting point of each device, for hooks that are registered without a state of ours: the reference
+# registers ``dummy_hook`` with ``state=None`` on every VSW but the first and builds the main VSW's state
+# without any handle to IIDP's local machinery (jabas/train/trainer.py:452-468), so both find the GPU's
+# LocalBucketSync here. Filled by ``LocalBucketSync.install`` (what stands in for IIDP's trainer calls it
+# when it builds the local models); weak references: an object nobody holds any more is not found.
+_installed = {}
+_installed_lock = threading.Lock()
+
+
+def _device_key(device):
+    if device is None:
+        return "cpu"
+    device = torch.device(device)
+    if device.type != "cuda":
+        return "cpu"
+    return device.index if device.index is not None else torch.cuda.current_device()
+
+
+def installed(device):
+    """The LocalBucketSync installed for ``device`` (a torch.device, or None for host tensors), or None."""
+    ref = _installed.get(_device_key(device))
+    return None if ref is None else ref()
 
 
 class BucketStats:
@@ -72,7 +96,8 @@ class LocalBucketSync:
     """
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
-                 optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True):
+                 optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True,
+                 launch_streams=1, auto_finish=True):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
@@ -92,6 +117,19 @@ class LocalBucketSync:
 
         stream: the stream the fused launches are queued on (the reference's dedicated optimizer
         stream, jabas/train/trainer.py:328); default: the stream VSW 0's hooks run on.
+
+        launch_streams (with ``stream=``): how many launch streams the buckets' launches alternate between
+        (bucket i goes to stream i mod launch_streams; the first is ``stream``, the others are made here at the
+        default priority). Consecutive buckets are independent of each other, so on two streams the last
+        workgroups of one bucket's launch drain while the next bucket's launch is already filling the chip,
+        instead of one launch waiting for the one before to finish to the last wave. ``finish_step`` orders the
+        VSW streams behind every one of them.
+
+        auto_finish: when the bucket objects tell which bucket is a replica's last (``GradBucket.is_last()``),
+        the hand-over that completes that bucket also ends the step (``finish_step`` with the streams the hooks
+        ran on), so a training loop that only registers the hooks needs no call of its own; a later
+        ``finish_step()`` of the same step is then a no-op (it still orders the streams it is given behind the
+        step's launches).
 
         share_weights (with ``optimizer=``): the parameters of the other VSWs' models become views of the main
         model's weight arena instead of arenas of their own that every launch refreshes. The VSWs of a GPU hold
@@ -118,7 +156,10 @@ class LocalBucketSync:
         self.batch_bytes = 0 if deferred else int(batch_bytes)
         if self.batch_bytes and launcher is not None:
             raise ValueError("batched launches drive the C ABI themselves: no launcher can be injected")
+        self._batch_bytes_asked = self.batch_bytes
+        self._bucket_bytes = {}                # batched mode: bucket index -> bytes of one VSW's buffer
         self._ready_bytes = 0
+        self._groups_fired = 0
         self._plans = {}                       # batched mode: group of buckets -> its plan
         self._stream_cache = {}
         self.stats_level = sync.stats_level(stats_level) or L.STATS_SIMILARITY
@@ -135,10 +176,19 @@ class LocalBucketSync:
         self.accumulations = 1                 # micro-batches each VSW summed into its buckets (no_sync() steps + 1)
         self.grad_clip = float("inf")          # per-bucket norm bound (ShardGNMTAdam's grad_clip)
         self._launcher = launcher or self._launch_fused
-        self._lock = threading.Lock()
+        self._lock = threading.RLock()
         self._slots = {}
         self._main_stream = None
+        self._n_launch_streams = max(1, int(launch_streams))
+        self._sync_streams = []                # the launch streams; empty: VSW 0's own stream carries the launches
         self._sync_stream = stream
+        self.auto_finish = bool(auto_finish)
+        self._step_open = False                # something was handed over since the last end of step
+        self._finishing = False                # an implied end of step is running
+        self._last_done = []                   # one event per launch stream behind the launches of the step finished last
+        self._replica_of = {}                  # id(parameter) -> VSW index (register_replicas)
+        self._stream_vsw = {}                  # raw stream -> VSW index (replicas found by the stream their hooks run on)
+        self._native_seen = {}                 # bucket index -> {k: what VSW k handed over natively in this step}
         self._calls = {}                       # bucket index -> prepared sync.BucketCall(s)
         self._args_cache = {}
         self._launch_streams = set()           # streams that carry launches of the current step
@@ -149,15 +199,89 @@ class LocalBucketSync:
         self.launched_with_opt = 0             # of them, launches that updated weights
         # Native meeting point (jabas_rdv_*): buckets that come with the same buffers step after step are
         # described to it after their first launch here; from then on a hook's hand-over is one foreign call.
-        self._native_ok = launcher is None and not self.deferred and not self.batch_bytes
+        self._own_launcher = launcher is None
         self._rdv = None
-        self._native = {}                      # bucket index -> (buffer addresses per VSW, elements, prepared call, dtype)
+        self._native = {}                      # bucket index -> (buffer addresses per VSW, elements, prepared call, dtype,
+                                               #                  ids of VSW 0's parameters in the bucket or None)
         self._native_on_done = {}
         self._native_args = {}
         self._main_ptr = None
         self.native_launches = 0               # launches queued by the native meeting point
         if optimizer is not None:
             self.bind_optimizer(optimizer)
+
+    # ------------------------------------------------------------------ launch streams
+    @property
+    def _sync_stream(self):
+        return self._sync_streams[0] if self._sync_streams else None
+
+    @_sync_stream.setter
+    def _sync_stream(self, stream):
+        if stream is None:
+            self._sync_streams = []
+            return
+        extra = [torch.cuda.Stream(stream.device) for _ in range(self._n_launch_streams - 1)]
+        self._sync_streams = [stream] + extra
+
+    def _launch_stream(self, bucket_index=0):
+        if self._sync_streams:
+            return self._sync_streams[bucket_index % len(self._sync_streams)]
+        return self._main_stream
+
+    # ------------------------------------------------------------------ who hands over what
+    def install(self, device=None):
+        """Makes this object the meeting point of ``device`` (default: the current GPU; "cpu" for host
+        tensors) for hooks registered without a state of ours: ``dummy_hook`` with ``state=None`` and a main
+        state nobody attached (the reference's own registration, jabas/train/trainer.py:452-468)."""
+        with _installed_lock:
+            _installed[_device_key("cuda" if device is None and torch.cuda.is_available() else device)] = weakref.ref(self)
+        return self
+
+    def uninstall(self):
+        with _installed_lock:
+            for key in [k for k, ref in _installed.items() if ref() is self or ref() is None]:
+                del _installed[key]
+
+    def register_replicas(self, models):
+        """models[k]: VSW k's module (or DistributedDataParallel wrapper), in VSW order: a hook that is
+        handed a bucket without a state finds the VSW index from the bucket's parameters. This is what makes
+        the assignment deterministic; without it replicas are numbered in the order their streams first show
+        up, which needs one stream per VSW and equal local batches."""
+        models = list(models)
+        if len(models) != self.K:
+            raise ValueError(f"{self.K} VSWs, {len(models)} models")
+        table = {}
+        for k, m in enumerate(models):
+            for p in m.parameters():
+                if table.setdefault(id(p), k) != k:
+                    raise ValueError("a parameter object belongs to two replicas")
+        with self._lock:
+            self._replica_of = table
+            self._stream_vsw = {}
+        return self
+
+    def vsw_of(self, bucket, tensor):
+        """VSW index of the replica a peer hook (``dummy_hook`` without a state) was called for."""
+        params = getattr(bucket, "parameters", None)
+        if self._replica_of and callable(params):
+            try:
+                return self._replica_of[id(params()[0])]
+            except (KeyError, IndexError):
+                raise RuntimeError("a bucket of a replica that register_replicas was not told about") from None
+        raw = torch._C._cuda_getCurrentStream(tensor.get_device()) if tensor.is_cuda else ("host", threading.get_ident())
+        with self._lock:
+            k = self._stream_vsw.get(raw)
+            if k is None:
+                if len(set(self.batches)) > 1:
+                    raise RuntimeError("VSWs with unequal local batches must be told apart: call register_replicas(models) "
+                                       "or register the peers with VSWPeerState(local, k)")
+                taken = set(self._stream_vsw.values())
+                free = [j for j in range(1, self.K) if j not in taken]
+                if not free:
+                    raise RuntimeError(f"more peer replicas than the {self.K - 1} this meeting point expects, or two "
+                                       "replicas on one stream: call register_replicas(models)")
+                k = self._stream_vsw[raw] = free[0]
+        return k
 
     # ------------------------------------------------------------------ optimizer binding
     def bind_optimizer(self, optimizer):
@@ -214,7 +338,7 @@ class LocalBucketSync:
                 raise ValueError(f"bucket {bucket_index} carries a parameter no group of the optimizer holds")
         order = sorted(range(len(params)), key=lambda i: offs[i])
         sgd = self.opt["kind"] == "sgd"
-        with torch.no_grad(), torch.cuda.stream(self._launch_stream()):
+        with torch.no_grad(), torch.cuda.stream(self._launch_stream(bucket_index)):
             new = dict(_key=key, param=_arena_like(buf0), fanout=[])
             if not sgd or self.opt.get("momentum", 0.0) != 0.0:
                 new["state1"] = _arena_like(buf0)
@@ -290,24 +414,30 @@ class LocalBucketSync:
         return pb.get("agg_out")
 
     # ------------------------------------------------------------------ hooks call this
-    def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None, bucket=None):
+    def publish(self, k, bucket_index, tensor, want_stats=False, on_done=None, value=None, bucket=None, _stream=None):
         """Hands VSW k's bucket ``bucket_index`` over; the fused launch for that bucket is
         queued by whichever VSW hands its bucket over last. Returns a completed Future
         carrying ``value`` (default the tensor). ``bucket``: the bucket object itself, whose
-        ``parameters()`` / ``gradients()`` place the weights when an optimizer is bound."""
+        ``parameters()`` / ``gradients()`` place the weights when an optimizer is bound and whose
+        ``is_last()`` ends the step (``auto_finish``)."""
         if not 0 <= k < self.K:
             raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
+        if self._finishing:                    # an implied end of step is running on another thread: let it finish
+            with self._lock:
+                pass
+        self._step_open = True
         fut = torch.futures.Future()
         fut.set_result(tensor if value is None else value)
         known = self._native.get(bucket_index)
-        if known is not None and tensor.is_cuda:
-            if known[0][k] == tensor.data_ptr() and known[1] == tensor.numel():
-                self._publish_native(k, bucket_index, tensor, want_stats, on_done, known)
+        if known is not None and tensor.is_cuda and _stream is None:
+            if known[0][k] == tensor.data_ptr() and known[1] == tensor.numel() and self._same_parameters(k, bucket, known):
+                if self._publish_native(k, bucket_index, tensor, want_stats, on_done, known, bucket):
+                    self._end_of_step(bucket)
                 return fut
-            self._forget_native(bucket_index, k)
+            self._leave_native(bucket_index, k)
         event = stream = None
         if tensor.is_cuda:
-            stream = self._current_stream(tensor)
+            stream = self._current_stream(tensor) if _stream is None else _stream
             if not self.deferred and not self.batch_bytes and (k != 0 or self._sync_stream is not None):
                 # VSW 0's own stream needs none when the launch is queued on it. A fresh event every time:
                 # recording one event again step after step (to save its creation) made the waits on it
@@ -330,9 +460,11 @@ class LocalBucketSync:
                 slot.want_stats, slot.on_done = want_stats, on_done
                 self._main_stream = stream
                 self._main_ptr = None if stream is None else stream.cuda_stream
-            ready = slot.count == self.K
+            complete = ready = slot.count == self.K
             if ready:
                 del self._slots[bucket_index]
+                if self._batch_bytes_asked and stream is not None:
+                    self._bucket_bytes[bucket_index] = tensor.numel() * tensor.element_size()
                 if self.deferred or (self.batch_bytes and stream is not None):
                     self._ready[bucket_index] = slot
                     self._ready_bytes += tensor.numel() * tensor.element_size()
@@ -343,7 +475,22 @@ class LocalBucketSync:
             self._fire(bucket_index, slot)
         elif batch is not None:
             self._fire_group(batch)
+        if complete:
+            self._end_of_step(bucket)
         return fut
+
+    def _end_of_step(self, bucket):
+        """Called by the hand-over that completed a bucket: when that bucket is the replicas' last one, every
+        launch of the step is queued (DDP hands a replica's buckets over in order), and the step ends here."""
+        is_last = getattr(bucket, "is_last", None)
+        if not self.auto_finish or not callable(is_last) or not is_last():
+            return
+        with self._lock:
+            self._finishing = True
+            try:
+                self.finish_step()
+            finally:
+                self._finishing = False
 
     def _current_stream(self, tensor):
         """torch.cuda.current_stream(tensor.device) without its per-call device bookkeeping (4.6 us a call,
@@ -363,7 +510,7 @@ class LocalBucketSync:
         """Describes a bucket that has just had its first launch from here to the native rendezvous."""
         dev = tensors[0].device
         lib = L.lib()
-        with torch.cuda.device(dev), torch.cuda.stream(self._launch_stream()):
+        with torch.cuda.device(dev), torch.cuda.stream(self._launch_stream(bucket_index)):
             if self._rdv is None:
                 handle = C.c_void_p()
                 L.check(lib.jabas_rdv_create(self.K, C.byref(handle)), "jabas_rdv_create")
@@ -372,26 +519,59 @@ class LocalBucketSync:
             call.prepare_stats()
             L.check(lib.jabas_rdv_set_bucket(self._rdv, bucket_index, C.byref(call.c_span),
                                              None if call.bounds_dev is None else call.bounds_dev.data_ptr(),
-                                             call._rows.data_ptr(), call.ws.buf.data_ptr(), call.ws.nbytes),
+                                             call._rows.data_ptr(), call.ws.buf.data_ptr(), call.ws.nbytes, call._flip),
                     "jabas_rdv_set_bucket")
-        self._native[bucket_index] = (tuple(t.data_ptr() for t in tensors), tensors[0].numel(), call, tensors[0].dtype)
+        # With weights behind the bucket the description is only good for the parameters it was made for, in their
+        # order: DDP's bucket rebuild can put other parameters at the old addresses, and the span's group bounds,
+        # the arenas and the replicas' views would silently belong to the old ones.
+        pb = self.param_buckets.get(bucket_index) or {}
+        sig = tuple(id(p) for p in pb["params"]) if call.with_opt and pb.get("params") is not None else None
+        self._native[bucket_index] = (tuple(t.data_ptr() for t in tensors), tensors[0].numel(), call, tensors[0].dtype, sig)
 
-    def _forget_native(self, bucket_index, k=None):
-        known = self._native.pop(bucket_index, None)
-        if known is None or self._rdv is None:
-            return
-        arrived = L.lib().jabas_rdv_drop_bucket(self._rdv, bucket_index)
-        if arrived > 0 and k is not None:
+    @staticmethod
+    def _same_parameters(k, bucket, known):
+        """Whether VSW 0's bucket still carries the parameters the native description was made for (every
+        replica rebuilds its buckets alike, so VSW 0's word covers the others)."""
+        sig = known[4]
+        if sig is None or k != 0:
+            return True
+        params = getattr(bucket, "parameters", None)
+        return callable(params) and tuple(id(p) for p in params()) == sig
+
+    def _leave_native(self, bucket_index, k):
+        """A VSW came with another buffer (or other parameters) than the native description holds: the
+        description is dropped and whoever has already handed the bucket over natively in this step is handed
+        over again on the Python path, on its own stream (an event recorded now covers everything the earlier
+        one covered)."""
+        with self._lock:
+            seen = self._native_seen.pop(bucket_index, {})
+        arrived = self._forget_native(bucket_index)
+        if arrived != len(seen):
             raise RuntimeError(f"bucket {bucket_index}: VSW {k} handed over another buffer than in the step before, "
                                f"after {arrived} other VSW(s) had handed over the same ones as before")
+        for j, (tensor, bucket, want_stats, on_done, stream) in sorted(seen.items()):
+            self.publish(j, bucket_index, tensor, want_stats=want_stats, on_done=on_done, bucket=bucket, _stream=stream)
 
-    def _publish_native(self, k, bucket_index, tensor, want_stats, on_done, known):
+    def _forget_native(self, bucket_index):
+        """Drops the native description; returns how many VSWs had handed the bucket over natively in this step."""
+        known = self._native.pop(bucket_index, None)
+        if known is None or self._rdv is None:
+            return 0
+        return max(0, L.lib().jabas_rdv_drop_bucket(self._rdv, bucket_index))
+
+    def _publish_native(self, k, bucket_index, tensor, want_stats, on_done, known, bucket=None):
+        """One hand-over at the native meeting point; True when this call completed the bucket."""
         stream, ptr = self._current_stream_and_ptr(tensor)
         self._vsw_streams[k] = stream
+        seen = self._native_seen.get(bucket_index)
+        if seen is None:
+            seen = self._native_seen.setdefault(bucket_index, {})
+        seen[k] = (tensor, bucket, want_stats, on_done, stream)
         if k == 0:
             self._main_stream, self._main_ptr = stream, ptr
             self._native_on_done[bucket_index] = on_done
-        main_ptr = self._sync_stream.cuda_stream if self._sync_stream is not None else self._main_ptr
+        launch = self._launch_stream(bucket_index)
+        main_ptr = launch.cuda_stream if self._sync_streams else self._main_ptr
         call = known[2]
         stamp = (self.step_count, self.lr_scale, self.accumulations)
         ent = self._native_args.get((known[3], call.with_opt))
@@ -400,14 +580,17 @@ class LocalBucketSync:
             ent = self._native_args[(known[3], call.with_opt)] = (stamp, args, C.byref(args))
         rc = self._rdv_publish(self._rdv, k, bucket_index, 1 if want_stats else 0, ptr, main_ptr, ent[2], self.stats_level)
         if rc == L.RDV_WAITING:
-            return
+            return False
         if rc < 0 or rc == L.RDV_UNKNOWN:
             with self._lock:
                 self._errors.append((bucket_index, L.JabasSyncError(rc if rc < 0 else L.ERR_STATE, "jabas_rdv_publish")))
-            return
+            return False
+        if rc >= L.RDV_LAUNCHED_ROW0:
+            call._flip = rc - L.RDV_LAUNCHED_ROW0          # the Python path continues the alternation from here
         row = call._rows[rc - L.RDV_LAUNCHED_ROW0] if rc >= L.RDV_LAUNCHED_ROW0 else None
         with self._lock:
-            self._launch_streams.add(self._launch_stream())
+            self._native_seen.pop(bucket_index, None)
+            self._launch_streams.add(self._launch_stream(bucket_index))
             self.launched += 1
             self.native_launches += 1
             if call.with_opt:
@@ -415,12 +598,10 @@ class LocalBucketSync:
         done = self._native_on_done.get(bucket_index)
         if done is not None:
             done(BucketStats(bucket_index, row) if row is not None else None)
-
-    def _launch_stream(self):
-        return self._sync_stream if self._sync_stream is not None else self._main_stream
+        return True
 
     def _fire(self, bucket_index, slot):
-        main = self._launch_stream()
+        main = self._launch_stream(bucket_index)
         try:
             if main is not None:
                 for ev in slot.events:
@@ -472,7 +653,7 @@ class LocalBucketSync:
         examples/gnmt/seq2seq/train/shard_optimizer.py:75-76) the bucket takes two launches: aggregate +
         statistics, the coefficient max_norm / (norm + 1e-6) on the device, then the update over the
         aggregate scaled by it: the norm has to be known before any weight moves."""
-        main = self._launch_stream()
+        main = self._launch_stream(bucket_index)
         with self._lock:
             call = self._calls.get(bucket_index)
         if call is None or not call.matches(tensors):
@@ -491,7 +672,7 @@ class LocalBucketSync:
             call.with_opt, call.clipped = with_opt, clipped
             with self._lock:
                 self._calls[bucket_index] = call
-            if self._native_ok and not clipped and main is not None:
+            if self._own_launcher and not self.deferred and not self.batch_bytes and not clipped and main is not None:
                 self._describe_native(bucket_index, tensors, call)
         if call.with_opt:
             with self._lock:
@@ -530,7 +711,8 @@ class LocalBucketSync:
             vsw_streams = sorted(self._vsw_streams.items())
         order = sorted(ready)
         slots = [ready[i] for i in order]
-        main = self._launch_stream()
+        main = self._launch_stream(0 if self.deferred else self._groups_fired)
+        self._groups_fired += 1
         if main is None:
             for i, slot in zip(order, slots):          # host tensors (protocol tests)
                 self._fire(i, slot)
@@ -602,10 +784,12 @@ class LocalBucketSync:
             self._launch_streams = set()
             self._vsw_streams = {}
             self._errors = []
+            self._step_open = False
         self._reset_native()
 
     def _reset_native(self):
         """Clears the native meeting point; returns how many of its buckets were incomplete."""
+        self._native_seen = {}
         return 0 if self._rdv is None else max(0, L.lib().jabas_rdv_reset(self._rdv))
 
     def __del__(self):
@@ -620,7 +804,14 @@ class LocalBucketSync:
         """End of a sync step: every VSW stream waits for the fused launches that read its
         buckets (and, with an optimizer bound, write its weights), and the step count (Adam's t, SGD's
         first-step flag) advances. ``streams``: the VSW streams; default: the streams the hooks of this
-        step ran on."""
+        step ran on. A step that the last bucket's hand-over has already ended (``auto_finish``) is not ended
+        twice: the call only orders ``streams`` behind that step's launches."""
+        if not self._step_open:
+            for done in self._last_done:
+                for s in streams:
+                    s.wait_event(done)
+            return
+        self._step_open = False
         left = self.pending()
         left_native = self._reset_native()
         if left or left_native:
@@ -639,12 +830,21 @@ class LocalBucketSync:
             errors, self._errors = self._errors, []
             self._args_cache_fresh = False
         streams = tuple(streams) or tuple(recorded.values())
+        self._last_done = []
         for main in launch_streams:
             done = torch.cuda.Event()
             done.record(main)
+            self._last_done.append(done)
             for s in streams:
                 if s != main:
                     s.wait_event(done)
+        if self._batch_bytes_asked and self.batch_bytes and self._bucket_bytes:
+            # Batching pays by merging several short launches into one; when a batch would hold fewer than two
+            # buckets on average it merges nothing and only holds buckets back (measured on the GNMT set, 11
+            # buckets of 58 MB on average in 64 MiB batches: 1.55 ms a step against 1.52 one launch per bucket).
+            mean = sum(self._bucket_bytes.values()) / len(self._bucket_bytes)
+            if 2 * mean > self._batch_bytes_asked:
+                self.batch_bytes = 0
         if errors:
             idx, exc = errors[0]
             self.reset()

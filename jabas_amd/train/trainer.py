@@ -51,6 +51,11 @@ def create_optimizer_hook(hook, optimizer):
     (examples/gnmt/seq2seq/train/shard_optimizer.py:41-46)."""
     def hook_then_step(state, bucket):
         local = getattr(state, "local", None)
+        if local is None:                  # a state built as the reference builds it: the device's meeting point
+            from ..ddp_comm_hooks.default_hooks import bucket_tensor, installed_local
+            local = installed_local(bucket_tensor(bucket))
+            if local is not None and state is not None:
+                state.local = local
         if local is not None:
             local.bind_optimizer(optimizer)
             return hook(state, bucket)

@@ -477,7 +477,7 @@ def test_rendezvous_calls_validate_their_arguments():
     assert lib.jabas_rdv_create(2, None) == L.ERR_NULL
     args, span = L.JabasStepArgs(), L.JabasSpan()
     assert lib.jabas_rdv_publish(None, 0, 0, 0, None, None, C.byref(args), L.STATS_SIMILARITY) == L.ERR_NULL
-    assert lib.jabas_rdv_set_bucket(None, 0, C.byref(span), None, None, None, 0) == L.ERR_NULL
+    assert lib.jabas_rdv_set_bucket(None, 0, C.byref(span), None, None, None, 0, 0) == L.ERR_NULL
     assert lib.jabas_rdv_drop_bucket(None, 0) == L.ERR_NULL
     assert lib.jabas_rdv_reset(None) == L.ERR_NULL
     lib.jabas_rdv_destroy(None)

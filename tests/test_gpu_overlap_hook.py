@@ -92,13 +92,33 @@ def test_overlap_mode_that_writes_no_aggregate(gpu, gdt):
     _hooks_with_optimizer(gpu, "adamw", gdt, "per_bucket_no_aggregate", (4, 2, 2))
 
 
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode,launch_streams", [("per_bucket", 2), ("per_bucket", 3), ("batched", 2)])
+def test_launches_alternating_between_launch_streams(gpu, kind, gdt, mode, launch_streams):
+    """Consecutive buckets' launches on alternating launch streams (they overlap on the GPU): the same bits."""
+    _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2), launch_streams=launch_streams)
+
+
+# buckets of 8, 12 and 17 MB: a bucket's launch is still running when the next bucket is handed over
+BIG_SHAPES = [[(1024, 2048), (2048,)], [(1536, 2048), (7,)], [(2048, 1024), (1024,), (1100, 2000)]]
+
+
+@pytest.mark.parametrize("gdt,launch_streams", [(torch.float32, 1), (torch.bfloat16, 2)])
+def test_multi_megabyte_buckets_through_the_native_meeting_point(gpu, gdt, launch_streams):
+    """K = 4 hook threads, buckets large enough that launches are in flight at the following hand-overs; the
+    second and third step go through the native meeting point."""
+    _hooks_with_optimizer(gpu, "adamw", gdt, "per_bucket", (48, 32, 32, 16), launch_streams=launch_streams,
+                          SHAPES=BIG_SHAPES)
+
+
 @pytest.mark.parametrize("mode", ["per_bucket", "batched"])
 def test_eight_vsw_threads_with_bf16_buckets(gpu, mode):
     """The largest configuration's shape: eight VSWs with batches 64..8, bf16 buckets, AdamW."""
     _hooks_with_optimizer(gpu, "adamw", torch.bfloat16, mode, (64, 56, 48, 40, 32, 24, 16, 8))
 
 
-def _hooks_with_optimizer(gpu, kind, gdt, mode, batches):
+def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPES=SHAPES):
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
@@ -113,11 +133,12 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches):
     layouts = [_layout(shapes) for shapes in SHAPES]
     bufs = [[torch.zeros(n, dtype=gdt, device=gpu) for _ in range(K)] for (_, _, n) in layouts]
     optimizer = _torch_optimizer(kind, [p for bucket in replicas[0] for p in bucket])
-    # batched: complete buckets wait until 100 kB of them are ready, then go out as one planned launch
+    # batched: complete buckets wait until 400 kB of them are ready, then go out as one planned launch
     keep = not mode.endswith("no_aggregate")
     mode = mode.replace("_no_aggregate", "")
-    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=100_000 if mode == "batched" else 0,
-                            stream=create_stream_for_optimizer(gpu), write_aggregate=keep)
+    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=400_000 if mode == "batched" else 0,
+                            stream=create_stream_for_optimizer(gpu), write_aggregate=keep, launch_streams=launch_streams)
+    assert len(local._sync_streams) == launch_streams
     st = H.GradientSimilarityState(None, K + K % 2, None, [], 2).attach_local(local)
     main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
     # the oracle's flat state per bucket
@@ -184,7 +205,7 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches):
                 assert _same(bufs[b][k], host[b][k])
         if want_stats:
             rows = {s.index: s.cpu() for s in st.grad_placeholder}
-            assert sorted(rows) == [0, 1, 2]
+            assert sorted(rows) == list(range(len(SHAPES)))
             for b, (_, _, n) in enumerate(layouts):
                 want = O.stats(host[b], batches)
                 tol = 1e-6 if gdt == torch.float32 else 1e-2
@@ -399,3 +420,92 @@ def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
         assert _same(flat, host)                                                # the gradient buffers are left alone
     with pytest.raises(ValueError, match="param_groups"):
         optim.ShardGNMTAdam([{"params": params[:1]}, {"params": params[1:]}], grad_clip=1.0)
+
+
+def test_batches_that_would_merge_nothing_fall_back_to_one_launch_per_bucket(gpu):
+    """``batch_bytes`` below twice the mean bucket size: a batch would hold one bucket most of the time, so after
+    the first step the buckets go out one launch each (and through the native meeting point) again."""
+    from jabas_amd.local_sync import LocalBucketSync
+    K, batches, sizes = 2, (4, 4), [60000, 50000, 70000]
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    bufs = [[torch.zeros(n, device=gpu) for _ in range(K)] for n in sizes]
+
+    def run(local, steps):
+        for step in range(steps):
+            host = [[torch.randn(n, generator=torch.Generator().manual_seed(9 * step + 3 * b + k)) * 1e-3
+                     for k in range(K)] for b, n in enumerate(sizes)]
+            for b in range(len(sizes)):
+                for k in range(K):
+                    with torch.cuda.stream(streams[k]):
+                        bufs[b][k].copy_(host[b][k].to(gpu))
+                        local.publish(k, b, bufs[b][k])
+            local.finish_step()
+            torch.cuda.synchronize()
+            for b, n in enumerate(sizes):
+                agg_h, _ = O.sync_step(host[b], batches, [(0, n, ((0, 0),))], None, None, None, None, step=1, first_step=True)
+                assert _same(bufs[b][0], agg_h), (step, b)
+
+    merging = LocalBucketSync(batches, batch_bytes=600_000)          # 240 kB a bucket: two or three per batch
+    run(merging, 3)
+    assert merging.batch_bytes == 600_000 and merging.launched < 3 * len(sizes)
+    alone = LocalBucketSync(batches, batch_bytes=300_000)            # 1.25 buckets per batch
+    run(alone, 4)
+    assert alone.batch_bytes == 0
+    assert alone.launched > 3 * len(sizes) - 3 and alone.native_launches == 2 * len(sizes)
+
+
+def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
+    """DDP's bucket rebuild can put the same parameters in another order (or other parameters) at the old buffer
+    addresses. With an optimizer bound, the native meeting point must not launch the span it was described for
+    the old order: VSW 0's bucket is checked against the parameters of the description, the arenas are laid out
+    again, and a peer that had already handed its (unchanged) buffer over natively is handed over again."""
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
+
+    K, batches = 2, (6, 2)
+    opt = _opt_dict("adamw")
+    shapes = {"vec": (4096,), "mat": (64, 64)}                      # equal sizes, different parameter groups
+    gen = torch.Generator().manual_seed(11)
+    init = {n: torch.randn(s, generator=gen) * 0.05 for n, s in shapes.items()}
+    replicas = [{n: torch.nn.Parameter(t.clone().to(gpu)) for n, t in init.items()} for _ in range(K)]
+    optimizer = _torch_optimizer("adamw", list(replicas[0].values()))
+    local = LocalBucketSync(batches, stream=create_stream_for_optimizer(gpu))
+    st = H.GradientSimilarityState(None, 2, None, [], 10 ** 9).attach_local(local)
+    main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
+    bufs = [torch.zeros(8192, device=gpu) for _ in range(K)]
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    p_h = {n: t.clone().reshape(-1) for n, t in init.items()}
+    s1_h = {n: torch.zeros(4096) for n in shapes}
+    s2_h = {n: torch.zeros(4096) for n in shapes}
+    group = {"vec": 0, "mat": 1}
+    # (order of the parameters in the bucket, who hands over first)
+    plan = [(("vec", "mat"), 0), (("vec", "mat"), 1), (("mat", "vec"), 0), (("mat", "vec"), 1), (("vec", "mat"), 1),
+            (("vec", "mat"), 0)]
+    native_before = 0
+    for step, (order, first) in enumerate(plan, start=1):
+        host = [torch.randn(8192, generator=torch.Generator().manual_seed(50 * step + k)) * 1e-3 for k in range(K)]
+        for k in ([0, 1] if first == 0 else [1, 0]):
+            with torch.cuda.stream(streams[k]):
+                bufs[k].copy_(host[k].to(gpu))
+                bucket = ParamBucket(0, bufs[k], [replicas[k][n] for n in order], [0, 4096])
+                if k == 0:
+                    main_hook(st, bucket).wait()
+                else:
+                    H.dummy_hook(H.VSWPeerState(local, k), bucket).wait()
+        local.finish_step()
+        torch.cuda.synchronize()
+        for j, n in enumerate(order):
+            sl = slice(4096 * j, 4096 * (j + 1))
+            agg = O.aggregate([host[k][sl] for k in range(K)], batches)
+            O.opt_step(opt, group[n], p_h[n], agg, s1_h[n], s2_h[n], step, step == 1)
+            assert _same(bufs[0][sl], agg), (step, n, "aggregate")
+            assert _same(replicas[0][n].data, p_h[n]), (step, n, "weights")
+            assert _same(replicas[1][n].data, p_h[n]), (step, n, "replica")
+            assert _same(optimizer.state[replicas[0][n]]["exp_avg"], s1_h[n]), (step, n)
+            assert _same(optimizer.state[replicas[0][n]]["exp_avg_sq"], s2_h[n]), (step, n)
+        # natively launched: a step whose bucket came as the step before left it
+        want_native = step >= 2 and plan[step - 2][0] == order
+        assert local.native_launches - native_before == (1 if want_native else 0), step
+        native_before = local.native_launches
+        st.step += 1

@@ -303,3 +303,133 @@ def test_shard_gnmt_adam_constructor_follows_the_reference():
         optim.ShardGNMTAdam([{"params": p[:1]}, {"params": p[1:]}], grad_clip=1.0)
     with pytest.raises(ValueError):
         optim.ShardGNMTAdam(p, betas=(0.9, 1.0))
+
+
+class DDPBucket(NewBucket):
+    """A GradBucket that also tells whether it is the replica's last one, as torch's does."""
+
+    def __init__(self, index, tensor, n_buckets, params=()):
+        super().__init__(index, tensor, params)
+        self._n = n_buckets
+
+    def is_last(self):
+        return self._i == self._n - 1
+
+
+def _reference_registration(num_models, similarity_state):
+    """The shape of the reference's own wiring (jabas/train/trainer.py:452-468): the main VSW gets the
+    similarity state and the chained hook, every other VSW ``None`` and ``dummy_hook``."""
+    main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
+    states, hooks = [], []
+    for i in range(num_models):
+        if i == 0:
+            states.append(similarity_state)
+            hooks.append(main_hook)
+        else:
+            states.append(None)
+            hooks.append(H.dummy_hook)
+    return states, hooks
+
+
+@pytest.mark.parametrize("registered", [True, False])
+def test_reference_registration_none_states_find_the_meeting_point_and_the_step_ends_itself(registered):
+    K, nb, rec = 3, 4, Recorder()
+    local = LocalBucketSync([4] * K, launcher=rec).install("cpu")
+    try:
+        # the state is built exactly as the reference builds it: nobody attaches anything to it
+        st = H.GradientSimilarityState(None, K + 1, None, [], 2)
+        states, hooks = _reference_registration(K, st)
+        assert states[1:] == [None] * (K - 1)
+        params = [[torch.nn.Parameter(torch.zeros(3)) for _ in range(nb)] for _ in range(K)]
+        if registered:
+            class Replica:
+                def __init__(self, ps):
+                    self._ps = ps
+
+                def parameters(self):
+                    return iter(self._ps)
+            local.register_replicas([Replica(ps) for ps in params])
+        steps = (1, 2, 3)
+        grads = {step: [[torch.full((3,), float(100 * step + 10 * b + k)) for k in range(K)] for b in range(nb)]
+                 for step in steps}
+        errors = []
+        go, done = threading.Barrier(K + 1), threading.Barrier(K + 1)
+
+        def vsw(k):                                        # one thread per VSW for the whole run, as IIDP has
+            for step in steps:
+                go.wait()
+                try:
+                    for b in range(nb):
+                        fut = hooks[k](states[k], DDPBucket(b, grads[step][b][k], nb, [params[k][b]]))
+                        assert fut.done()
+                except Exception as exc:                   # pragma: no cover - reported below
+                    errors.append(exc)
+                done.wait()
+        threads = [threading.Thread(target=vsw, args=(k,), daemon=True) for k in range(K)]
+        for t in threads:
+            t.start()
+        for step in steps:
+            go.wait(timeout=30)
+            done.wait(timeout=30)
+            assert not errors, errors
+            # the last bucket's last hand-over ended the step: no call from the training loop
+            assert local.step_count == step and local.pending() == []
+            local.finish_step()                            # a loop that still calls it changes nothing
+            assert local.step_count == step
+            assert len(rec.calls) == nb * step
+            for idx, seen, want in rec.calls[-nb:]:
+                assert want is (step % 2 == 0)
+                got = sorted(float(t[0]) for t in seen)
+                assert got == [float(100 * step + 10 * idx + k) for k in range(K)]
+                if registered:                             # VSW order, whatever the arrival order
+                    assert [float(t[0]) for t in seen] == got
+            assert len(st.grad_placeholder) == (nb if step % 2 == 0 else 0)
+            st.grad_placeholder.clear()
+            st.step += 1
+        for t in threads:
+            t.join(timeout=30)
+        assert st.local is local
+    finally:
+        local.uninstall()
+    t = torch.ones(3)
+    assert H.dummy_hook(None, NewBucket(0, t)).wait() is t        # nothing installed: the pass-through again
+
+
+def test_replicas_with_unequal_batches_must_be_told_apart():
+    local = LocalBucketSync([4, 2], launcher=Recorder()).install("cpu")
+    try:
+        with pytest.raises(RuntimeError, match="register_replicas"):
+            H.dummy_hook(None, NewBucket(0, torch.ones(2)))
+        with pytest.raises(ValueError):
+            local.register_replicas([torch.nn.Linear(2, 2)])
+        a, b = torch.nn.Linear(2, 2), torch.nn.Linear(2, 2)
+        local.register_replicas([a, b])
+        H.dummy_hook(None, NewBucket(0, torch.ones(6), list(b.parameters())))
+        assert local.pending() == [0]
+        with pytest.raises(RuntimeError, match="was not told about"):
+            H.dummy_hook(None, NewBucket(1, torch.ones(6), list(torch.nn.Linear(2, 2).parameters())))
+    finally:
+        local.uninstall()
+
+
+def test_more_peers_than_the_meeting_point_expects():
+    local = LocalBucketSync([1, 1], launcher=Recorder()).install("cpu")
+    try:
+        seen = []
+
+        alive = threading.Barrier(2)
+
+        def peer():
+            alive.wait()                                   # both threads exist at once: two identities
+            try:
+                H.dummy_hook(None, NewBucket(0, torch.ones(2)))
+            except RuntimeError as exc:
+                seen.append(str(exc))
+        threads = [threading.Thread(target=peer) for _ in range(2)]    # two peer threads, one peer slot
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert len(seen) == 1 and "more peer replicas" in seen[0]
+    finally:
+        local.uninstall()

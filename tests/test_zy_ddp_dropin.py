@@ -178,7 +178,7 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
 
     share = mode.endswith("shared_weights")              # the replica's parameters become views of the main weight arena
-    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=150_000 if mode == "batched" else 0,
+    local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=250_000 if mode == "batched" else 0,
                             share_weights=share)
     state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 2).attach_local(local)
     rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), main)
@@ -218,3 +218,143 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     assert len(sd["state"]) == len(p_h)
     del replicas
     dist.destroy_process_group()
+
+
+class _ReferenceWiring:
+    """The hook wiring of the reference's trainer, statement for statement (jabas/train/trainer.py:327-337 and
+    452-468), over the attributes it reads there. What the reference reaches in its base class (IIDP's trainer,
+    not part of the JABAS repository) is the three methods at the bottom."""
+
+    def __init__(self, local_models, main_optimizer, interval, local):
+        self.local_models, self.main_optimizer, self.local = local_models, main_optimizer, local
+        self.num_models = self.total_num_decoupled_workers = len(local_models)
+        self.interval = interval
+
+    def _prepare_similarity_allreduce_hooks(self):
+        from jabas_amd import ddp_comm_hooks as H
+        self.states, self.hooks = [], []
+        self.similarity_state = H.GradientSimilarityState(
+            dist.group.WORLD, self.total_num_decoupled_workers, None, [], self.interval)
+        subgroup_allreduce_hook = H.subgroup_allreduce_hook
+        main_hook = H.similimarity_allreduce_hook(subgroup_allreduce_hook)
+        dummy_hook = H.dummy_hook
+        for i in range(self.num_models):
+            if i == 0:
+                self.states.append(self.similarity_state)
+                self.hooks.append(main_hook)
+            else:
+                self.states.append(None)
+                self.hooks.append(dummy_hook)
+
+    def _register_comm_hook(self):
+        for _, (local_model, state, hook) in enumerate(zip(self.local_models, self.states, self.hooks)):
+            local_model.register_comm_hook(state=state, hook=hook)
+
+    def _prepare_overlap_optimizer_with_ddp(self):
+        self._create_stream_for_optimizer()
+        self._check_overlap_with_ddp()
+        for i, (local_model, state, hook) in enumerate(zip(self.local_models, self.states, self.hooks)):
+            if i == 0:
+                hook = self._create_optimizer_hook(hook)
+            local_model.register_comm_hook(state=state, hook=hook)
+
+    # ---- IIDP's side
+    def _create_stream_for_optimizer(self):
+        from jabas_amd.train import create_stream_for_optimizer
+        self.local._sync_stream = create_stream_for_optimizer(next(self.local_models[0].parameters()).device)
+
+    def _check_overlap_with_ddp(self):
+        assert all(m.gradient_as_bucket_view for m in self.local_models)
+
+    def _create_optimizer_hook(self, hook):
+        from jabas_amd.train import create_optimizer_hook
+        return create_optimizer_hook(hook, self.main_optimizer)
+
+
+@pytest.mark.parametrize("batches,registered,overlap", [((4, 4), False, False), ((6, 2, 4, 4), True, False),
+                                                        ((3, 3, 3, 3), False, True), ((6, 2), True, True)])
+def test_the_references_own_registration_block_with_none_states(gpu, batches, registered, overlap):
+    """Nothing of ours is handed to the hooks: the main state is built as the reference builds it, the peers
+    register ``dummy_hook`` with ``state=None``, and the training loop calls neither ``attach_local`` nor
+    ``finish_step``. The meeting point is found through the device (``install``, IIDP's side of the set-up),
+    the VSW index through the bucket's parameters (``register_replicas``) or the hook's stream, the step ends
+    with the last bucket. Aggregate (sequential mode) or weights and optimizer state (overlap mode) bit-exact
+    against the oracle over four steps, across DDP's bucket rebuild."""
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+
+    _init_pg()
+    K = len(batches)
+    crit = torch.nn.MSELoss()
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    replicas = _replicas(gpu, K, streams)
+    main = replicas[0].module
+    groups = [{"params": [p for p in main.parameters() if p.dim() <= 1], "weight_decay": 0.0},
+              {"params": [p for p in main.parameters() if p.dim() > 1], "weight_decay": 0.05}]
+    optimizer = torch.optim.AdamW(groups, lr=1e-3)
+    opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+               groups=[dict(lr=1e-3, weight_decay=0.0), dict(lr=1e-3, weight_decay=0.05)])
+    group_of = [0 if p.dim() <= 1 else 1 for p in main.parameters()]
+    p_h = [p.detach().cpu().clone().reshape(-1) for p in main.parameters()]
+    s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
+
+    # IIDP's side of the set-up: the GPU's meeting point exists and knows the device (and, when told, the replicas)
+    local = LocalBucketSync(batches, launch_streams=2).install(gpu)
+    if registered:
+        local.register_replicas(replicas)
+    try:
+        wiring = _ReferenceWiring(replicas, optimizer, 2, local)
+        wiring._prepare_similarity_allreduce_hooks()
+        assert wiring.states[1:] == [None] * (K - 1) and wiring.similarity_state.local is None
+        rec = Recorder(wiring.hooks[0], main)              # the test's own tap on VSW 0's bucket, for the oracle
+        wiring.hooks[0] = rec.hook
+        if overlap:
+            wiring._prepare_overlap_optimizer_with_ddp()
+        else:
+            wiring._register_comm_hook()
+        state = wiring.similarity_state
+        for step in range(1, 5):
+            gen = torch.Generator().manual_seed(70 + step)
+            data = [(torch.randn(b, 64, generator=gen).to(gpu), torch.randn(b, 16, generator=gen).to(gpu)) for b in batches]
+            rec.seen.clear()
+            _backward_all(replicas, streams, data, crit)
+            assert local.step_count == step                # ended by the last bucket's last hand-over
+            torch.cuda.synchronize()
+            # which replica the meeting point took for which VSW index
+            if registered:
+                vsw_of = list(range(K))
+            else:
+                by_stream = {(s.stream_id, s.device_index, s.device_type): j for j, s in enumerate(streams)}
+                vsw_of = [0] + [None] * (K - 1)
+                for raw, k in local._stream_vsw.items():
+                    vsw_of[k] = by_stream[raw]
+                assert sorted(vsw_of) == list(range(K))
+            per_rep = _per_parameter_grads(rec, replicas)
+            per_vsw = [per_rep[j] for j in vsw_of]
+            for i, p in enumerate(main.parameters()):
+                agg = O.aggregate([per_vsw[k][i] for k in range(K)], batches)
+                assert torch.equal(_bits(p.grad), _bits(agg)), (step, i, "aggregate")
+                if overlap:
+                    O.opt_step(opt, group_of[i], p_h[i], agg, s1_h[i], s2_h[i], step, step == 1)
+                    assert torch.equal(_bits(p.data), _bits(p_h[i])), (step, i, "weights")
+                    for r in replicas[1:]:
+                        assert torch.equal(_bits(list(r.module.parameters())[i].data), _bits(p_h[i])), (step, i, "replica")
+                    assert torch.equal(_bits(optimizer.state[p]["exp_avg"]), _bits(s1_h[i])), (step, i)
+                    assert torch.equal(_bits(optimizer.state[p]["exp_avg_sq"]), _bits(s2_h[i])), (step, i)
+            if state.step % state.interval == 0:
+                halves = []
+                for h in (0, 1):
+                    ks = [k for k in range(K) if k % 2 == h]
+                    tot = float(sum(batches[k] for k in ks))
+                    halves.append(sum(torch.cat(per_vsw[k]).double() * (batches[k] / tot) for k in ks))
+                want_cos = torch.nn.functional.cosine_similarity(halves[0], halves[1], dim=0).item()
+                assert H.cosine_similarity_from_placeholder(state.grad_placeholder) == pytest.approx(want_cos, rel=1e-6, abs=1e-9)
+            else:
+                assert state.grad_placeholder == []
+            state.grad_placeholder = []                    # jabas/train/trainer.py:480
+            state.step += 1
+        assert state.local is local and len(local._sync_streams) == (2 if overlap else 0)
+    finally:
+        local.uninstall()
+        del replicas
+        dist.destroy_process_group()
