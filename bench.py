@@ -125,7 +125,7 @@ class _Bucket:
         return self._t
 
 
-def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0):
+def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0, launch_streams=1):
     """The same step as the reference's calling convention reaches it: per bucket, VSW 0's similarity
     hook (with the optimizer bound: the overlap weight-sync mode) and K - 1 dummy hooks, each handing
     over its bucket view; one fused launch per bucket (or one per step, deferred) on a launch stream
@@ -141,7 +141,7 @@ def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0):
                       agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
     stream = torch.cuda.Stream(device)
     local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, deferred=deferred, stream=stream,
-                            batch_bytes=batch_bytes)
+                            batch_bytes=batch_bytes, launch_streams=launch_streams)
     local.step_count = eng.step_count
     local._momentum_ready = eng.step_count > 0
     state = H.GradientSimilarityState(None, cfg.K + cfg.K % 2, None, [], 1 if cfg.stats else 10 ** 9).attach_local(local)
@@ -163,7 +163,156 @@ def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0):
     launched_before = local.launched
     ms, wall = timed_region(one_step, steps, 0, torch)
     eng.step_count = local.step_count
-    return dict(ms_per_step=ms, wall_ms_per_step=wall, launches_per_step=(local.launched - launched_before) / steps)
+    return dict(ms_per_step=ms, wall_ms_per_step=wall, launches_per_step=(local.launched - launched_before) / steps,
+                host_us_per_hook_call=1e3 * wall / (cfg.K * len(buckets)), launch_streams=launch_streams)
+
+
+def bucket_launches(cfg, eng, device, steps, warmup, torch, launch_streams):
+    """One jabas_sync_bucket launch per bucket of the gradient set (what the per-bucket hook mode queues), with no
+    hand-over events in between, bucket i on launch stream i mod launch_streams: what the GPU needs for the
+    launches themselves. ms per step, HIP events on the current stream around the steps (which waits for the
+    launch streams at the end of every step)."""
+    from jabas_amd import sync
+    calls = []
+    for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
+        sl = slice(off, off + numel)
+        calls.append(sync.BucketCall(sync.SpanSpec(
+            [g[sl] for g in eng.grads], agg_out=eng.agg[sl], param=eng.param[sl],
+            state1=None if eng.state1 is None else eng.state1[sl],
+            state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds)))
+    streams = [torch.cuda.Stream(device) for _ in range(launch_streams)]
+    cur = torch.cuda.current_stream(device)
+    level = "similarity" if cfg.stats else False
+
+    def one_step(_):
+        args = eng.step_args(stats=level)
+        for s in streams:
+            s.wait_stream(cur)
+        for b, call in enumerate(calls):
+            call.run(args, stream=streams[b % launch_streams])
+        for s in streams:
+            cur.wait_stream(s)
+        eng.step_count += 1
+
+    return timed_region(one_step, steps, warmup, torch)[0]
+
+
+_sleep_cycles_per_us = None
+
+
+def sleep_cycles_per_us(torch):
+    """Cycles of torch.cuda._sleep per microsecond on this box (one wave spinning on the clock: a stand-in
+    for backward work that takes time on a stream without touching HBM)."""
+    global _sleep_cycles_per_us
+    if _sleep_cycles_per_us is None:
+        torch.cuda._sleep(1000)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = 2_000_000
+        a.record()
+        torch.cuda._sleep(n)
+        b.record()
+        torch.cuda.synchronize()
+        _sleep_cycles_per_us = n / (a.elapsed_time(b) * 1e3)
+    return _sleep_cycles_per_us
+
+
+def hook_path_threads(cfg, eng, device, steps, warmup, torch, launch_streams, backward_factor=3.0, engine_ms=None):
+    """The hook path as training runs it (jabas/train/trainer.py:327-337, 452-468, 494-514): K host threads on K
+    streams, one per VSW; ahead of every bucket each VSW's stream carries a stand-in for the backward work
+    that produces the bucket (a one-wave spin of backward_factor x the bucket's share of the engine step, so
+    the K backward passes of a step take backward_factor x the sync step and leave HBM to the sync launches),
+    then the VSW's hook is called: VSW 0's similarity hook with the optimizer bound, dummy_hook on the others.
+    One fused launch per bucket, alternating between `launch_streams` launch streams.
+    Reported: ms per step (HIP events from the release of the VSW streams to the end of finish_step),
+    exposed_sync_ms = end of step - the moment the last VSW's stream passed its last hand-over (what the sync
+    adds to a step after backward is over), host_us_per_hook_call (wall time inside the hook calls, per call,
+    measured in the calling threads: includes waiting for the interpreter lock)."""
+    import threading
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    K = cfg.K
+    pbs, bucket_slices = {}, []
+    for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
+        sl = slice(off, off + numel)
+        bucket_slices.append(sl)
+        pbs[b] = dict(param=eng.param[sl], state1=None if eng.state1 is None else eng.state1[sl],
+                      state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds,
+                      agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
+    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, stream=torch.cuda.Stream(device),
+                            launch_streams=launch_streams)
+    local.step_count = eng.step_count
+    local._momentum_ready = eng.step_count > 0
+    state = H.GradientSimilarityState(None, K + K % 2, None, [], 1 if cfg.stats else 10 ** 9).attach_local(local)
+    main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
+    peers = [None] + [H.VSWPeerState(local, k) for k in range(1, K)]
+    buckets = [[_Bucket(b, eng.grads[k][sl]) for k in range(K)] for b, sl in enumerate(bucket_slices)]
+    total = sum(sl.stop - sl.start for sl in bucket_slices)
+    per_us = sleep_cycles_per_us(torch)
+    spin = [int(backward_factor * engine_ms * 1e3 * (sl.stop - sl.start) / total * per_us) for sl in bucket_slices]
+    streams = [torch.cuda.Stream(device) for _ in range(K)]
+    cur = torch.cuda.current_stream(device)
+    n_iter = warmup + steps
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(n_iter)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(n_iter)]
+    lasts = [[torch.cuda.Event(enable_timing=True) for _ in range(K)] for _ in range(n_iter)]
+    go, done = threading.Barrier(K + 1), threading.Barrier(K + 1)
+    host_s, errors = [0.0] * K, []
+
+    def vsw(k):
+        torch.cuda.set_device(device)
+        hook, st = (main_hook, state) if k == 0 else (H.dummy_hook, peers[k])
+        try:
+            with torch.cuda.stream(streams[k]):
+                for it in range(n_iter):
+                    go.wait()
+                    streams[k].wait_event(starts[it])
+                    spent = 0.0
+                    for b, per_vsw in enumerate(buckets):
+                        torch.cuda._sleep(spin[b])
+                        t0 = time.perf_counter()
+                        hook(st, per_vsw[k])
+                        spent += time.perf_counter() - t0
+                    lasts[it][k].record(streams[k])
+                    if it >= warmup:
+                        host_s[k] += spent
+                    done.wait()
+        except Exception as exc:                    # pragma: no cover - reported below
+            errors.append(exc)
+            go.abort()
+            done.abort()
+
+    threads = [threading.Thread(target=vsw, args=(k,), daemon=True) for k in range(K)]
+    for t in threads:
+        t.start()
+    wall0 = 0.0
+    try:
+        for it in range(n_iter):
+            if it == warmup:
+                torch.cuda.synchronize()
+                wall0 = time.perf_counter()
+            starts[it].record(cur)
+            go.wait(timeout=120)
+            done.wait(timeout=120)
+            local.finish_step((cur,))
+            ends[it].record(cur)
+            state.grad_placeholder.clear()
+    except threading.BrokenBarrierError:
+        raise RuntimeError(f"hook threads failed: {errors}")
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - wall0) * 1e3 / steps
+    for t in threads:
+        t.join(timeout=30)
+    ms = [starts[it].elapsed_time(ends[it]) for it in range(warmup, n_iter)]
+    exposed = [min(lasts[it][k].elapsed_time(ends[it]) for k in range(K)) for it in range(warmup, n_iter)]
+    backward = [max(starts[it].elapsed_time(lasts[it][k]) for k in range(K)) for it in range(warmup, n_iter)]
+    eng.step_count = local.step_count
+    calls = steps * K * len(buckets)
+    return dict(ms_per_step=sum(ms) / len(ms), exposed_sync_ms=sum(exposed) / len(exposed),
+                exposed_sync_ms_max=max(exposed), backward_stand_in_ms=sum(backward) / len(backward),
+                wall_ms_per_step=wall_ms, host_us_per_hook_call=1e6 * sum(host_s) / calls,
+                hook_calls_per_step=K * len(buckets), launch_streams=launch_streams,
+                backward_factor=backward_factor, native_launches=local.native_launches)
 
 
 def time_config(cfg, device, steps, warmup, torch, extras=True):
@@ -208,6 +357,15 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         res["hook_path_per_bucket_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False)
         res["hook_path_batched_64MiB_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False, 64 << 20)
         res["hook_path_deferred_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, True)
+        res["hook_path_per_bucket_2_streams_ms"] = hook_path(cfg, engines[0], device, hsteps, hwarm, torch, False,
+                                                             launch_streams=2)
+        # the GPU's share of the per-bucket mode: one launch per bucket, back to back, on 1, 2 and 3 launch streams
+        res["bucket_launches_back_to_back_ms"] = {
+            str(ls): bucket_launches(cfg, engines[0], device, hsteps, hwarm, torch, ls) for ls in (1, 2, 3)}
+        # the same hooks as training calls them: K threads on K streams with backward-like work between the buckets
+        for ls in (1, 2):
+            res[f"hook_path_threads_{ls}_launch_stream{'s' if ls > 1 else ''}"] = hook_path_threads(
+                cfg, engines[0], device, hsteps, max(3, hwarm // 3), torch, ls, engine_ms=ms_per_step)
     if cfg.name == "gnmt" and extras:
         # global-norm clipping (examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
         # coefficient on the device, then the update over the scaled aggregate
@@ -388,6 +546,9 @@ def main():
                          "run holds one kind of launch per kernel name and grid)")
     ap.add_argument("--cpu-seconds", type=float, default=20.0,
                     help="CPU time the headline's baseline may take; the other workloads get a third each")
+    ap.add_argument("--bucket-launches", type=int, default=0, metavar="S",
+                    help="run only this: the headline workload's gradient set as one launch per bucket, bucket i on "
+                         "launch stream i mod S, --steps steps after --warmup (for a kernel trace of the launches)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB copy 5 times before anything else (the K=1, weight-1 aggregate: "
                          "same 16-byte nontemporal loads and stores as the fused kernel, known traffic) for "
@@ -414,6 +575,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         torch.cuda.empty_cache()
+    if args.bucket_launches:
+        engines, numel, _ = build_engines(head_cfg, device, torch)
+        ms = bucket_launches(head_cfg, engines[0], device, args.steps, args.warmup, torch, args.bucket_launches)
+        print(json.dumps(dict(workload=head_cfg.name, launch_streams=args.bucket_launches, steps=args.steps,
+                              buckets=engines[0].plan.n_span, **rate(numel * algorithmic_bytes_per_elem(head_cfg), ms))))
+        return
     results = {}
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
     for cfg in order:

@@ -97,7 +97,7 @@ class LocalBucketSync:
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
                  optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True,
-                 launch_streams=1, auto_finish=True):
+                 launch_streams=2, auto_finish=True):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
@@ -122,8 +122,10 @@ class LocalBucketSync:
         (bucket i goes to stream i mod launch_streams; the first is ``stream``, the others are made here at the
         default priority). Consecutive buckets are independent of each other, so on two streams the last
         workgroups of one bucket's launch drain while the next bucket's launch is already filling the chip,
-        instead of one launch waiting for the one before to finish to the last wave. ``finish_step`` orders the
-        VSW streams behind every one of them.
+        instead of one launch waiting for the one before to finish to the last wave (measured on the ViT-L/16 set,
+        38 buckets: 2.61 ms a step on one stream, 6 us of idle queue between launches, 2.37 ms on two, which is
+        what one launch over all buckets takes; a third stream gains nothing). ``finish_step`` orders the VSW
+        streams behind every one of them.
 
         auto_finish: when the bucket objects tell which bucket is a replica's last (``GradBucket.is_last()``),
         the hand-over that completes that bucket also ends the step (``finish_step`` with the streams the hooks
