@@ -65,7 +65,12 @@ typedef enum JabasStatus {
 } JabasStatus;
 
 enum { JABAS_F32 = 0, JABAS_BF16 = 1 };
-enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAMW = 3 };
+/* ..._AMSGRAD: Adam / AdamW with amsgrad=True (torch 1.8.1 _functional.adam: max_exp_avg_sq =
+ * max(max_exp_avg_sq, exp_avg_sq), the denominator formed from the maximum), as
+ * examples/gnmt/seq2seq/train/shard_optimizer.py:58-66,79-90 threads it into F.adam; the span
+ * carries the maximum in state3. */
+enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAMW = 3,
+       JABAS_OPT_ADAM_AMSGRAD = 4, JABAS_OPT_ADAMW_AMSGRAD = 5 };
 /* Statistics level of a launch (JabasStepArgs.stats). SIMILARITY: the four sums the cosine
  * similarity between the halves and global-norm clipping read (slots DOT_AB .. NORM_AGG of a
  * row; the per-VSW slots are written as 0): the reference's adaptive batching consumes nothing
@@ -96,7 +101,7 @@ enum {
  * element grid at that 256-byte line and moves whole cache lines; spans that start at arbitrary
  * elements lose 8-17 % of the rate without it.
  * agg_out may be exactly one of the fp32 gradient buffers (in-place bucket update); apart
- * from that every written buffer (agg_out, param, state1, state2, fanout) must be disjoint
+ * from that every written buffer (agg_out, param, state1, state2, state3, fanout) must be disjoint
  * from every other buffer of the span, else JABAS_ERR_ALIAS. Overlap between different
  * spans of one plan is the caller's responsibility. Unused pointers are NULL. */
 typedef struct JabasSpan {
@@ -105,6 +110,7 @@ typedef struct JabasSpan {
     float*      param;                  /* fp32 weights (optimizer kinds other than NONE) */
     float*      state1;                 /* SGD momentum buffer / Adam exp_avg          */
     float*      state2;                 /* Adam exp_avg_sq                             */
+    float*      state3;                 /* Adam max_exp_avg_sq (the ..._AMSGRAD kinds only) */
     float*      fanout[JABAS_MAX_K - 1];/* replicas that receive the updated weights   */
     uint64_t    numel;
     uint32_t    n_fanout;
@@ -154,7 +160,7 @@ typedef struct JabasStepArgs {
                                            groups' lr, weight_decay and step from the block as it is
                                            when the kernel runs, not from this struct (which must
                                            still be filled in: it is what the call is checked
-                                           against). Optimizer kinds other than NONE only.      */
+                                           against). SGD, ADAM and ADAMW only.                  */
 } JabasStepArgs;
 
 /* Library identification. No reference counterpart. */
@@ -315,10 +321,12 @@ int jabas_sgd(const float* grad, float* param, float* momentum_buf, uint64_t num
 
 /* Adam (adamw == 0) / AdamW (adamw != 0) step with a ready fp32 gradient
  * (torch 1.8.1 optim/_functional.adam / adamw as called by
- * examples/gnmt/seq2seq/train/shard_optimizer.py:78-90, examples/vit/main.py:425-437). */
+ * examples/gnmt/seq2seq/train/shard_optimizer.py:78-90, examples/vit/main.py:425-437).
+ * max_exp_avg_sq: NULL, or the running maximum of the second moment (amsgrad=True). */
 int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq,
-               uint64_t numel, double lr, double weight_decay, double beta1, double beta2,
-               double eps, int64_t step, int32_t adamw, jabas_stream_t stream);
+               float* max_exp_avg_sq, uint64_t numel, double lr, double weight_decay,
+               double beta1, double beta2, double eps, int64_t step, int32_t adamw,
+               jabas_stream_t stream);
 
 /* ---- Rendezvous of the K VSW comm hooks of one GPU --------------------------------------------
  * In IIDP each VSW has its own DDP reducer, thread and stream, only VSW 0's hook communicates and

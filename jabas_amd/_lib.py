@@ -20,7 +20,7 @@ STATIC_MAX_NUMEL = 1 << 26
 STEP_SCALARS_BYTES = 688
 
 F32, BF16 = 0, 1
-OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW = 0, 1, 2, 3
+OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW, OPT_ADAM_AMSGRAD, OPT_ADAMW_AMSGRAD = 0, 1, 2, 3, 4, 5
 STATS_NONE, STATS_FULL, STATS_SIMILARITY = 0, 1, 2
 
 STAT_DOT_AB, STAT_NORM_A, STAT_NORM_B, STAT_NORM_AGG, STAT_NORM_VSW0 = 0, 1, 2, 3, 4
@@ -38,6 +38,7 @@ class JabasSpan(C.Structure):
         ("param", C.c_void_p),
         ("state1", C.c_void_p),
         ("state2", C.c_void_p),
+        ("state3", C.c_void_p),
         ("fanout", C.c_void_p * (MAX_K - 1)),
         ("numel", C.c_uint64),
         ("n_fanout", C.c_uint32),
@@ -106,7 +107,7 @@ SIGNATURES = {
     "jabas_clip_coef": (C.c_int, [C.c_void_p, C.c_uint32, C.c_double, C.c_double, C.c_void_p, C.c_void_p]),
     "jabas_sgd": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double, C.c_double,
                             C.c_double, C.c_double, C.c_int32, C.c_int32, C.c_void_p]),
-    "jabas_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double,
+    "jabas_adam": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint64, C.c_double,
                              C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64, C.c_int32,
                              C.c_void_p]),
     "jabas_rdv_create": (C.c_int, [C.c_int32, C.POINTER(C.c_void_p)]),

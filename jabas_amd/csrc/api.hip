@@ -56,6 +56,8 @@ inline int opt_class_of(int kind) {
         case JABAS_OPT_SGD: return 1;
         case JABAS_OPT_ADAM:
         case JABAS_OPT_ADAMW: return 2;
+        case JABAS_OPT_ADAM_AMSGRAD:
+        case JABAS_OPT_ADAMW_AMSGRAD: return 3;
         default: return -1;
     }
 }
@@ -93,7 +95,8 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     const int oc = opt_class_of(opt_kind);
     if (oc < 0) return JABAS_ERR_OPT;
     if (oc != 0 && !in.param) return JABAS_ERR_NULL;
-    if (oc == 2 && (!in.state1 || !in.state2)) return JABAS_ERR_NULL;
+    if (oc >= 2 && (!in.state1 || !in.state2)) return JABAS_ERR_NULL;
+    if (oc == 3 && !in.state3) return JABAS_ERR_NULL;
     if (oc == 0 && in.n_fanout) return JABAS_ERR_OPT;
     for (uint32_t r = 0; r < in.n_fanout; ++r)
         if (!in.fanout[r]) return JABAS_ERR_NULL;
@@ -112,6 +115,7 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
         same_wide(in.param, 4);
         same_wide(in.state1, 4);
         same_wide(in.state2, 4);
+        if (oc == 3) same_wide(in.state3, 4);
         for (uint32_t r = 0; r < in.n_fanout; ++r) same_wide(in.fanout[r], 4);
     }
     // elements before the line the grid starts at
@@ -136,6 +140,7 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     if (oc != 0) {
         if (!rebase_f(in.param, &out->p) || !rebase_f(in.state1, &out->s1) || !rebase_f(in.state2, &out->s2))
             return JABAS_ERR_ALIGN;
+        if (oc == 3 && !rebase_f(in.state3, &out->s3)) return JABAS_ERR_ALIGN;
         for (uint32_t r = 0; r < in.n_fanout; ++r)
             if (!rebase_f(in.fanout[r], &out->fan[r])) return JABAS_ERR_ALIGN;
         out->n_fan = in.n_fanout;
@@ -150,13 +155,14 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     // Every buffer the launch writes must be disjoint from every other buffer of the span (the
     // in-place aggregate above is the one exception): each element is read and written by a
     // different thread at a different time, so any overlap would be a silent race.
-    const void* written[4 + JABAS_MAX_K - 1];
+    const void* written[5 + JABAS_MAX_K - 1];
     int nw = 0;
     if (in.agg_out) written[nw++] = in.agg_out;
     if (oc != 0) {
         written[nw++] = in.param;
         if (in.state1) written[nw++] = in.state1;
-        if (oc == 2) written[nw++] = in.state2;
+        if (oc >= 2) written[nw++] = in.state2;
+        if (oc == 3) written[nw++] = in.state3;
         for (uint32_t r = 0; r < in.n_fanout; ++r) written[nw++] = in.fanout[r];
     }
     const size_t fb = in.numel * 4;
@@ -222,7 +228,7 @@ int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
     o.has_momentum = (oc == 1 && s->momentum != 0.0) ? 1 : 0;
     o.first_step = s->first_step ? 1 : 0;
     o.nesterov = s->nesterov ? 1 : 0;
-    o.adamw = s->opt_kind == JABAS_OPT_ADAMW ? 1 : 0;
+    o.adamw = (s->opt_kind == JABAS_OPT_ADAMW || s->opt_kind == JABAS_OPT_ADAMW_AMSGRAD) ? 1 : 0;
     if (oc == 1 && o.nesterov && (s->momentum <= 0.0 || s->dampening != 0.0)) return JABAS_ERR_OPT;
     for (int i = 0; i < s->n_groups; ++i) {
         const JabasGroup& g = s->groups[i];
@@ -232,7 +238,7 @@ int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
         d.decay = static_cast<float>(1.0 - g.lr * g.weight_decay);
         d.neg_step_size = 0.0f;
         d.sqrt_bc2 = 1.0f;
-        if (oc == 2) {
+        if (oc >= 2) {
             if (g.step < 1) return JABAS_ERR_OPT;
             const double bc1 = 1.0 - pow(s->beta1, static_cast<double>(g.step));
             const double bc2 = 1.0 - pow(s->beta2, static_cast<double>(g.step));
@@ -257,7 +263,9 @@ int fill_kargs(const JabasStepArgs* s, KArgs* a) {
     memcpy(a->groups, sc.groups, sizeof(sc.groups));
     a->grad_scale = s->grad_scale;
     if (s->scalars_dev) {
-        if (opt_class_of(s->opt_kind) == 0) return JABAS_ERR_OPT;      // nothing of an aggregate-only launch moves between steps
+        const int oc = opt_class_of(s->opt_kind);
+        if (oc == 0) return JABAS_ERR_OPT;           // nothing of an aggregate-only launch moves between steps
+        if (oc == 3) return JABAS_ERR_OPT;           // the amsgrad kernels take their scalars by value only
         if (reinterpret_cast<uintptr_t>(s->scalars_dev) % 16) return JABAS_ERR_ALIGN;
         a->dyn = static_cast<const StepScal*>(s->scalars_dev);
     }
@@ -432,7 +440,7 @@ JABAS_API int jabas_step_scalars_encode(const JabasStepArgs* args, void* host_bl
     StepScal sc;
     const int rc = fill_step_scal(args, &sc);
     if (rc != JABAS_OK) return rc;
-    if (opt_class_of(args->opt_kind) == 0) return JABAS_ERR_OPT;
+    if (opt_class_of(args->opt_kind) == 0 || opt_class_of(args->opt_kind) == 3) return JABAS_ERR_OPT;
     memcpy(host_block, &sc, sizeof(sc));
     return JABAS_OK;
 }
@@ -839,9 +847,9 @@ JABAS_API int jabas_sgd(const float* grad, float* param, float* momentum_buf, ui
     return jabas_sync_bucket(&sp, nullptr, &s, nullptr, nullptr, 0, stream);
 }
 
-JABAS_API int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq, uint64_t numel,
-                         double lr, double weight_decay, double beta1, double beta2, double eps, int64_t step,
-                         int32_t adamw, jabas_stream_t stream) {
+JABAS_API int jabas_adam(const float* grad, float* param, float* exp_avg, float* exp_avg_sq, float* max_exp_avg_sq,
+                         uint64_t numel, double lr, double weight_decay, double beta1, double beta2, double eps,
+                         int64_t step, int32_t adamw, jabas_stream_t stream) {
     if (!grad || !param || !exp_avg || !exp_avg_sq) return JABAS_ERR_NULL;
     JabasSpan sp;
     memset(&sp, 0, sizeof(sp));
@@ -851,11 +859,13 @@ JABAS_API int jabas_adam(const float* grad, float* param, float* exp_avg, float*
     sp.param = param;
     sp.state1 = exp_avg;
     sp.state2 = exp_avg_sq;
+    sp.state3 = max_exp_avg_sq;
     sp.numel = numel;
     s.K = 1;
     s.grad_dtype = JABAS_F32;
     s.weight[0] = 1.0f;
-    s.opt_kind = adamw ? JABAS_OPT_ADAMW : JABAS_OPT_ADAM;
+    s.opt_kind = max_exp_avg_sq ? (adamw ? JABAS_OPT_ADAMW_AMSGRAD : JABAS_OPT_ADAM_AMSGRAD)
+                                : (adamw ? JABAS_OPT_ADAMW : JABAS_OPT_ADAM);
     s.n_groups = 1;
     s.beta1 = beta1;
     s.beta2 = beta2;

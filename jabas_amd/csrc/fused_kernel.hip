@@ -92,7 +92,8 @@ template <> struct Grad<JABAS_BF16> {
     }
 };
 
-constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2;
+constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2, OPT_AMS = 3;    // OPT_AMS: Adam / AdamW with amsgrad
+__host__ __device__ constexpr bool is_adam(int opt) { return opt == OPT_ADAM || opt == OPT_AMS; }
 // Kernels with statistics over more than four gradient streams form the addresses of the vector path as
 // scalar base + 32-bit lane offset (measured on the ViT-L/16 set, K = 8 bf16: +0.5 % with full rows, +2 % with
 // similarity sums); their spans of more than kNarrowElems elements (over 4 GiB of fp32 per buffer) go
@@ -159,7 +160,7 @@ struct DynView {
 
 // One element of the optimizer step. g is the aggregated gradient.
 template <int OPT>
-__device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2,
+__device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2, float& s3,
                                          const GroupDev& G, const OptDev& O) {
     if constexpr (OPT == OPT_SGD) {
         float d = g;
@@ -170,12 +171,17 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
             d = O.nesterov ? d + O.momentum * s1 : s1;
         }
         p = p + G.neg_lr * d;
-    } else if constexpr (OPT == OPT_ADAM) {
+    } else if constexpr (is_adam(OPT)) {
         if (O.adamw) p = p * G.decay;
         else if (G.wd != 0.0f) g = g + G.wd * p;
         s1 = s1 * O.beta1 + g * O.one_minus_beta1;
         s2 = s2 * O.beta2 + (O.one_minus_beta2 * g) * g;
-        const float denom = __builtin_sqrtf(s2) / G.sqrt_bc2 + O.eps;
+        float second = s2;
+        if constexpr (OPT == OPT_AMS) {       // torch.maximum(max_exp_avg_sq, exp_avg_sq): a NaN on either side stays
+            s3 = (s3 != s3) ? s3 : ((s2 != s2) ? s2 : (s3 > s2 ? s3 : s2));
+            second = s3;
+        }
+        const float denom = __builtin_sqrtf(second) / G.sqrt_bc2 + O.eps;
         p = p + (G.neg_step_size * s1) / denom;
     }
 }
@@ -183,7 +189,7 @@ __device__ __forceinline__ void opt_elem(float g, float& p, float& s1, float& s2
 // Aggregate, statistics and optimizer for N consecutive elements held in registers.
 template <int K, int N, int DT, int OPT, int SL, bool HD, class A>
 __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], float (&s1)[N],
-                                        float (&s2)[N], float (&agg)[N], const A& a,
+                                        float (&s2)[N], float (&s3)[N], float (&agg)[N], const A& a,
                                         const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
@@ -213,7 +219,7 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
             acc[JABAS_STAT_NORM_B] = stat_fma(gb, gb, acc[JABAS_STAT_NORM_B]);
             acc[JABAS_STAT_NORM_AGG] = stat_fma(s, s, acc[JABAS_STAT_NORM_AGG]);
         }
-        if constexpr (OPT != OPT_NONE) opt_elem<OPT>(s, p[i], s1[i], s2[i], G, a.opt);
+        if constexpr (OPT != OPT_NONE) opt_elem<OPT>(s, p[i], s1[i], s2[i], s3[i], G, a.opt);
         // keep the elements' dependency chains apart: interleaving them costs the statistics
         // kernels a third of their occupancy in registers and buys nothing in a memory-bound loop
         if constexpr (SL) __builtin_amdgcn_sched_barrier(0);
@@ -238,15 +244,16 @@ template <int NV> __device__ __forceinline__ void unpack_vec(const f32x4 (&r)[NV
 }
 
 // Registers of U consecutive full tiles: the raw 16-byte vectors as loaded.
-template <int K, int DT, int U> struct TileRegs {
+template <int K, int DT, int U, int OPT = OPT_ADAM> struct TileRegs {
     typename Grad<DT>::Raw g[U][K];
     f32x4 p[U][Grad<DT>::EPT / 4], s1[U][Grad<DT>::EPT / 4], s2[U][Grad<DT>::EPT / 4];
+    f32x4 s3[OPT == OPT_AMS ? U : 1][Grad<DT>::EPT / 4];
 };
 
 // Issues every load of U consecutive full tiles. e is the (rebased) index of this
 // thread's first element in the first tile.
 template <int K, int DT, int OPT, int U, int BS, bool NARROW>
-__device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
+__device__ __forceinline__ void issue_loads(TileRegs<K, DT, U, OPT>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * EPT;
@@ -258,14 +265,15 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U>& r, const SpanDev
         if constexpr (OPT != OPT_NONE) {
             load_vec<NV, NARROW>(r.p[u], sp.p, eu);
             if (load_s1) load_vec<NV, NARROW>(r.s1[u], sp.s1, eu);
-            if constexpr (OPT == OPT_ADAM) load_vec<NV, NARROW>(r.s2[u], sp.s2, eu);
+            if constexpr (is_adam(OPT)) load_vec<NV, NARROW>(r.s2[u], sp.s2, eu);
+            if constexpr (OPT == OPT_AMS) load_vec<NV, NARROW>(r.s3[u], sp.s3, eu);
         }
     }
 }
 
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
 template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW, class A>
-__device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanDev& sp, uint64_t e, const A& a,
+__device__ __forceinline__ void consume(const TileRegs<K, DT, U, OPT>& r, const SpanDev& sp, uint64_t e, const A& a,
                                         const GroupDev& G, float clip, bool use_s1, bool load_s1,
                                         typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
@@ -274,7 +282,7 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 #pragma unroll
     for (int u = 0; u < U; ++u) {
         const uint64_t eu = e + u * TE;
-        float g[K][EPT], p[EPT], s1[EPT], s2[EPT], agg[EPT];
+        float g[K][EPT], p[EPT], s1[EPT], s2[EPT], s3[EPT], agg[EPT];
 #pragma unroll
         for (int k = 0; k < K; ++k) GR::widen(r.g[u][k], g[k]);
         if constexpr (OPT != OPT_NONE) {
@@ -284,14 +292,16 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U>& r, const SpanD
 #pragma unroll
                 for (int i = 0; i < EPT; ++i) s1[i] = 0.0f;
             }
-            if constexpr (OPT == OPT_ADAM) unpack_vec<NV>(r.s2[u], s2);
+            if constexpr (is_adam(OPT)) unpack_vec<NV>(r.s2[u], s2);
+            if constexpr (OPT == OPT_AMS) unpack_vec<NV>(r.s3[u], s3);
         }
-        compute<K, EPT, DT, OPT, SL, HD>(g, p, s1, s2, agg, a, G, clip, acc);
+        compute<K, EPT, DT, OPT, SL, HD>(g, p, s1, s2, s3, agg, a, G, clip, acc);
         if (sp.out) store_vec<NV, NARROW>(agg, sp.out, eu);
         if constexpr (OPT != OPT_NONE) {
             store_vec<NV, NARROW>(p, sp.p, eu);
             if (use_s1) store_vec<NV, NARROW>(s1, sp.s1, eu);
-            if constexpr (OPT == OPT_ADAM) store_vec<NV, NARROW>(s2, sp.s2, eu);
+            if constexpr (is_adam(OPT)) store_vec<NV, NARROW>(s2, sp.s2, eu);
+            if constexpr (OPT == OPT_AMS) store_vec<NV, NARROW>(s3, sp.s3, eu);
             for (uint32_t f = 0; f < sp.n_fan; ++f) store_vec<NV, NARROW>(p, sp.fan[f], eu);
         }
     }
@@ -304,11 +314,11 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
                                          const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     constexpr int BS = launch_block(K, DT, OPT, SL);
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
-    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
-    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
+    const bool use_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum);
+    const bool load_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     uint32_t i = 0;
     for (; i + U <= nfull; i += U, e += U * TE) {
-        TileRegs<K, DT, U> r;
+        TileRegs<K, DT, U, OPT> r;
         issue_loads<K, DT, OPT, U, BS, narrow_addressing(K, SL)>(r, sp, e, load_s1);
         consume<K, DT, OPT, SL, HD, U, narrow_addressing(K, SL)>(r, sp, e, a, G, clip, use_s1, load_s1, acc);
     }
@@ -328,8 +338,8 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr int BS = launch_block(K, DT, OPT, SL);
-    const bool use_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum);
-    const bool load_s1 = (OPT == OPT_ADAM) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
+    const bool use_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum);
+    const bool load_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
     const BoundDev* bd = sp.bound_count ? a.bounds + sp.bound_begin : nullptr;
     const uint64_t e_first = tile_e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
     const bool all_live = e_first >= sp.lo && e_first + EPT <= sp.hi;
@@ -344,7 +354,7 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
     }
     if (all_live && one_group) {
         const GroupDev G = a.groups[gid_first];
-        TileRegs<K, DT, 1> r;
+        TileRegs<K, DT, 1, OPT> r;
         issue_loads<K, DT, OPT, 1, BS, false>(r, sp, e_first, load_s1);
         consume<K, DT, OPT, SL, false, 1, false>(r, sp, e_first, a, G, clip, use_s1, load_s1, acc);   // halves from the mask: always right
         return;
@@ -360,20 +370,22 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
             gid = bd[jj].group & (JABAS_MAX_GROUPS - 1);   // a bound table on the device cannot be checked by the host
         }
         const GroupDev G = a.groups[gid];
-        float g[K][1], p[1] = {0.0f}, s1[1] = {0.0f}, s2[1] = {0.0f}, agg[1];
+        float g[K][1], p[1] = {0.0f}, s1[1] = {0.0f}, s2[1] = {0.0f}, s3[1] = {0.0f}, agg[1];
 #pragma unroll
         for (int k = 0; k < K; ++k) g[k][0] = GR::load1(sp.g[k], e);
         if constexpr (OPT != OPT_NONE) {
             p[0] = sp.p[e];
             if (load_s1) s1[0] = sp.s1[e];
-            if constexpr (OPT == OPT_ADAM) s2[0] = sp.s2[e];
+            if constexpr (is_adam(OPT)) s2[0] = sp.s2[e];
+            if constexpr (OPT == OPT_AMS) s3[0] = sp.s3[e];
         }
-        compute<K, 1, DT, OPT, SL, false>(g, p, s1, s2, agg, a, G, clip, acc);
+        compute<K, 1, DT, OPT, SL, false>(g, p, s1, s2, s3, agg, a, G, clip, acc);
         if (sp.out) sp.out[e] = agg[0];
         if constexpr (OPT != OPT_NONE) {
             sp.p[e] = p[0];
             if (use_s1) sp.s1[e] = s1[0];
-            if constexpr (OPT == OPT_ADAM) sp.s2[e] = s2[0];
+            if constexpr (is_adam(OPT)) sp.s2[e] = s2[0];
+            if constexpr (OPT == OPT_AMS) sp.s3[e] = s3[0];
             for (uint32_t r = 0; r < sp.n_fan; ++r) sp.fan[r][e] = p[0];
         }
     }
@@ -577,7 +589,7 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
 #endif
     constexpr unsigned idle = (OPT == OPT_ADAM && !SL && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
     const dim3 block(launch_block(K, DT, OPT, SL));
-    if constexpr (OPT != OPT_NONE) {
+    if constexpr (OPT == OPT_SGD || OPT == OPT_ADAM) {
         if (dyn) return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, true>, dim3(grid), block, idle, stream, a));
     } else {
         if (dyn) return static_cast<int>(hipErrorInvalidValue);     // refused by the front before it gets here
@@ -591,7 +603,8 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
 #define JABAS_CAT(a, b) JABAS_CAT_(a, b)
 
 #define JABAS_DISPATCH(FN, ...)                                                              \
-    const int key = (grad_dtype == JABAS_BF16 ? 9 : 0) + opt_class * 3 + stats;              \
+    const int key = opt_class == OPT_AMS ? 18 + (grad_dtype == JABAS_BF16 ? 3 : 0) + stats     \
+                                         : (grad_dtype == JABAS_BF16 ? 9 : 0) + opt_class * 3 + stats; \
     switch (key) {                                                                           \
         case 0:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 0>(__VA_ARGS__);                    \
         case 1:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 1>(__VA_ARGS__);                    \
@@ -611,6 +624,12 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
         case 15: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 0>(__VA_ARGS__);                   \
         case 16: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 1>(__VA_ARGS__);                   \
         case 17: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 2>(__VA_ARGS__);                   \
+        case 18: return FN<JABAS_K, JABAS_F32, OPT_AMS, 0>(__VA_ARGS__);                     \
+        case 19: return FN<JABAS_K, JABAS_F32, OPT_AMS, 1>(__VA_ARGS__);                     \
+        case 20: return FN<JABAS_K, JABAS_F32, OPT_AMS, 2>(__VA_ARGS__);                     \
+        case 21: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 0>(__VA_ARGS__);                    \
+        case 22: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 1>(__VA_ARGS__);                    \
+        case 23: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 2>(__VA_ARGS__);                    \
         default: return -1;                                                                  \
     }
 

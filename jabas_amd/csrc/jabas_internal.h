@@ -58,7 +58,8 @@ static_assert(block_ok(JABAS_BLOCK) && block_ok(JABAS_BLOCK_SGD) && block_ok(JAB
               block_ok(JABAS_BLOCK_SIM_MANYK), "whole waves");
 constexpr int kMinChunkTiles = JABAS_CHUNK_TILES_LO;
 constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
-// opt_class: 0 none, 1 SGD, 2 Adam/AdamW; stats: 0 none, 1 full rows, 2 similarity sums. The shape depends
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW, 3 Adam/AdamW with amsgrad (launch shapes of class 2);
+// stats: 0 none, 1 full rows, 2 similarity sums. The shape depends
 // on what a plan is encoded for (K, gradient dtype, optimizer class) and on the statistics level of the
 // launch; a plan holds one chunk table per shape, so it serves every step.
 __host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, int stats) {
@@ -97,6 +98,7 @@ struct SpanDev {
     float* p;
     float* s1;
     float* s2;
+    float* s3;
     float* fan[JABAS_MAX_K - 1];
     uint64_t lo, hi;
     uint32_t n_fan;
@@ -207,7 +209,8 @@ __device__ __forceinline__ double wave_sum_to_lane63(double v) {
 #endif
 
 // Per-K launchers, one translation unit each (fused_kernel.hip with -DJABAS_K=k).
-// opt_class: 0 none, 1 SGD, 2 Adam/AdamW; dyn: the step's scalars come from a.dyn (optimizer classes only).
+// opt_class: 0 none, 1 SGD, 2 Adam/AdamW, 3 the same with amsgrad; dyn: the step's scalars come from a.dyn
+// (classes 1 and 2 only).
 // Returns hipError_t as int.
 #define JABAS_DECLARE_K(k)                                                                   \
     int launch_fused_k##k(int grad_dtype, int opt_class, int stats, int dyn, const KArgs& a, \

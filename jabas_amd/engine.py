@@ -47,7 +47,7 @@ class VSWFlatSync:
         else:                                    # an arena of its own, unless nothing will ever be written to it
             self.agg = torch.zeros(n, dtype=torch.float32, device=self.device) if self.write_aggregate else None
         kind = opt_kind(opt)
-        self.param = self.state1 = self.state2 = None
+        self.param = self.state1 = self.state2 = self.state3 = None
         self.fanout = []
         if kind != L.OPT_NONE:
             if len(opt["groups"]) < self.layout.n_groups:
@@ -56,8 +56,10 @@ class VSWFlatSync:
             self.param = torch.zeros(n, dtype=torch.float32, device=self.device)
             if kind != L.OPT_SGD or opt.get("momentum", 0.0) != 0.0:
                 self.state1 = torch.zeros(n, dtype=torch.float32, device=self.device)
-            if kind in (L.OPT_ADAM, L.OPT_ADAMW):
+            if kind in (L.OPT_ADAM, L.OPT_ADAMW, L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD):
                 self.state2 = torch.zeros(n, dtype=torch.float32, device=self.device)
+            if kind in (L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD):       # amsgrad: max_exp_avg_sq
+                self.state3 = torch.zeros(n, dtype=torch.float32, device=self.device)
             self.fanout = [torch.zeros(n, dtype=torch.float32, device=self.device) for _ in range(n_fanout)]
         self._fanout_wanted = n_fanout > 0
         self._build_plan()
@@ -73,6 +75,7 @@ class VSWFlatSync:
                 param=None if self.param is None else self.param[sl],
                 state1=None if self.state1 is None else self.state1[sl],
                 state2=None if self.state2 is None else self.state2[sl],
+                state3=None if self.state3 is None else self.state3[sl],
                 fanout=[f[sl] for f in self.fanout],
                 bounds=bounds if kind != L.OPT_NONE else ()))
         self.span_bucket = [s[3] for s in self.layout.spans]
@@ -180,6 +183,8 @@ class VSWFlatSync:
         ``accumulations`` are fixed by the recording; ``reconfigure`` invalidates it."""
         if self.opt is None:
             raise ValueError("nothing moves between the steps of an engine without optimizer: record its launch directly")
+        if self.opt.get("amsgrad", False):
+            raise ValueError("the amsgrad kernels take the step's scalars by value only: an amsgrad step cannot be replayed")
         return GraphedStep(self, stats, clip_norm, accumulations)
 
     def _build_clip_plans(self):
@@ -193,6 +198,7 @@ class VSWFlatSync:
                                       param=self.param[sl],
                                       state1=None if self.state1 is None else self.state1[sl],
                                       state2=None if self.state2 is None else self.state2[sl],
+                                      state3=None if self.state3 is None else self.state3[sl],
                                       fanout=[f[sl] for f in self.fanout], bounds=bounds))
         self._plan_agg = SyncPlan(agg_spans, L.OPT_NONE)
         self._plan_opt = SyncPlan(opt_spans, opt_kind(self.opt))

@@ -146,7 +146,7 @@ class LocalBucketSync:
         under a norm bound (``grad_clip``) keep the write: their second launch reads the aggregate.
 
         opt + param_buckets: hyperparameter dictionary and, per bucket index, dict(param=, state1=,
-        state2=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket; the launch of
+        state2=, state3=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket; the launch of
         such a bucket also runs the optimizer. ``optimizer=`` (or ``bind_optimizer``) takes a
         torch.optim.SGD / Adam / AdamW or Shard* object instead and builds those arenas itself from the
         ``parameters()`` / ``gradients()`` of the bucket objects the hooks publish."""
@@ -346,22 +346,24 @@ class LocalBucketSync:
                 new["state1"] = _arena_like(buf0)
             if not sgd:
                 new["state2"] = _arena_like(buf0)
+            if self.opt.get("amsgrad", False):
+                new["state3"] = _arena_like(buf0)
             if buf0.dtype != torch.float32 and (self.write_aggregate or self.grad_clip != float("inf")):
                 new["agg_out"] = _arena_like(buf0)
-            names = ("momentum_buffer",) if sgd else ("exp_avg", "exp_avg_sq")
+            names = ("momentum_buffer",) if sgd else ("exp_avg", "exp_avg_sq", "max_exp_avg_sq")
             had_state = 0
             for p, o in zip(params, offs):
                 view = new["param"][o:o + p.numel()].view(p.shape)
                 view.copy_(p.data)
                 p.data = view
                 st = self.optimizer.state[p]
-                for name, arena in zip(names, ("state1", "state2")):
+                for name, arena in zip(names, ("state1", "state2", "state3")):
                     if arena not in new:
                         continue
                     sview = new[arena][o:o + p.numel()].view(p.shape)
                     if torch.is_tensor(st.get(name)):
                         sview.copy_(st[name])
-                        had_state += name != "exp_avg_sq"
+                        had_state += name in ("momentum_buffer", "exp_avg")
                     st[name] = sview
                 if not sgd:
                     if "step" in st and int(float(st["step"])) != self.step_count:
@@ -666,7 +668,7 @@ class LocalBucketSync:
                 call = sync.BucketCall(agg_span)
                 call.update = sync.BucketCall(sync.SpanSpec(
                     [span.agg_out], agg_out=span.agg_out, param=span.param, state1=span.state1, state2=span.state2,
-                    fanout=span.fanout, bounds=span.bounds))
+                    state3=span.state3, fanout=span.fanout, bounds=span.bounds))
                 with torch.cuda.stream(main):
                     call.coef = torch.ones(1, dtype=torch.float32, device=tensors[0].device)
             else:
@@ -698,7 +700,8 @@ class LocalBucketSync:
             agg_out = None
         span = sync.SpanSpec(tensors, agg_out=agg_out,
                              param=pb and pb.get("param"), state1=pb and pb.get("state1"),
-                             state2=pb and pb.get("state2"), fanout=(pb or {}).get("fanout", ()),
+                             state2=pb and pb.get("state2"), state3=pb and pb.get("state3"),
+                             fanout=(pb or {}).get("fanout", ()),
                              bounds=(pb or {}).get("bounds", ()) if opt else ())
         return span, opt is not None
 

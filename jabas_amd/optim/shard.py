@@ -156,8 +156,8 @@ class _ShardOptimizer(torch.optim.Optimizer):
         return g
 
     def _launch(self, spans, args):
-        key = tuple((s.grads[0].data_ptr(), s.param.data_ptr(), s.grads[0].numel(), s.bounds[0][1]) +
-                    tuple(f.data_ptr() for f in s.fanout) for s in spans)
+        key = (args.opt_kind,) + tuple((s.grads[0].data_ptr(), s.param.data_ptr(), s.grads[0].numel(), s.bounds[0][1],
+                                         s.agg_out is not None) + tuple(f.data_ptr() for f in s.fanout) for s in spans)
         plan = self._plans.get(key)
         if plan is None:
             if len(self._plans) >= self._max_cached_plans:
@@ -281,29 +281,37 @@ class ShardAdam(_ShardOptimizer):
             return loss
         self._copies, self._volatile, launches, self._late_copies = [], False, [], []
         batches = {}
+        write_back = getattr(self, "_grad_scale", None) is not None     # a clipped step leaves the clipped gradients behind
         for gi, p, g in pairs:
             group = self.param_groups[gi]
-            if group["amsgrad"]:
-                raise NotImplementedError("amsgrad is not part of the fused path")
+            amsgrad = bool(group["amsgrad"])
             st = self.state[p]
             if len(st) == 0:
                 self._volatile = True             # state created in this call: remember the next one
                 st["step"] = 0
                 st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
                 st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                if amsgrad:                       # the maximum of the second moment so far (shard_optimizer.py:58-60)
+                    st["max_exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            elif amsgrad and "max_exp_avg_sq" not in st:
+                raise RuntimeError("amsgrad was switched on after the state was created: no max_exp_avg_sq to continue from")
             st["step"] += 1
-            key = (tuple(group["betas"]), group["eps"])
+            key = (tuple(group["betas"]), group["eps"], amsgrad)
             batches.setdefault(key, []).append((gi, int(st["step"]), p, self._prepare(p, g), st))
-        for (betas, eps), items in batches.items():
+        for (betas, eps, amsgrad), items in batches.items():
             slots, spans = {}, []
-            args = self._new_args(L.OPT_ADAMW if self._adamw else L.OPT_ADAM)
+            if amsgrad:
+                args = self._new_args(L.OPT_ADAMW_AMSGRAD if self._adamw else L.OPT_ADAM_AMSGRAD)
+            else:
+                args = self._new_args(L.OPT_ADAMW if self._adamw else L.OPT_ADAM)
             for gi, step, p, g, st in items:
                 slot = slots.setdefault((gi, step), len(slots))
                 if slot >= L.MAX_GROUPS:
                     raise RuntimeError(f"more than {L.MAX_GROUPS} (group, step) combinations in one launch")
-                spans.append(sync.SpanSpec([g], param=p.data.view(-1), state1=st["exp_avg"].view(-1),
-                                           state2=st["exp_avg_sq"].view(-1), fanout=self._fanout(p),
-                                           bounds=((0, slot),)))
+                spans.append(sync.SpanSpec([g], agg_out=g if write_back else None, param=p.data.view(-1),
+                                           state1=st["exp_avg"].view(-1), state2=st["exp_avg_sq"].view(-1),
+                                           state3=st["max_exp_avg_sq"].view(-1) if amsgrad else None,
+                                           fanout=self._fanout(p), bounds=((0, slot),)))
             for (gi, step), slot in slots.items():
                 args.groups[slot].lr = float(self.param_groups[gi]["lr"])
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
@@ -315,8 +323,11 @@ class ShardAdam(_ShardOptimizer):
             reps = {}
             for gi, step, p, g, st in items:
                 reps.setdefault(slots[(gi, step)], (gi, st))
-            launches.append((plan, args, (betas, eps), sorted(reps.items()),
+            launches.append((plan, args, (betas, eps, amsgrad), sorted(reps.items()),
                              [(st, slots[(gi, step)]) for gi, step, p, g, st in items]))
+        if write_back:
+            for tmp, g in self._copies:           # gradients that were realigned into a copy: the clipped values go back
+                g.copy_(tmp)
         self._copy_late(self._late_copies)
         if not self._volatile:
             self._remember(sig, launches, self._copies)
@@ -332,7 +343,7 @@ class ShardAdam(_ShardOptimizer):
         for _, _, key, reps, items in launches:
             for _, (gi, _) in reps:
                 group = self.param_groups[gi]
-                if (tuple(group["betas"]), group["eps"]) != key or group["amsgrad"]:
+                if (tuple(group["betas"]), group["eps"], bool(group["amsgrad"])) != key:
                     return False
             steps = [st["step"] for _, (_, st) in reps]
             for st, slot in items:
@@ -348,6 +359,9 @@ class ShardAdam(_ShardOptimizer):
                 args.groups[slot].weight_decay = float(self.param_groups[gi]["weight_decay"])
                 args.groups[slot].step = int(st["step"])
             plan.run(args)
+        if getattr(self, "_grad_scale", None) is not None:
+            for tmp, g in copies:
+                g.copy_(tmp)
         self._copy_late(late)
         return True
 
@@ -364,8 +378,9 @@ class ShardGNMTAdam(ShardAdam):
     the gradients handed to one ``step(gradients)`` call (one DDP bucket in the overlap mode) are scaled to a
     joint 2-norm of at most ``grad_clip`` before the update, torch.nn.utils.clip_grad_norm_'s rule
     (coefficient max_norm / (norm + 1e-6), applied when below 1). One statistics launch over the gradients
-    forms the norm, the coefficient stays on the device, and the Adam launch multiplies it in; the gradient
-    buffers themselves are left as they were."""
+    forms the norm, the coefficient stays on the device, and the Adam launch multiplies it in and writes the
+    scaled gradients back in place, as ``clip_grad_norm_for_overlap`` leaves the tensors it was handed
+    (shard_optimizer.py:75-76): a caller that reads gradient norms after the step sees the clipped ones."""
 
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0, amsgrad=False,
                  grad_clip=float('inf')):

@@ -59,9 +59,15 @@ _KIND = {None: L.OPT_NONE, "none": L.OPT_NONE, "sgd": L.OPT_SGD, "adam": L.OPT_A
 
 
 def opt_kind(opt):
+    """JABAS_OPT_* code of a hyperparameter dictionary; ``amsgrad=True`` selects the Adam / AdamW kinds that
+    keep the running maximum of the second moment (``state3`` of the spans)."""
     kind = None if opt is None else opt["kind"]
     if kind not in _KIND:
         raise ValueError(f"unknown optimizer kind {kind!r}")
+    if opt is not None and opt.get("amsgrad", False):
+        if kind not in ("adam", "adamw"):
+            raise ValueError("amsgrad belongs to Adam and AdamW")
+        return L.OPT_ADAMW_AMSGRAD if kind == "adamw" else L.OPT_ADAM_AMSGRAD
     return _KIND[kind]
 
 
@@ -170,9 +176,9 @@ def _check_tensor(t, n, dtype, what, device):
 class SpanSpec:
     """Tensors of one span. All 1-D (or contiguous) with the same number of elements."""
 
-    def __init__(self, grads, agg_out=None, param=None, state1=None, state2=None, fanout=(), bounds=()):
+    def __init__(self, grads, agg_out=None, param=None, state1=None, state2=None, fanout=(), bounds=(), state3=None):
         self.grads = list(grads)
-        self.agg_out, self.param, self.state1, self.state2 = agg_out, param, state1, state2
+        self.agg_out, self.param, self.state1, self.state2, self.state3 = agg_out, param, state1, state2, state3
         self.fanout = list(fanout)
         self.bounds = list(bounds)          # [(start_element, group), ...], first start 0
 
@@ -189,6 +195,7 @@ class SpanSpec:
         _check_tensor(self.param, n, torch.float32, "param", dev)
         _check_tensor(self.state1, n, torch.float32, "state1", dev)
         _check_tensor(self.state2, n, torch.float32, "state2", dev)
+        _check_tensor(self.state3, n, torch.float32, "state3", dev)
         for r, f in enumerate(self.fanout):
             _check_tensor(f, n, torch.float32, f"fanout[{r}]", dev)
         return n, dev, gdt
@@ -202,6 +209,7 @@ class SpanSpec:
         s.param = _ptr(self.param)
         s.state1 = _ptr(self.state1)
         s.state2 = _ptr(self.state2)
+        s.state3 = _ptr(self.state3)
         for r, f in enumerate(self.fanout):
             s.fanout[r] = f.data_ptr()
         s.numel = n
@@ -453,11 +461,14 @@ def sgd_step(grad, param, momentum_buf, lr, weight_decay=0.0, momentum=0.0, damp
                               dampening, int(bool(nesterov)), int(bool(first_step)), _stream_ptr(stream)), "jabas_sgd")
 
 
-def adam_step(grad, param, exp_avg, exp_avg_sq, lr, weight_decay, betas, eps, step, adamw, stream=None):
+def adam_step(grad, param, exp_avg, exp_avg_sq, lr, weight_decay, betas, eps, step, adamw, stream=None,
+              max_exp_avg_sq=None):
+    """``max_exp_avg_sq``: the running maximum of the second moment: the step is then amsgrad's."""
     n = param.numel()
-    for t, what in ((grad, "grad"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+    for t, what in ((grad, "grad"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq"), (max_exp_avg_sq, "max_exp_avg_sq")):
         _check_tensor(t, n, torch.float32, what, param.device)
-    L.check(L.lib().jabas_adam(grad.data_ptr(), param.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
+    L.check(L.lib().jabas_adam(grad.data_ptr(), param.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(),
+                               _ptr(max_exp_avg_sq), n,
                                lr, weight_decay, betas[0], betas[1], eps, int(step), int(bool(adamw)),
                                _stream_ptr(stream)), "jabas_adam")
 

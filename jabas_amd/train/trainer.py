@@ -133,10 +133,11 @@ def opt_from_torch_optimizer(optimizer):
             raise ValueError("maximize=True is not supported")
     elif isinstance(optimizer, (torch.optim.AdamW, ShardAdamW, torch.optim.Adam, ShardAdam)):
         adamw = isinstance(optimizer, (torch.optim.AdamW, ShardAdamW))
-        if g0.get("amsgrad", False) or g0.get("maximize", False):
-            raise ValueError("amsgrad / maximize are not supported")
+        if g0.get("maximize", False):
+            raise ValueError("maximize=True is not supported")
         b1, b2 = same("betas")
-        opt = dict(kind="adamw" if adamw else "adam", betas=(float(b1), float(b2)), eps=float(same("eps")))
+        opt = dict(kind="adamw" if adamw else "adam", betas=(float(b1), float(b2)), eps=float(same("eps")),
+                   amsgrad=bool(same("amsgrad")) if "amsgrad" in g0 else False)
     else:
         raise TypeError(f"unsupported optimizer type {type(optimizer).__name__}: SGD, Adam, AdamW or their "
                         "Shard counterparts")
@@ -262,6 +263,8 @@ class VSWSyncTrainer:
                 st["step"] = self._step_tensor
                 st["exp_avg"] = eng._view(eng.state1, i).view(p.shape)
                 st["exp_avg_sq"] = eng._view(eng.state2, i).view(p.shape)
+                if eng.state3 is not None:
+                    st["max_exp_avg_sq"] = eng._view(eng.state3, i).view(p.shape)
 
     def _refresh_hyperparameters(self):
         """Learning rate and weight decay as the caller's optimizer object holds them now."""
@@ -337,6 +340,7 @@ class VSWSyncTrainer:
                 "numel": eng.layout.total,
                 "state1": None if eng.state1 is None else eng.state1.detach().clone(),
                 "state2": None if eng.state2 is None else eng.state2.detach().clone(),
+                "state3": None if eng.state3 is None else eng.state3.detach().clone(),
                 "groups": [dict(g) for g in self.opt["groups"]],
             }
         return out
@@ -365,7 +369,8 @@ class VSWSyncTrainer:
             steps, has_momentum = set(), False
             for i, p in enumerate(self.main_model.parameters()):        # ... copied into the arenas
                 st = self.main_optimizer.state.get(p, {})
-                for key, arena in (("momentum_buffer", eng.state1), ("exp_avg", eng.state1), ("exp_avg_sq", eng.state2)):
+                for key, arena in (("momentum_buffer", eng.state1), ("exp_avg", eng.state1), ("exp_avg_sq", eng.state2),
+                                   ("max_exp_avg_sq", eng.state3)):
                     if arena is not None and st.get(key) is not None:
                         eng._view(arena, i).copy_(st[key].reshape(-1))
                         has_momentum = has_momentum or key == "momentum_buffer"
@@ -385,7 +390,8 @@ class VSWSyncTrainer:
             arenas = state["optimizer_arenas"]
             if arenas["numel"] != eng.layout.total:
                 raise ValueError("the checkpoint's state arenas belong to another layout")
-            for mine, theirs in ((eng.state1, arenas["state1"]), (eng.state2, arenas["state2"])):
+            for mine, theirs in ((eng.state1, arenas["state1"]), (eng.state2, arenas["state2"]),
+                                 (eng.state3, arenas.get("state3"))):
                 if (mine is None) != (theirs is None):
                     raise ValueError("the checkpoint's optimizer keeps other state than this one")
                 if mine is not None:

@@ -75,10 +75,10 @@ def sgd_step(p, g, buf, lr, weight_decay=0.0, momentum=0.0, dampening=0.0, neste
                  int(momentum != 0), int(first_step), int(nesterov))
 
 
-def adam_step(p, g, m, v, lr, weight_decay, betas, eps, step, adamw):
+def adam_step(p, g, m, v, lr, weight_decay, betas, eps, step, adamw, vmax=None):
     beta1, beta2 = betas
     bc1 = 1 - beta1 ** step
     bc2 = 1 - beta2 ** step
     lib().oc_adam(C.c_void_p(p.data_ptr()), C.c_void_p(g.data_ptr()), C.c_void_p(m.data_ptr()), C.c_void_p(v.data_ptr()),
-                  C.c_size_t(p.numel()), _f(weight_decay), _f(1 - lr * weight_decay), _f(beta1), _f(1 - beta1),
+                  C.c_void_p(vmax.data_ptr() if vmax is not None else 0), C.c_size_t(p.numel()), _f(weight_decay), _f(1 - lr * weight_decay), _f(beta1), _f(1 - beta1),
                   _f(beta2), _f(1 - beta2), _f(math.sqrt(bc2)), _f(eps), _f(-(lr / bc1)), int(adamw))

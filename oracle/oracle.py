@@ -140,8 +140,11 @@ def _ieee_sqrt(t):
     return torch.from_numpy(np.sqrt(t.detach().contiguous().numpy()))
 
 
-def adam_step(p, g, m, v, lr, weight_decay, betas, eps, step, adamw):
-    """torch 1.8.1 _functional.adam / adamw (amsgrad off) on one tensor, in place."""
+def adam_step(p, g, m, v, lr, weight_decay, betas, eps, step, adamw, vmax=None):
+    """torch 1.8.1 _functional.adam / adamw on one tensor, in place. ``vmax``: the running maximum of the
+    second moment (``max_exp_avg_sq``) when amsgrad is on, as ShardGNMTAdam.step threads it into F.adam
+    (examples/gnmt/seq2seq/train/shard_optimizer.py:58-66,79-90): torch.maximum(max_exp_avg_sq, exp_avg_sq,
+    out=max_exp_avg_sq), and the denominator is formed from the maximum."""
     beta1, beta2 = betas
     bc1 = 1 - beta1 ** step
     bc2 = 1 - beta2 ** step
@@ -151,13 +154,16 @@ def adam_step(p, g, m, v, lr, weight_decay, betas, eps, step, adamw):
         g = torch.add(g, torch.mul(p, weight_decay))
     m.copy_(torch.add(torch.mul(m, beta1), torch.mul(g, 1 - beta1)))
     v.copy_(torch.add(torch.mul(v, beta2), torch.mul(torch.mul(g, 1 - beta2), g)))
-    denom = torch.add(torch.div(_ieee_sqrt(v), math.sqrt(bc2)), eps)
+    if vmax is not None:
+        vmax.copy_(torch.maximum(vmax, v))
+    denom = torch.add(torch.div(_ieee_sqrt(v if vmax is None else vmax), math.sqrt(bc2)), eps)
     step_size = lr / bc1
     p.copy_(torch.add(p, torch.div(torch.mul(m, -step_size), denom)))
 
 
-def opt_step(opt, group, p, g, s1, s2, step, first_step, lr_scale=1.0):
-    """Dispatch on the optimizer dictionary used throughout the build."""
+def opt_step(opt, group, p, g, s1, s2, step, first_step, lr_scale=1.0, s3=None):
+    """Dispatch on the optimizer dictionary used throughout the build (``s3``: max_exp_avg_sq when
+    ``opt['amsgrad']``)."""
     grp = opt["groups"][group]
     lr = grp["lr"] * lr_scale
     step = grp.get("step", step)               # a group may carry its own Adam step count
@@ -166,8 +172,10 @@ def opt_step(opt, group, p, g, s1, s2, step, first_step, lr_scale=1.0):
         sgd_step(p, g, s1, lr, wd, opt.get("momentum", 0.0), opt.get("dampening", 0.0),
                  opt.get("nesterov", False), first_step)
     elif opt["kind"] in ("adam", "adamw"):
+        if bool(opt.get("amsgrad", False)) != (s3 is not None):
+            raise ValueError("amsgrad needs the max_exp_avg_sq tensor, and only amsgrad takes one")
         adam_step(p, g, s1, s2, lr, wd, opt.get("betas", (0.9, 0.999)), opt.get("eps", 1e-8), step,
-                  opt["kind"] == "adamw")
+                  opt["kind"] == "adamw", vmax=s3)
     else:
         raise ValueError(opt["kind"])
 
@@ -188,7 +196,7 @@ def clip(agg, max_norm, eps=1e-6):
 
 # ---------------------------------------------------------------------- whole sync step
 def sync_step(grads, batches, spans, opt=None, param=None, state1=None, state2=None, step=1, first_step=False,
-              want_stats=False, half_id=None, lr_scale=1.0, clip_norm=None):
+              want_stats=False, half_id=None, lr_scale=1.0, clip_norm=None, state3=None):
     """Fused-step semantics over flat CPU arenas.
 
     grads: K flat tensors; spans: [(offset, numel, bounds)] with bounds [(start, group)].
@@ -216,5 +224,6 @@ def sync_step(grads, batches, spans, opt=None, param=None, state1=None, state2=N
                 s2_ = slice(off + start, off + end)
                 opt_step(opt, group, param[s2_], agg[s2_],
                          None if state1 is None else state1[s2_],
-                         None if state2 is None else state2[s2_], step, first_step, lr_scale)
+                         None if state2 is None else state2[s2_], step, first_step, lr_scale,
+                         None if state3 is None else state3[s2_])
     return agg, rows

@@ -95,7 +95,8 @@ void oc_sgd(float* p, const float* g, float* buf, size_t n, float wd, float neg_
     }
 }
 
-void oc_adam(float* p, const float* g, float* m, float* v, size_t n, float wd, float decay, float beta1,
+/* vmax: NULL, or max_exp_avg_sq of amsgrad (torch.maximum propagates NaN from either side) */
+void oc_adam(float* p, const float* g, float* m, float* v, float* vmax, size_t n, float wd, float decay, float beta1,
              float one_minus_beta1, float beta2, float one_minus_beta2, float sqrt_bc2, float eps,
              float neg_step_size, int adamw) {
     for (size_t i = 0; i < n; ++i) {
@@ -107,7 +108,13 @@ void oc_adam(float* p, const float* g, float* m, float* v, size_t n, float wd, f
         float c = v[i] * beta2, e = gi * one_minus_beta2;
         e = e * gi;
         v[i] = c + e;
-        float denom = sqrtf(v[i]);
+        float second = v[i];
+        if (vmax) {
+            float a0 = vmax[i], b0 = v[i];
+            vmax[i] = (a0 != a0) ? a0 : ((b0 != b0) ? b0 : (a0 > b0 ? a0 : b0));
+            second = vmax[i];
+        }
+        float denom = sqrtf(second);
         denom = denom / sqrt_bc2;
         denom = denom + eps;
         float num = m[i] * neg_step_size;

@@ -18,6 +18,7 @@ int main(void) {
     SHOW_OFF(JabasSpan, param);
     SHOW_OFF(JabasSpan, state1);
     SHOW_OFF(JabasSpan, state2);
+    SHOW_OFF(JabasSpan, state3);
     SHOW_OFF(JabasSpan, fanout);
     SHOW_OFF(JabasSpan, numel);
     SHOW_OFF(JabasSpan, n_fanout);

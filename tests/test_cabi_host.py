@@ -34,7 +34,7 @@ def test_struct_layouts_match_the_header():
     # sizes a C compiler gives the header's structs on x86-64 / amdgcn host ABI
     K = L.MAX_K
     assert K == 16 and L.STATS_STRIDE == 4 + K
-    assert C.sizeof(L.JabasSpan) == K * 8 + 4 * 8 + (K - 1) * 8 + 8 + 4 * 4
+    assert C.sizeof(L.JabasSpan) == K * 8 + 5 * 8 + (K - 1) * 8 + 8 + 4 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
     assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 4 * K + 4 + K + 4 * K + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8 + 8
@@ -209,8 +209,23 @@ def test_entry_points_validate_before_launching():
     # nesterov needs momentum and zero dampening
     assert lib.jabas_sgd(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 10, 0.1, 0.0, 0.9, 0.1, 1, 0, None) == L.ERR_OPT
     # Adam's step count is 1-based
-    assert lib.jabas_adam(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 0x7f0300000000, 10, 1e-3, 0.0, 0.9, 0.999,
-                          1e-8, 0, 0, None) == L.ERR_OPT
+    assert lib.jabas_adam(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 0x7f0300000000, None, 10, 1e-3, 0.0, 0.9,
+                          0.999, 1e-8, 0, 0, None) == L.ERR_OPT
+    # amsgrad: the maximum is one more written buffer (it must not overlap the second moment), and its launches
+    # take their scalars by value only
+    assert lib.jabas_adam(0x7f0000000000, 0x7f0100000000, 0x7f0200000000, 0x7f0300000000, 0x7f0300000010, 10, 1e-3, 0.0,
+                          0.9, 0.999, 1e-8, 1, 0, None) == L.ERR_ALIAS
+    ams = L.JabasStepArgs()
+    ams.K, ams.grad_dtype, ams.opt_kind, ams.n_groups = 1, L.F32, L.OPT_ADAMW_AMSGRAD, 1
+    ams.weight[0], ams.beta1, ams.beta2, ams.eps = 1.0, 0.9, 0.999, 1e-8
+    ams.groups[0].lr, ams.groups[0].step = 1e-3, 1
+    sp = _span(1000, K=1, opt=True)
+    assert lib.jabas_sync_bucket(C.byref(sp), None, C.byref(ams), None, None, 0, None) == L.ERR_NULL     # no state3
+    block = np.zeros(L.STEP_SCALARS_BYTES, dtype=np.uint8)
+    assert lib.jabas_step_scalars_encode(C.byref(ams), block.ctypes.data, block.nbytes) == L.ERR_OPT
+    sp.state3 = 0x7f0000000000 + 21 * (1 << 32)
+    ams.scalars_dev = 0x7f0000000000 + 22 * (1 << 32)
+    assert lib.jabas_sync_bucket(C.byref(sp), None, C.byref(ams), None, None, 0, None) == L.ERR_OPT
     hid = (C.c_uint8 * 2)(0, 1)
     assert lib.jabas_stats(g, 2, L.F32, w, hid, w, 100, 0x7f0400000000, None, 0, None) == L.ERR_ALIGN
     g[1] = 0x7f0100000000
@@ -249,7 +264,7 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
             s, f = name.split(".")
             assert getattr(structs[s], f).offset == int(val), name
             checked += 1
-    assert checked == 37
+    assert checked == 38
     # every field of the ctypes mirror was reported by the C side (reserved words aside)
     for sname, st in structs.items():
         for f, _ in st._fields_:

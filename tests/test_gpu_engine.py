@@ -108,6 +108,33 @@ def test_global_norm_clipping(gpu, opt, clip_norm, keep):
         assert norm == pytest.approx(clip_norm, rel=1e-4)
 
 
+@pytest.mark.parametrize("dtype,clip", [(torch.float32, None), (torch.bfloat16, None), (torch.float32, 0.05)])
+def test_engine_amsgrad_matches_oracle(gpu, dtype, clip):
+    """A planned launch over several buckets and parameter groups with amsgrad, plain and under a global norm
+    bound: weights, both moments and the maximum bit-identical to the oracle; an amsgrad step is not recordable."""
+    batches = (4, 2, 2)
+    opt = dict(ADAM, amsgrad=True)
+    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=1)
+    host["s3"] = torch.zeros(eng.layout.total)
+    assert eng.state3 is not None
+    for step in (1, 2, 3, 4):
+        gen = torch.Generator().manual_seed(900 + step)
+        host["g"] = [(torch.randn(eng.layout.total, generator=gen) * (5e-2 if step <= 2 else 2e-3)).to(dtype) for _ in batches]
+        for k, g in enumerate(host["g"]):
+            eng.grads[k].copy_(g)
+        eng.step(stats="similarity", clip_norm=clip)
+        torch.cuda.synchronize()
+        O.sync_step(host["g"], batches, spans, opt, host["p"], host["s1"], host["s2"], step=step, want_stats=False,
+                    clip_norm=clip, state3=host["s3"])
+        for off, cnt, _ in spans:
+            sl = slice(off, off + cnt)
+            for name, d, h in (("p", eng.param, host["p"]), ("m", eng.state1, host["s1"]), ("v", eng.state2, host["s2"]),
+                               ("max", eng.state3, host["s3"]), ("replica", eng.fanout[0], host["p"])):
+                assert torch.equal(d[sl].cpu().view(torch.int32), h[sl].view(torch.int32)), (step, name)
+    with pytest.raises(ValueError, match="amsgrad"):
+        eng.capture()
+
+
 def test_reconfigure_changes_k_and_keeps_weights_and_state(gpu):
     batches = (4, 4)
     eng, host, spans = _make(gpu, batches, ADAM, n_fanout=1)

@@ -32,7 +32,7 @@ def _groups(model):
     return [{"params": no_decay, "weight_decay": 0.0}, {"params": decay, "weight_decay": 0.05}]
 
 
-@pytest.mark.parametrize("kind", ["sgd", "sgd_nesterov", "adam", "adamw"])
+@pytest.mark.parametrize("kind", ["sgd", "sgd_nesterov", "adam", "adamw", "adam_amsgrad", "adamw_amsgrad", "gnmt_adam_amsgrad"])
 def test_shard_optimizers_match_torch_optim(gpu, kind):
     from jabas_amd import optim
     ref_model, my_model = _mlp(0).to(gpu), _mlp(0).to(gpu)
@@ -45,15 +45,26 @@ def test_shard_optimizers_match_torch_optim(gpu, kind):
     elif kind == "adam":
         ref = torch.optim.Adam(_groups(ref_model), lr=2e-3, foreach=False)
         mine = optim.ShardAdam(_groups(my_model), lr=2e-3)
+    elif kind == "adam_amsgrad":
+        ref = torch.optim.Adam(_groups(ref_model), lr=2e-3, foreach=False, amsgrad=True)
+        mine = optim.ShardAdam(_groups(my_model), lr=2e-3, amsgrad=True)
+    elif kind == "adamw_amsgrad":
+        ref = torch.optim.AdamW(_groups(ref_model), lr=5e-4, foreach=False, amsgrad=True)
+        mine = optim.ShardAdamW(_groups(my_model), lr=5e-4, amsgrad=True)
+    elif kind == "gnmt_adam_amsgrad":           # the reference's own subclass, amsgrad threaded through as it does
+        ref = torch.optim.Adam(ref_model.parameters(), lr=2e-3, foreach=False, amsgrad=True)
+        mine = optim.ShardGNMTAdam(my_model.parameters(), lr=2e-3, amsgrad=True)
     else:
         ref = torch.optim.AdamW(_groups(ref_model), lr=5e-4, foreach=False)
         mine = optim.ShardAdamW(_groups(my_model), lr=5e-4)
-    for step in range(4):
+    for step in range(6 if kind.endswith("amsgrad") else 4):
         g = torch.Generator(device="cpu").manual_seed(step)
+        # (amsgrad: the loss shrinks after the second step, so the second moment falls below its maximum)
         x = torch.randn(16, 37, generator=g).to(gpu)
+        scale = 0.01 if kind.endswith("amsgrad") and step >= 2 else 1.0
         for model in (ref_model, my_model):
             model.zero_grad(set_to_none=True)
-            model(x).square().mean().backward()
+            (model(x).square().mean() * scale).backward()
         ref.step()
         mine.step()
         torch.cuda.synchronize()
@@ -62,6 +73,12 @@ def test_shard_optimizers_match_torch_optim(gpu, kind):
     key = "momentum_buffer" if kind.startswith("sgd") else "exp_avg"
     for pr, pm in zip(ref_model.parameters(), my_model.parameters()):
         assert _close(mine.state[pm][key], ref.state[pr][key], 1e-6, 1e-8)
+        if kind.endswith("amsgrad"):
+            assert _close(mine.state[pm]["max_exp_avg_sq"], ref.state[pr]["max_exp_avg_sq"], 1e-6, 1e-14)
+            assert bool((mine.state[pm]["max_exp_avg_sq"] >= mine.state[pm]["exp_avg_sq"]).all())
+    if kind.endswith("amsgrad"):
+        above = torch.cat([(mine.state[p]["max_exp_avg_sq"] > mine.state[p]["exp_avg_sq"]).reshape(-1) for p in my_model.parameters()])
+        assert bool(above.any())                             # somewhere the maximum did part from the moment
 
 
 def test_shard_step_with_bucket_gradients_updates_only_matching_parameters(gpu):
@@ -373,7 +390,7 @@ def test_trainer_steps_at_lr_times_the_controllers_modifier(gpu, kind):
     assert mine.param_groups[0]["lr"] == (0.05 if kind == "sgd" else 1e-3)      # the caller's lr itself is left alone
 
 
-@pytest.mark.parametrize("kind", ["sgd", "adamw", "shard_adam"])
+@pytest.mark.parametrize("kind", ["sgd", "adamw", "shard_adam", "adamw_amsgrad"])
 def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
     """The reference's order of calls (examples/resnet50/main.py:351-366, examples/vit/main.py:425-478):
     prepare_stream_parallel, an optimizer built over trainer.main_model, prepare_weight_sync_method
@@ -392,6 +409,8 @@ def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
             return torch.optim.SGD(groups, lr=0.05, momentum=0.9, foreach=False)
         if kind == "adamw":
             return torch.optim.AdamW(groups, lr=1e-3, foreach=False)
+        if kind == "adamw_amsgrad":
+            return torch.optim.AdamW(groups, lr=1e-3, foreach=False, amsgrad=True)
         return (optim.ShardAdam if shard else torch.optim.Adam)(groups, lr=2e-3, **({} if shard else {"foreach": False}))
 
     mine, ref_opt = build(trainer.main_model, True), build(ref_model, False)
@@ -407,7 +426,9 @@ def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
                 for g in opt_.param_groups:
                     g["lr"] = 0.05 * (0.8 ** step)
         gen = torch.Generator().manual_seed(70 + step)
-        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        shrink = 0.01 if kind.endswith("amsgrad") and step >= 3 else 1.0    # the second moment falls below its maximum
+        data = [(torch.randn(b, 37, generator=gen).to(gpu) * shrink, torch.randn(b, 10, generator=gen).to(gpu) * shrink)
+                for b in batches]
         trainer.compute(data)
         per_vsw = []
         for x, y in data:
@@ -435,6 +456,8 @@ def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
         if kind != "sgd":
             assert float(mine.state[p]["step"]) == 5.0
             assert _close(mine.state[p]["exp_avg_sq"], ref_opt.state[rp]["exp_avg_sq"], 1e-6, 1e-12)
+        if kind.endswith("amsgrad"):
+            assert _close(mine.state[p]["max_exp_avg_sq"], ref_opt.state[rp]["max_exp_avg_sq"], 1e-6, 1e-12)
 
 
 def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
@@ -446,7 +469,7 @@ def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
     with pytest.raises(TypeError):
         trainer.prepare_weight_sync_method(torch.optim.RMSprop(trainer.main_model.parameters(), lr=0.1))
     with pytest.raises(ValueError):
-        trainer.prepare_weight_sync_method(torch.optim.Adam(trainer.main_model.parameters(), lr=0.1, amsgrad=True))
+        trainer.prepare_weight_sync_method(torch.optim.Adam(trainer.main_model.parameters(), lr=0.1, maximize=True))
     groups = _groups(trainer.main_model)
     groups[0]["momentum"] = 0.5
     with pytest.raises(ValueError):

@@ -54,7 +54,7 @@ def _opt_dict(kind):
     if kind == "sgd":
         return dict(kind="sgd", momentum=0.9, dampening=0.0, nesterov=False,
                     groups=[dict(lr=0.1, weight_decay=0.0), dict(lr=0.1, weight_decay=1e-4)])
-    return dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
+    return dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8, amsgrad=kind.endswith("amsgrad"),
                 groups=[dict(lr=5e-4, weight_decay=0.0), dict(lr=5e-4, weight_decay=0.05)])
 
 
@@ -63,7 +63,7 @@ def _torch_optimizer(kind, params):
               {"params": [p for p in params if p.dim() > 1], "weight_decay": 1e-4 if kind == "sgd" else 0.05}]
     if kind == "sgd":
         return torch.optim.SGD(groups, lr=0.1, momentum=0.9)
-    return torch.optim.AdamW(groups, lr=5e-4)
+    return torch.optim.AdamW(groups, lr=5e-4, amsgrad=kind.endswith("amsgrad"))
 
 
 def _layout(shapes):
@@ -83,6 +83,14 @@ def _layout(shapes):
 @pytest.mark.parametrize("mode", ["per_bucket", "deferred", "batched"])
 def test_optimizer_in_the_hook_is_bit_exact_with_the_oracle(gpu, kind, gdt, mode):
     _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2))
+
+
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["per_bucket", "deferred"])
+def test_optimizer_in_the_hook_with_amsgrad(gpu, gdt, mode):
+    """AdamW(amsgrad=True) bound to the hooks: the running maximum lives in a third state arena laid out like
+    the bucket, ``optimizer.state[p]['max_exp_avg_sq']`` shows it."""
+    _hooks_with_optimizer(gpu, "adamw_amsgrad", gdt, mode, (4, 2, 2))
 
 
 @pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
@@ -145,10 +153,12 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
     p_h = [torch.cat([t.reshape(-1) for t in bucket]) for bucket in init]
     s1_h = [torch.zeros_like(p) for p in p_h]
     s2_h = [torch.zeros_like(p) for p in p_h]
+    s3_h = [torch.zeros_like(p) if kind.endswith("amsgrad") else None for p in p_h]
     gate = [threading.Event() for _ in range(len(SHAPES))]
     for step in range(1, 4):
         local.lr_scale = (1.0, math.sqrt(20 / 8), 0.75)[step - 1]              # the adaptive-batching modifier moves
-        host = [[(torch.randn(n, generator=torch.Generator().manual_seed(1000 * step + 10 * b + k)) * 1e-3).to(gdt)
+        std = 1e-3 if step == 1 or not kind.endswith("amsgrad") else 5e-5     # amsgrad: the moment falls below its maximum
+        host = [[(torch.randn(n, generator=torch.Generator().manual_seed(1000 * step + 10 * b + k)) * std).to(gdt)
                  for k in range(K)] for b, (_, _, n) in enumerate(layouts)]
         for g in gate:
             g.clear()
@@ -184,7 +194,8 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
         want_stats = st.step % st.interval == 0
         for b, (offs, bounds, n) in enumerate(layouts):
             agg_h, rows_h = O.sync_step(host[b], batches, [(0, n, bounds)], opt, p_h[b], s1_h[b], s2_h[b], step=step,
-                                        first_step=(step == 1), want_stats=want_stats, lr_scale=local.lr_scale)
+                                        first_step=(step == 1), want_stats=want_stats, lr_scale=local.lr_scale,
+                                        state3=s3_h[b])
             agg_d = bufs[b][0] if gdt == torch.float32 else local.aggregate_of(b)
             if keep:
                 assert _same(agg_d, agg_h), (step, b, "aggregate")
@@ -199,6 +210,8 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
                 else:
                     assert _same(state["exp_avg"], s1_h[b][sl]) and _same(state["exp_avg_sq"], s2_h[b][sl]), (step, b, i)
                     assert int(state["step"]) == step
+                    if kind.endswith("amsgrad"):
+                        assert _same(state["max_exp_avg_sq"], s3_h[b][sl]), (step, b, i, "maximum")
                 for k in range(1, K):
                     assert _same(replicas[k][b][i].data, p.data), (step, b, i, k, "replica")
             for k in range(1, K):                                               # the peers' buckets are only read
@@ -379,7 +392,7 @@ def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
 def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
     """ShardGNMTAdam.step(gradients) outside any hook: torch.nn.utils.clip_grad_norm_ over the gradients
     of the call, then torch.optim.Adam, is the library statement of the same step (1e-6; the oracle's
-    sequence bit for bit)."""
+    sequence bit for bit), and the gradient tensors of the call hold the clipped values afterwards."""
     from jabas_amd import optim
     from jabas_amd.train.trainer import tag_parameter_indices
     torch.manual_seed(0)
@@ -417,7 +430,11 @@ def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
             off += n
             assert _same(p.data, p_h[i]), (step, i)
             assert torch.allclose(p.data, rp.data, rtol=1e-6, atol=1e-8), (step, i)
-        assert _same(flat, host)                                                # the gradient buffers are left alone
+        # the gradients handed over are clipped in place, as clip_grad_norm_for_overlap leaves them
+        # (examples/gnmt/seq2seq/train/shard_optimizer.py:75-76); untouched when the norm is under the bound
+        assert _same(flat, clipped), step
+        assert torch.allclose(flat, torch.cat([rp.grad.reshape(-1) for rp in ref.parameters()]), rtol=1e-6, atol=1e-12)
+        assert (step == 2) == _same(flat, host)
     with pytest.raises(ValueError, match="param_groups"):
         optim.ShardGNMTAdam([{"params": params[:1]}, {"params": params[1:]}], grad_clip=1.0)
 

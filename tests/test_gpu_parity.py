@@ -271,6 +271,92 @@ def test_adam_steps(gpu, hp):
         assert same == tot
 
 
+@pytest.mark.parametrize("hp", [
+    dict(lr=5e-4, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8, adamw=True),
+    dict(lr=2e-3, weight_decay=0.0, betas=(0.9, 0.999), eps=1e-8, adamw=False),
+    dict(lr=1e-3, weight_decay=1e-2, betas=(0.8, 0.99), eps=1e-6, adamw=False),
+])
+def test_amsgrad_steps(gpu, hp):
+    """Adam / AdamW with amsgrad (examples/gnmt/seq2seq/train/shard_optimizer.py:58-66,79-90): weights, both
+    moments and the running maximum bit-identical to the oracle over six steps whose gradients shrink after
+    the second, so that the maximum and the moment part ways; a NaN gradient element poisons its maximum."""
+    from jabas_amd import sync
+    n, steps = 70001, 6
+    p_h, m_h, v_h, x_h = _host_state(n, 3), torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    p_d, m_d, v_d, x_d = _dev(p_h, gpu), _dev(m_h, gpu), _dev(v_h, gpu), _dev(x_h, gpu)
+    for s in range(1, steps + 1):
+        g = _host_grads(1, n, 170 + s, std=5e-3 if s <= 2 else 2e-4)[0]
+        if s == steps:
+            g[12345] = float("nan")
+        O.adam_step(p_h, g, m_h, v_h, step=s, vmax=x_h, **hp)
+        sync.adam_step(_dev(g, gpu), p_d, m_d, v_d, step=s, max_exp_avg_sq=x_d, **hp)
+        torch.cuda.synchronize()
+        for name, a, b in (("p", p_d, p_h), ("m", m_d, m_h), ("v", v_d, v_h), ("max", x_d, x_h)):
+            a = a.detach().cpu()
+            nan = torch.isnan(b)                            # (a NaN's payload is not part of the contract)
+            assert torch.equal(torch.isnan(a), nan) and int(nan.sum()) == (1 if s == steps else 0), (s, name)
+            same, tot = _same_bits(a[~nan], b[~nan])
+            assert same == tot, (s, name, same, tot)
+    assert float((x_h > v_h).float().mean()) > 0.5 and bool(torch.isnan(x_d[12345])) and bool(torch.isnan(p_d[12345]))
+
+
+@pytest.mark.parametrize("K,dtype,kind,stats", [(3, torch.float32, "adam", "full"), (8, torch.bfloat16, "adamw", "similarity"),
+                                                (4, torch.float32, "adamw", False), (16, torch.bfloat16, "adam", "full"),
+                                                (9, torch.float32, "adamw", "similarity")])
+def test_sync_bucket_fused_amsgrad(gpu, K, dtype, kind, stats):
+    """The fused launch with the amsgrad kinds: aggregate, statistics, weights, moments, maximum and the
+    replica all from one pass, bit-identical to the oracle (statistics within their bar)."""
+    from jabas_amd import sync
+    n = 200003
+    skew = 3 if dtype == torch.bfloat16 else 1
+    bounds = ((0, 1), (5, 0), (1029, 1), (70000, 0), (70001, 1), (150000, 0))
+    opt = dict(ADAMW if kind == "adamw" else ADAM, amsgrad=True)
+    p_h, s1_h, s2_h, s3_h = _host_state(n, 5), torch.zeros(n), torch.zeros(n), torch.zeros(n)
+    agg_d = _dev(torch.zeros(n), gpu, skew)
+    p_d, s1_d, s2_d, s3_d = (_dev(t, gpu, skew) for t in (p_h, s1_h, s2_h, s3_h))
+    fan = [_dev(torch.zeros(n), gpu, skew)]
+    dg = [_dev(torch.zeros(n, dtype=dtype), gpu, skew) for _ in range(K)]
+    span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d, state1=s1_d, state2=s2_d, state3=s3_d, fanout=fan, bounds=bounds)
+    ws = sync.Workspace.for_span(n, dtype, gpu)
+    for step in (1, 2, 3, 4):
+        hg = _host_grads(K, n, 460 + K + step, std=5e-3 if step <= 2 else 2e-4, dtype=dtype)
+        for d, h in zip(dg, hg):
+            d.copy_(h)
+        args = sync.make_step_args(BATCHES[K], dtype, stats=stats, opt=opt, step=step)
+        row = sync.sync_bucket(span, args, workspace=ws)
+        torch.cuda.synchronize()
+        agg_h, rows_h = O.sync_step(hg, BATCHES[K], [(0, n, bounds)], opt, p_h, s1_h, s2_h, step=step,
+                                    want_stats=bool(stats), state3=s3_h)
+        assert torch.equal(_bits(agg_d), _bits(agg_h)), f"step {step}"
+        for name, a, b in (("p", p_d, p_h), ("m", s1_d, s1_h), ("v", s2_d, s2_h), ("max", s3_d, s3_h), ("replica", fan[0], p_h)):
+            same, tot = _same_bits(a, b)
+            assert same == tot, (step, name, same, tot)
+        if stats:
+            rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+            width = 4 + K if stats == "full" else 4
+            assert _close(row.cpu()[1:width], rows_h[0][1:width], rtol, 1e-30)[0]
+            assert abs(float(row[0].cpu() - rows_h[0][0])) <= rtol * float(torch.sqrt(rows_h[0][1] * rows_h[0][2]))
+    assert float((s3_h > s2_h).float().mean()) > 0.1          # the maximum did part from the moment
+
+
+def test_amsgrad_needs_its_maximum_and_is_not_replayed_from_a_block(gpu):
+    from jabas_amd import sync, _lib as L
+    n = 4096
+    g = [torch.zeros(n, device=gpu)]
+    p, m, v = (torch.zeros(n, device=gpu) for _ in range(3))
+    opt = dict(ADAM, amsgrad=True)
+    args = sync.make_step_args((1,), torch.float32, opt=opt, step=1)
+    assert args.opt_kind == L.OPT_ADAM_AMSGRAD
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.sync_bucket(sync.SpanSpec(g, param=p, state1=m, state2=v), args)
+    assert e.value.status == L.ERR_NULL
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.SyncPlan([sync.SpanSpec(g, param=p, state1=m, state2=v)], L.OPT_ADAMW_AMSGRAD)
+    assert e.value.status == L.ERR_NULL
+    with pytest.raises(ValueError):
+        sync.opt_kind(dict(SGD, amsgrad=True))
+
+
 # ------------------------------------------------------------------ fused, single bucket
 @pytest.mark.parametrize("K,dtype,opt", [(2, torch.float32, SGD), (4, torch.float32, ADAMW),
                                          (3, torch.float32, ADAM), (8, torch.bfloat16, ADAMW),

@@ -294,6 +294,56 @@ def test_adamw_decay_is_decoupled():
     assert torch.count_nonzero(m) == 0 and torch.count_nonzero(v) == 0     # decay never enters the moments
 
 
+@pytest.mark.parametrize("hp", ADAM_CASES)
+def test_amsgrad_matches_c_bitwise_and_torch_optim(hp):
+    """amsgrad as ShardGNMTAdam.step threads it into F.adam (examples/gnmt/seq2seq/train/shard_optimizer.py:58-66,
+    79-90): both restatements bit for bit, torch.optim.Adam / AdamW(amsgrad=True) as the library routine. The
+    gradients shrink after the second step, so the second moment falls below its maximum and a denominator
+    taken from the moment instead of the maximum would show."""
+    n, steps = 3001, 6
+    p_o, p_c, p_plain = _state(n, 3), _state(n, 3), _state(n, 3)
+    p_t = torch.nn.Parameter(_state(n, 3))
+    m_o, v_o, x_o, m_c, v_c, x_c = (torch.zeros(n) for _ in range(6))
+    m_p, v_p = torch.zeros(n), torch.zeros(n)
+    cls = torch.optim.AdamW if hp["adamw"] else torch.optim.Adam
+    opt = cls([p_t], lr=hp["lr"], weight_decay=hp["weight_decay"], betas=hp["betas"], eps=hp["eps"], foreach=False,
+              amsgrad=True)
+    history = []
+    for s in range(1, steps + 1):
+        g = _grads(1, n, 170 + s, std=5e-3 if s <= 2 else 2e-4)[0]
+        O.adam_step(p_o, g, m_o, v_o, step=s, vmax=x_o, **hp)
+        OC.adam_step(p_c, g, m_c, v_c, step=s, vmax=x_c, **hp)
+        O.adam_step(p_plain, g, m_p, v_p, step=s, **hp)
+        history.append(v_o.clone())
+        p_t.grad = g.clone()
+        opt.step()
+        for a, b in ((p_o, p_c), (m_o, m_c), (v_o, v_c), (x_o, x_c)):
+            assert torch.equal(_bits(a), _bits(b))
+        assert torch.equal(_bits(x_o), _bits(torch.stack(history).max(dim=0).values))      # the running maximum, exactly
+    assert torch.allclose(p_o, p_t.detach(), rtol=1e-6, atol=1e-9)
+    assert torch.allclose(m_o, opt.state[p_t]["exp_avg"], rtol=1e-6, atol=2e-10)
+    assert torch.allclose(v_o, opt.state[p_t]["exp_avg_sq"], rtol=1e-6, atol=1e-16)
+    assert torch.allclose(x_o, opt.state[p_t]["max_exp_avg_sq"], rtol=1e-6, atol=1e-16)
+    if hp["adamw"] or hp["weight_decay"] == 0:            # (L2 decay feeds the weights back into the moments)
+        assert torch.equal(_bits(v_o), _bits(v_p)) and torch.equal(_bits(m_o), _bits(m_p))     # the moments are Adam's own
+    assert (x_o > v_o).float().mean() > 0.5                 # the maximum is what the last steps mostly divided by ...
+    assert not torch.allclose(p_o, p_plain, rtol=1e-6, atol=1e-9)                          # ... and it shows in the weights
+
+
+def test_amsgrad_maximum_propagates_nan_like_torch_maximum():
+    n = 8
+    g = torch.full((n,), 1e-3)
+    g[3] = float("nan")
+    outs = []
+    for mod in (O, OC):
+        p, m, v, x = torch.ones(n), torch.zeros(n), torch.zeros(n), torch.full((n,), 1e-3)
+        mod.adam_step(p, g, m, v, lr=1e-3, weight_decay=0.0, betas=(0.9, 0.999), eps=1e-8, step=1, adamw=False, vmax=x)
+        assert torch.isnan(x[3]) and torch.isnan(p[3]) and not torch.isnan(x[[0, 1, 2, 4, 5, 6, 7]]).any()
+        assert torch.equal(x[:3], torch.full((3,), 1e-3))    # the old maximum stands where the moment is below it
+        outs.append((p, x))
+    assert torch.equal(_bits(outs[0][0]), _bits(outs[1][0])) and torch.equal(_bits(outs[0][1]), _bits(outs[1][1]))
+
+
 # --------------------------------------------------------------------- composite step
 def test_sync_step_composes_pieces_per_span_and_group():
     K, n = 3, 5000
