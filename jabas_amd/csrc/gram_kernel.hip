@@ -357,7 +357,12 @@ __global__ void __launch_bounds__(kBlock) gram_bf16_mfma_kernel(const SpanDev sp
     }
     // fp64 sums of the wave: [pair * 4 + i][16-lane row * 4 + j]
     __shared__ double sums[kWaves][P * 4][16];
-    for (int i = lane; i < P * 64; i += 64) (&sums[wave][0][0])[i] = 0.0;
+    double* const wave_sums = &sums[0][0][0] + static_cast<size_t>(wave) * (P * 64);     // this wave's P * 64 sums, flat
+    for (int i = lane; i < P * 64; i += 64) wave_sums[i] = 0.0;
+    // the zeros are written by other lanes than the ones that add to them later: order the two within the wave
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     f32x4 acc[P];
 #pragma unroll
     for (int p = 0; p < P; ++p) acc[p] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};

@@ -148,7 +148,7 @@ def opt_from_torch_optimizer(optimizer):
 class VSWSyncTrainer:
     def __init__(self, gpu, local_batch_sizes, opt=None, interval=100, grad_dtype=torch.float32,
                  param_groups_func=None, similarity_target=None, controller=None, clip_norm=None,
-                 share_weights=True):
+                 share_weights=True, keep_grads=False):
         """opt: hyperparameter dictionary, or None when an optimizer object follows through
         ``prepare_weight_sync_method`` (the reference's order of calls).
 
@@ -157,8 +157,15 @@ class VSWSyncTrainer:
         VSW reads weights while the step runs (the launch waits for all K backward passes), so one copy serves
         them all: nothing is written per replica (4 (K - 1) bytes per element and step saved: 28 of 72 for
         eight VSWs) and K - 1 copies of the model's weights stay out of HBM. False: one weight arena per
-        VSW, refreshed by the launch (the reference's layout: separate modules with separate storage)."""
+        VSW, refreshed by the launch (the reference's layout: separate modules with separate storage).
+
+        keep_grads: after ``step()`` the ``.grad`` of the main model's parameters shows the synchronised gradient
+        (views of the aggregate arena, the clipped values under a norm bound), as the reference leaves the averaged
+        gradient in the main VSW's ``.grad`` for code that logs gradient norms or inspects gradients after the step;
+        the launch then writes the aggregate (4 more bytes per element). Default: ``.grad`` is None after a step and
+        the aggregate is written nowhere."""
         self.share_weights = bool(share_weights)
+        self.keep_grads = bool(keep_grads)
         self.gpu = torch.device("cuda", gpu) if isinstance(gpu, int) else torch.device(gpu)
         self.local_batch_sizes = tuple(local_batch_sizes)
         self.num_models = len(self.local_batch_sizes)
@@ -237,7 +244,7 @@ class VSWSyncTrainer:
         # clipped step the clipped aggregate) back
         self.engine = VSWFlatSync(specs, self.local_batch_sizes, grad_dtype=self.grad_dtype, opt=self.opt,
                                   device=self.gpu, n_fanout=0 if self.share_weights else max(1, self.num_models - 1),
-                                  keep_clipped_grads=False, write_aggregate=False)
+                                  keep_clipped_grads=self.keep_grads, write_aggregate=self.keep_grads)
         if self.num_models == 1 and not self.share_weights:
             self.engine.reconfigure(self.local_batch_sizes)       # keeps the fan-out slot for later replicas
         self.local_models = [model] + [copy.deepcopy(model) for _ in range(self.num_models - 1)]
@@ -418,6 +425,9 @@ class VSWSyncTrainer:
             raise ValueError(f"expected {self.num_models} local batches, got {len(data)}")
         cur = torch.cuda.current_stream(self.gpu)
         losses = []
+        if self.keep_grads and self.accumulated == 0:
+            for p in self._params.get(0, ()):            # the last step's synchronised gradient: backward must not add to it
+                p.grad = None
         for k, ((x, y), m, s) in enumerate(zip(data, self.local_models, self.model_streams)):
             s.wait_stream(cur)
             with torch.cuda.stream(s):
@@ -464,6 +474,9 @@ class VSWSyncTrainer:
                                 accumulations=max(1, self.accumulated))
         self.accumulated = 0
         self.sync_step += 1
+        if self.keep_grads:
+            for i, p in enumerate(self._params.get(0) or list(self.main_model.parameters())):
+                p.grad = self.engine.agg_view(i).view(p.shape)
         self._step_tensor.fill_(float(self.engine.step_count))
         if self.local_schedulers:
             self.main_optimizer._opt_called = True      # what torch's schedulers look at to see that an update preceded them

@@ -249,9 +249,11 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
         assert plans[0] is not None and plans[1] is plans[0] and plans[2] is plans[0]
 
 
-@pytest.mark.parametrize("share", [True, False])
+@pytest.mark.parametrize("share,keep_grads", [(True, False), (False, False), (True, True)])
 @pytest.mark.parametrize("kind", ["sgd", "adamw"])
-def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind, share):
+def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind, share, keep_grads):
+    """keep_grads: after a step the main model's .grad holds the synchronised gradient, as the reference leaves it
+    in the main VSW; by default .grad is None after a step (the launch writes the aggregate nowhere)."""
     from jabas_amd.train import VSWSyncTrainer
     batches = (6, 2)
     if kind == "sgd":
@@ -261,7 +263,8 @@ def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind, share):
         opt = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
                    groups=[dict(lr=1e-3, weight_decay=0.0), dict(lr=1e-3, weight_decay=0.05)])
     crit = torch.nn.MSELoss()
-    trainer = VSWSyncTrainer(gpu, batches, opt, interval=2, param_groups_func=_groups, share_weights=share)
+    trainer = VSWSyncTrainer(gpu, batches, opt, interval=2, param_groups_func=_groups, share_weights=share,
+                             keep_grads=keep_grads)
     trainer.prepare_stream_parallel(_mlp(3), crit)
     # one weight arena for every VSW's model, or one per VSW refreshed by the launch
     assert len(trainer.engine.fanout) == (0 if share else 1)
@@ -295,6 +298,10 @@ def test_trainer_end_to_end_matches_plain_torch_step(gpu, kind, share):
         torch.cuda.synchronize()
         for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
             assert _close(p, rp, 1e-6, 1e-7), f"{kind} step {step}"
+            if keep_grads:
+                assert _close(p.grad, rp.grad, 1e-5, 1e-7), f"{kind} step {step}: synchronised gradient"
+            else:
+                assert p.grad is None
         for m in trainer.local_models[1:]:
             for p, q in zip(m.parameters(), trainer.main_model.parameters()):
                 assert torch.equal(p, q)                       # replicas refreshed by the same launch

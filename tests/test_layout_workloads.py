@@ -79,3 +79,26 @@ def test_per_tensor_spans_cover_every_tensor_once():
     lay = L.FlatLayout(specs, per_tensor_spans=True)
     assert len(lay.spans) == len(specs)
     assert sum(n for _, n, _, _ in lay.spans) == lay.numel
+
+
+def test_tracked_hbm_traffic_covers_every_workload_at_its_algorithmic_bytes():
+    """bench.py's roofline.traffic is read from a tracked summary of two rocprofv3 counter runs: it must name every
+    workload the package defines, at the algorithmic bytes bench.py prices that workload with (a workload whose
+    shape or byte count moved needs the counters taken again), and the traffic may not be below the algorithmic
+    bytes nor more than a few per cent above."""
+    import json
+    import os
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    sys.path.insert(0, root)
+    import bench
+    from jabas_amd import workloads as W
+    with open(os.path.join(root, bench.TRAFFIC_FILE)) as f:
+        table = json.load(f)["workloads"]
+    for cfg in W.configs():
+        assert cfg.name in table, f"{bench.TRAFFIC_FILE} lacks {cfg.name}"
+        want = sum(s.numel for s in cfg.specs) * bench.algorithmic_bytes_per_elem(cfg)
+        entry = table[cfg.name]
+        assert abs(entry["algorithmic_bytes"] - want) <= 1e-5 * want, (cfg.name, entry["algorithmic_bytes"], want)
+        assert 1.0 <= entry["hbm_bytes_per_launch"] / want <= 1.02, cfg.name
+        assert bench.measured_traffic(cfg.name) == entry["hbm_bytes_per_launch"]

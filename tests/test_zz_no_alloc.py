@@ -1,13 +1,27 @@
-"""The entry point that allocates nothing, ``jabas_sync_bucket_static``, against
-``jabas_sync_bucket`` through the C ABI: aggregate, weights, optimizer state and the statistics
-row bit for bit, on two calls in a row, the second over a smaller span (the static scratch still
-holds the first call's partial rows). Collected last: a failure here must not hide other tests."""
+"""The entry point that allocates nothing, ``jabas_sync_bucket_static``, through the C ABI: against the CPU
+oracle (aggregate, weights and optimizer state bit for bit, statistics within their bar) and against
+``jabas_sync_bucket`` (everything bit for bit, the statistics row included), on two calls in a row, the second
+over a smaller span (the static scratch still holds the first call's partial rows). Collected last: a failure
+here must not hide other tests."""
 import ctypes as C
 
 import pytest
 import torch
 
+from oracle import oracle as O
+
 pytestmark = pytest.mark.gpu
+
+
+def _oracle(n, K, seed, dtype, kind, step):
+    """The same call on the host: (aggregate, weights, state1, state2, statistics row)."""
+    grads, p, m, v = _case("cpu", n, K, seed, dtype, kind)
+    bounds = ((0, 1), (n // 3, 0)) if n >= 3 else ()
+    opt = dict(kind=kind, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
+               groups=[dict(lr=5e-4, weight_decay=0.05), dict(lr=5e-4, weight_decay=0.0)])
+    agg, rows = O.sync_step(grads, tuple(range(K, 0, -1)), [(0, n, bounds)], opt, p, m, v if kind != "sgd" else None,
+                            step=step, first_step=False, want_stats=True)
+    return agg, p, m, v, rows[0]
 
 
 def _case(gpu, n, K, seed, dtype, opt_kind):
@@ -58,6 +72,16 @@ def test_static_entry_matches_sync_bucket_on_two_calls_the_second_smaller(gpu, K
                                b.view(torch.int64) if b.dtype == torch.float64 else b.view(torch.int32))
             assert same, (call, n, name)
         assert float(got[5][3]) > 0.0
+        # and against the oracle itself, not only through the other entry point
+        agg_h, p_h, m_h, v_h, row_h = _oracle(n, K, 31 + call, dtype, kind, 2 + call)
+        names = ("aggregate", "weights", "state1") + (("state2",) if kind != "sgd" else ())
+        for name, a, b in zip(names, got, (agg_h, p_h, m_h, v_h)):
+            assert torch.equal(a.cpu().view(torch.int32), b.view(torch.int32)), (call, n, name, "oracle")
+        assert torch.equal(got[4].cpu().view(torch.int32), p_h.view(torch.int32)), (call, n, "fan-out", "oracle")
+        row = got[5].cpu()
+        rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+        assert torch.allclose(row[1:4 + K], row_h[1:4 + K], rtol=rtol, atol=0.0), (call, n, "statistics", "oracle")
+        assert abs(float(row[0] - row_h[0])) <= rtol * float(torch.sqrt(row_h[1] * row_h[2])), (call, n, "dot", "oracle")
 
 
 def test_static_entry_without_statistics_and_size_limit(gpu):
