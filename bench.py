@@ -91,8 +91,14 @@ def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0, write
     return engines, numel, copies
 
 
+_last_host_us = 0.0
+
+
 def timed_region(fn, steps, warmup, torch):
-    """ms per call of fn(i) over exactly `steps` calls, HIP events on the current stream."""
+    """ms per call of fn(i) over exactly `steps` calls, HIP events on the current stream. The host time the
+    calls themselves took (queueing only: measured before the closing synchronisation) is left in
+    ``host_us_of_last_region()``."""
+    global _last_host_us
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
@@ -102,9 +108,14 @@ def timed_region(fn, steps, warmup, torch):
     for i in range(steps):
         fn(i)
     e1.record()
+    _last_host_us = (time.perf_counter() - t0) * 1e6 / steps
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     return max(e0.elapsed_time(e1), 1e-6) / steps, wall_ms / steps
+
+
+def host_us_of_last_region():
+    return _last_host_us
 
 
 def rate(bytes_per_step, ms):
@@ -322,6 +333,7 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
     level = "similarity" if cfg.stats else False
     # timed region: exactly `steps` steps, back to back on one stream
     ms_per_step, wall_ms = timed_region(lambda i: engines[i % n].step(stats=level), steps, warmup, torch)
+    host_us_direct = host_us_of_last_region()
     # per-launch durations (instrumentation pass, outside the timed region): one event pair per step
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for i, (a, b) in enumerate(evs):
@@ -334,7 +346,7 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         workload=cfg.name, elements=numel, K=cfg.K, batches=list(cfg.batches), grad_dtype=cfg.grad_dtype,
         optimizer=cfg.opt["kind"], stats="similarity" if cfg.stats else "none", spans=engines[0].plan.n_span,
         bytes_per_elem=algorithmic_bytes_per_elem(cfg), GB_per_step=bytes_per_step / 1e9,
-        wall_ms_per_step=wall_ms, buffer_copies=copies,
+        wall_ms_per_step=wall_ms, host_us_per_step=host_us_direct, buffer_copies=copies,
         launch_ms_mean=sum(launch_ms) / len(launch_ms), launch_ms_median=launch_ms[len(launch_ms) // 2],
         launch_ms_min=launch_ms[0])
     res.update(rate(bytes_per_step, ms_per_step))
@@ -350,7 +362,10 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         # block (Adam's bias correction moves every step): one graph launch per step instead of the step's launches
         graphed = [e.capture(stats=level) for e in engines]
         ms, wall = timed_region(lambda i: graphed[i % n].replay(), steps, warmup, torch)
-        res["recorded_step"] = dict(rate(bytes_per_step, ms), wall_ms_per_step=wall)
+        # what a replay trades: the GPU pays the scalar-refresh kernel and the graph launch, the host queues one
+        # graph launch (plus that refresh) instead of the step's launches
+        res["recorded_step"] = dict(rate(bytes_per_step, ms), wall_ms_per_step=wall,
+                                    host_us_per_step=host_us_of_last_region(), host_us_per_step_direct=host_us_direct)
         del graphed
     if extras:
         hsteps, hwarm = max(5, steps // 2), max(10, warmup)
@@ -490,6 +505,61 @@ def launch_modes(cfg, device, steps, torch):
     return out
 
 
+def reference_profile_metrics(device, steps, torch):
+    """The two figures of this path that the reference itself records (IIDPTrainer.profile_step, written to
+    examples/resnet50/quickstart/cluster_comp_profile_data/*/*/resnet50_*_comp_profile.json:1): ``update_time`` =
+    the optimizer step over the main VSW's parameters, ``copy_time`` = the copy of the main VSW's weights to the
+    other K - 1 VSWs, ResNet-50, SGD with momentum, K = 1..4. Here the step is ShardSGD.step() over the 161
+    tensors (one planned launch) and the copy is part of that launch (``attach_replicas``): update_time_ms is the
+    launch without replicas, copy_time_ms what K - 1 replicas add to it. Beside them, on the same GPU, the
+    reference's own structure with stock torch: torch.optim.SGD's single-tensor loop and one ``copy_`` per
+    parameter and replica (jabas/train/trainer.py:530-534). ms per call, HIP events, gradients in place."""
+    from jabas_amd import workloads as W
+    from jabas_amd import optim
+    cfg = W.config("resnet50")
+    hp = dict(lr=cfg.opt["groups"][0]["lr"], momentum=cfg.opt["momentum"])
+
+    def params(seed):
+        gen = torch.Generator(device=device).manual_seed(seed)
+        return [torch.nn.Parameter(torch.randn(s.numel, generator=gen, device=device) * 0.05) for s in cfg.specs]
+
+    def groups(ps):
+        return [dict(params=[p for p, s in zip(ps, cfg.specs) if s.group == gi], weight_decay=g["weight_decay"])
+                for gi, g in enumerate(cfg.opt["groups"])]
+
+    out, base = {}, None
+    for K in (1, 2, 3, 4):
+        main, stock = params(1), params(1)
+        for ps in (main, stock):
+            for p in ps:
+                p.grad = torch.randn_like(p) * cfg.grad_std
+        replicas = [[torch.nn.Parameter(p.detach().clone()) for p in main] for _ in range(K - 1)]
+        stock_replicas = [[torch.nn.Parameter(p.detach().clone()) for p in stock] for _ in range(K - 1)]
+        mine = optim.ShardSGD(groups(main), **hp)
+        if replicas:
+            mine.attach_replicas(main, *replicas)
+        theirs = torch.optim.SGD(groups(stock), foreach=False, **hp)
+
+        def copy_loop(_):
+            with torch.no_grad():
+                for rep_ in stock_replicas:
+                    for src, dst in zip(stock, rep_):
+                        dst.data.copy_(src.data)
+
+        n = max(10, steps)
+        fused = timed_region(lambda i: mine.step(), n, 5, torch)[0]
+        update_stock = timed_region(lambda i: theirs.step(), max(5, n // 5), 2, torch)[0]
+        copy_stock = timed_region(copy_loop, max(5, n // 5), 2, torch)[0] if K > 1 else 0.0
+        if K == 1:
+            base = fused
+        out[str(K)] = dict(update_time_ms=base, copy_time_ms=max(0.0, fused - base), update_and_copy_one_launch_ms=fused,
+                           stock_torch_update_time_ms=update_stock, stock_torch_copy_time_ms=copy_stock)
+        del main, stock, replicas, stock_replicas, mine, theirs
+        torch.cuda.empty_cache()
+    return dict(model="resnet50", optimizer="sgd momentum 0.9", tensors=len(cfg.specs),
+                elements=sum(s.numel for s in cfg.specs), per_K=out)
+
+
 def cpu_baseline(cfg, torch, budget_s):
     """Reference-structured unfused step on the host cores: 1 warm-up step (allocates the optimizer state),
     then at least 3 whole steps and as many more as fit about budget_s, all threads; then the same step
@@ -599,10 +669,14 @@ def main():
               f"{r['pct_hbm_peak']:.1f} % of HBM peak{extra}; hooks per bucket "
               f"{r['hook_path_per_bucket_ms']['ms_per_step']:.4f} ms, batched "
               f"{r['hook_path_batched_64MiB_ms']['ms_per_step']:.4f} ms, deferred "
-              f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms", file=sys.stderr, flush=True)
+              f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms; one launch per bucket back to back on 1 / 2 launch "
+              f"streams {r['bucket_launches_back_to_back_ms']['1']:.4f} / {r['bucket_launches_back_to_back_ms']['2']:.4f} ms; "
+              f"K hook threads: exposed sync {r['hook_path_threads_2_launch_streams']['exposed_sync_ms']:.4f} ms",
+              file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results and not args.no_extras:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
                                                                       args.steps, torch)
+    ref_metrics = None if args.no_all or args.no_extras else reference_profile_metrics(device, args.steps, torch)
     copy_gbps = copy_rate(device, args.steps, torch)
     stat_launches = None if args.no_all or args.no_extras else statistics_launches(device, args.steps, torch)
     gram = None if args.no_all or args.no_extras else gram_launches(device, args.steps, torch)
@@ -636,6 +710,11 @@ def main():
         "cpu_baseline": head.get("cpu_baseline"),
         "copy_GBps": copy_gbps,
         "workloads": list(results.values()),
+        "reference_profile_metrics_resnet50": ref_metrics,
+        # the configuration the first round's headline was quoted on (ViT-B/16, K = 4, fp32 gradients, full statistics
+        # rows), so that figures stay comparable from round to round whatever the headline workload is
+        "like_for_like": {"vit_b16_K4_f32_full_statistics_rows":
+                          results.get("vit_b16", {}).get("step_with_per_vsw_norms")},
         "statistics_launches": stat_launches,
         "gram_launches": gram,
     }
