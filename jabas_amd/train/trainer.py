@@ -85,14 +85,20 @@ def create_stream_for_optimizer(device=None):
 
 
 def prepare_overlap_optimizer_with_ddp(local_models, states, hooks, optimizer, local):
-    """jabas/train/trainer.py:327-333 for one GPU: a launch stream of its own for ``local`` (the GPU's
-    LocalBucketSync) unless it has one, the optimizer hook on VSW 0, every other VSW's hook as it is.
+    """jabas/train/trainer.py:327-333 for one GPU: launch streams of its own for ``local`` (the GPU's
+    LocalBucketSync) unless it has them, ``local`` installed as the device's meeting point with the replicas
+    registered in VSW order, the optimizer hook on VSW 0, every other VSW's hook as it is.
     ``local_models`` are the K DistributedDataParallel replicas (built with
     ``gradient_as_bucket_view=True``: the fused launch writes the aggregate into the bucket, and only a
     ``.grad`` that is a view of the bucket sees it)."""
+    p = next(iter(local_models[0].parameters()))
     if local._sync_stream is None:
-        p = next(iter(local_models[0].parameters()))
         local._sync_stream = create_stream_for_optimizer(p.device)
+    # states built without a handle of ours (the reference's: a plain GradientSimilarityState and None for every
+    # other VSW, jabas/train/trainer.py:452-468) find the meeting point through the device and the VSW index
+    # through the replica a bucket's parameters belong to
+    local.install(p.device)
+    local.register_replicas(local_models)
     for i, (model, state, hook) in enumerate(zip(local_models, states, hooks)):
         if getattr(model, "gradient_as_bucket_view", True) is False:
             raise ValueError("build the DistributedDataParallel replicas with gradient_as_bucket_view=True")
