@@ -378,9 +378,15 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         res["bucket_launches_back_to_back_ms"] = {
             str(ls): bucket_launches(cfg, engines[0], device, hsteps, hwarm, torch, ls) for ls in (1, 2, 3)}
         # the same hooks as training calls them: K threads on K streams with backward-like work between the buckets
+        # (a leg of K host threads: whatever goes wrong in it is reported in its place, not instead of the line)
         for ls in (1, 2):
-            res[f"hook_path_threads_{ls}_launch_stream{'s' if ls > 1 else ''}"] = hook_path_threads(
-                cfg, engines[0], device, hsteps, max(3, hwarm // 3), torch, ls, engine_ms=ms_per_step)
+            key = f"hook_path_threads_{ls}_launch_stream{'s' if ls > 1 else ''}"
+            try:
+                res[key] = hook_path_threads(cfg, engines[0], device, hsteps, max(3, hwarm // 3), torch, ls,
+                                             engine_ms=ms_per_step)
+            except Exception as exc:
+                torch.cuda.synchronize()
+                res[key] = dict(error=f"{type(exc).__name__}: {exc}")
     if cfg.name == "gnmt" and extras:
         # global-norm clipping (examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
         # coefficient on the device, then the update over the scaled aggregate
@@ -671,7 +677,7 @@ def main():
               f"{r['hook_path_batched_64MiB_ms']['ms_per_step']:.4f} ms, deferred "
               f"{r['hook_path_deferred_ms']['ms_per_step']:.4f} ms; one launch per bucket back to back on 1 / 2 launch "
               f"streams {r['bucket_launches_back_to_back_ms']['1']:.4f} / {r['bucket_launches_back_to_back_ms']['2']:.4f} ms; "
-              f"K hook threads: exposed sync {r['hook_path_threads_2_launch_streams']['exposed_sync_ms']:.4f} ms",
+              f"K hook threads: exposed sync {r['hook_path_threads_2_launch_streams'].get('exposed_sync_ms', float('nan')):.4f} ms",
               file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results and not args.no_extras:
         results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
