@@ -421,6 +421,16 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
                                                       bytes_per_elem=algorithmic_bytes_per_elem(cfg) - 4)
         del engines
         torch.cuda.empty_cache()
+    if extras and cfg.opt["kind"] != "sgd":
+        # the same step with amsgrad (examples/gnmt/seq2seq/train/shard_optimizer.py:58-66): the running maximum of
+        # the second moment is one more state stream, 8 more bytes per element
+        ams = cfg._replace(opt=dict(cfg.opt, amsgrad=True))
+        engines, _, _ = build_engines(ams, device, torch)
+        ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
+        ams_bytes = numel * (algorithmic_bytes_per_elem(cfg) + 8)
+        res["step_with_amsgrad"] = dict(rate(ams_bytes, ms), bytes_per_elem=ams_bytes // numel)
+        del engines
+        torch.cuda.empty_cache()
     if cfg.name == "gnmt" and extras:
         engines, _, _ = build_engines(cfg, device, torch, independent_masks=True)
         ms, _ = timed_region(lambda i: engines[i % len(engines)].step(stats=level), steps, warmup, torch)
