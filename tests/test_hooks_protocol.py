@@ -433,3 +433,37 @@ def test_more_peers_than_the_meeting_point_expects():
         assert len(seen) == 1 and "more peer replicas" in seen[0]
     finally:
         local.uninstall()
+
+
+def test_a_failed_launch_surfaces_in_the_hand_over_that_ends_the_step():
+    """With the step ended by the last bucket's last hand-over, what went wrong in one of the step's launches is
+    raised there (in training: inside that VSW's backward pass), once, and the next step starts clean."""
+    calls = []
+
+    def launcher(bucket_index, tensors, want_stats):
+        calls.append(bucket_index)
+        if bucket_index == 0 and len(calls) == 1:
+            raise RuntimeError("launch refused")
+        return None
+    local = LocalBucketSync([1, 1], launcher=launcher)
+    grads = [torch.ones(2), torch.ones(2)]
+    for b in (0, 1):
+        local.publish(0, b, grads[0], bucket=DDPBucket(b, grads[0], 2))
+    local.publish(1, 0, grads[1], bucket=DDPBucket(0, grads[1], 2))           # bucket 0 complete: its launch fails
+    with pytest.raises(RuntimeError, match="launch refused"):
+        local.publish(1, 1, grads[1], bucket=DDPBucket(1, grads[1], 2))       # the step ends here
+    assert local.step_count == 0 and local.pending() == []
+    local.finish_step()                                                        # nothing left to report
+    for k in (0, 1):
+        for b in (0, 1):
+            local.publish(k, b, grads[k], bucket=DDPBucket(b, grads[k], 2))
+    assert local.step_count == 1 and calls == [0, 1, 0, 1]
+
+
+def test_auto_finish_can_be_switched_off():
+    local = LocalBucketSync([1, 1], launcher=Recorder(), auto_finish=False)
+    for k in (0, 1):
+        local.publish(k, 0, torch.ones(2), bucket=DDPBucket(0, torch.ones(2), 1))
+    assert local.step_count == 0 and local.launched == 1
+    local.finish_step()
+    assert local.step_count == 1
