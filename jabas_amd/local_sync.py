@@ -676,13 +676,17 @@ class LocalBucketSync:
             call.with_opt, call.clipped = with_opt, clipped
             with self._lock:
                 self._calls[bucket_index] = call
-            if self._own_launcher and not self.deferred and not self.batch_bytes and not clipped and main is not None:
-                self._describe_native(bucket_index, tensors, call)
+            describe = self._own_launcher and not self.deferred and not self.batch_bytes and not clipped and main is not None
+        else:
+            describe = False
         if call.with_opt:
             with self._lock:
                 self.launched_with_opt += 1
         if not call.clipped:
-            return call.run(self._step_args(tensors[0].dtype, want_stats, call.with_opt), stream=main)
+            row = call.run(self._step_args(tensors[0].dtype, want_stats, call.with_opt), stream=main)
+            if describe:                                # after the launch: the description continues from the row it wrote
+                self._describe_native(bucket_index, tensors, call)
+            return row
         row = call.run(self._step_args(tensors[0].dtype, True, False), stream=main)
         sync.clip_coef(row, self.grad_clip, out=call.coef, stream=main)
         call.update.run(self._step_args(torch.float32, False, True, grad_scale=call.coef, batches=(1,)), stream=main)

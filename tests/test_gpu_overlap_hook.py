@@ -526,3 +526,35 @@ def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
         assert local.native_launches - native_before == (1 if want_native else 0), step
         native_before = local.native_launches
         st.step += 1
+
+
+def test_statistics_rows_keep_alternating_when_a_bucket_moves_to_the_native_meeting_point(gpu):
+    """A bucket's statistics launches alternate between two device rows, so that the row a step handed out stays
+    valid until the second-next statistics step. The first launch of a bucket goes through the Python path, the
+    following ones through the native meeting point: the alternation continues across the two."""
+    from jabas_amd.local_sync import LocalBucketSync
+    K, batches, n = 2, (3, 1), 40_001
+    local = LocalBucketSync(batches)
+    streams = [torch.cuda.Stream(gpu) for _ in range(K)]
+    bufs = [torch.zeros(n, device=gpu) for _ in range(K)]
+    handed, want = [], []
+
+    for step in range(4):
+        host = [torch.randn(n, generator=torch.Generator().manual_seed(77 * step + k)) * 1e-3 for k in range(K)]
+        want.append(O.stats(host, batches))
+        for k in (1, 0):
+            with torch.cuda.stream(streams[k]):
+                bufs[k].copy_(host[k].to(gpu))
+                local.publish(k, 0, bufs[k], want_stats=True, on_done=handed.append if k == 0 else None)
+        local.finish_step()
+        torch.cuda.synchronize()
+        assert local.native_launches == step                      # the first launch describes the bucket, the rest are native
+        assert len(handed) == step + 1
+        # this step's row and the one before it are both intact; the one before that has been written over
+        for back in (0, 1):
+            if step - back >= 0:
+                got = handed[step - back].cpu()
+                assert torch.allclose(got[1:4], want[step - back][1:4], rtol=1e-6, atol=0.0), (step, back)
+        if step >= 2:
+            assert handed[step].row.data_ptr() == handed[step - 2].row.data_ptr()
+            assert handed[step].row.data_ptr() != handed[step - 1].row.data_ptr()
