@@ -522,7 +522,7 @@ def test_trainer_accumulates_micro_batches_between_steps(gpu):
             assert _close(p, rp, 1e-6, 1e-7), step
 
 
-@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+@pytest.mark.parametrize("kind", ["sgd", "adamw", "adamw_amsgrad"])
 def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     """state_dict() after 3 steps, through a file, into a fresh trainer (other initial weights, another
     number of VSWs): the next 3 steps give the bits of the uninterrupted run. The optimizer entry is in
@@ -537,7 +537,7 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
         if kind == "sgd":
             o = torch.optim.SGD(_groups(t.main_model), lr=0.05, momentum=0.9, foreach=False)
         else:
-            o = torch.optim.AdamW(_groups(t.main_model), lr=1e-3, foreach=False)
+            o = torch.optim.AdamW(_groups(t.main_model), lr=1e-3, foreach=False, amsgrad=kind.endswith("amsgrad"))
         sch = torch.optim.lr_scheduler.LambdaLR(o, lambda it: 1.0 / (1.0 + 0.25 * it))
         t.prepare_weight_sync_method(o, sch)
         return t, o
@@ -569,11 +569,13 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     for m in b.local_models[1:]:
         for pm, pb in zip(m.parameters(), b.main_model.parameters()):
             assert torch.equal(pm, pb)
-    keys = ("momentum_buffer",) if kind == "sgd" else ("exp_avg", "exp_avg_sq")
+    keys = ("momentum_buffer",) if kind == "sgd" else ("exp_avg", "exp_avg_sq") + (("max_exp_avg_sq",) if kind.endswith("amsgrad") else ())
+    arenas = {"momentum_buffer": b.engine.state1, "exp_avg": b.engine.state1, "exp_avg_sq": b.engine.state2,
+              "max_exp_avg_sq": b.engine.state3}
     for pa, pb in zip(a.main_model.parameters(), b.main_model.parameters()):
         for key in keys:
             assert torch.equal(opt_a.state[pa][key], opt_b.state[pb][key])
-            arena = b.engine.state2 if key == "exp_avg_sq" else b.engine.state1      # still views of the arenas
+            arena = arenas[key]                                                      # still views of the arenas
             assert opt_b.state[pb][key].untyped_storage().data_ptr() == arena.untyped_storage().data_ptr()
     assert opt_a.param_groups[0]["lr"] == opt_b.param_groups[0]["lr"]
 
@@ -581,7 +583,7 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     plain = _mlp(5).to(gpu)
     plain.load_state_dict(b.state_dict()["model"])
     stock = (torch.optim.SGD(_groups(plain), lr=0.05, momentum=0.9) if kind == "sgd"
-             else torch.optim.AdamW(_groups(plain), lr=1e-3))
+             else torch.optim.AdamW(_groups(plain), lr=1e-3, amsgrad=kind.endswith("amsgrad")))
     stock.load_state_dict(b.state_dict()["optimizer"])
     for pp, pb in zip(plain.parameters(), b.main_model.parameters()):
         assert torch.equal(stock.state[pp][keys[0]], opt_b.state[pb][keys[0]])
@@ -592,7 +594,8 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     assert c.engine.step_count == (1 if kind == "sgd" else 6)
     for pc, pb in zip(c.main_model.parameters(), b.main_model.parameters()):
         assert torch.equal(pc, pb)
-        assert torch.equal(opt_c.state[pc][keys[0]], opt_b.state[pb][keys[0]])
+        for key in keys:
+            assert torch.equal(opt_c.state[pc][key], opt_b.state[pb][key])
 
 
 def test_trainer_with_bf16_gradient_buckets(gpu):
