@@ -389,7 +389,8 @@ def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
     assert clipped_any and kept_any
 
 
-def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
+@pytest.mark.parametrize("amsgrad", [False, True])
+def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu, amsgrad):
     """ShardGNMTAdam.step(gradients) outside any hook: torch.nn.utils.clip_grad_norm_ over the gradients
     of the call, then torch.optim.Adam, is the library statement of the same step (1e-6; the oracle's
     sequence bit for bit), and the gradient tensors of the call hold the clipped values afterwards."""
@@ -399,12 +400,13 @@ def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
     model = tag_parameter_indices(torch.nn.Sequential(torch.nn.Linear(40, 50), torch.nn.Linear(50, 7)).to(gpu))
     ref = torch.nn.Sequential(torch.nn.Linear(40, 50), torch.nn.Linear(50, 7)).to(gpu)
     ref.load_state_dict(model.state_dict())
-    mine = optim.ShardGNMTAdam(model.parameters(), lr=2e-3, grad_clip=5e-3)
-    theirs = torch.optim.Adam(ref.parameters(), lr=2e-3, foreach=False)
+    mine = optim.ShardGNMTAdam(model.parameters(), lr=2e-3, grad_clip=5e-3, amsgrad=amsgrad)
+    theirs = torch.optim.Adam(ref.parameters(), lr=2e-3, foreach=False, amsgrad=amsgrad)
     params = list(model.parameters())
     p_h = [p.detach().cpu().clone().reshape(-1) for p in params]
     m_h, v_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
-    opt = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, groups=[dict(lr=2e-3, weight_decay=0.0)])
+    x_h = [torch.zeros_like(p) if amsgrad else None for p in p_h]
+    opt = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, amsgrad=amsgrad, groups=[dict(lr=2e-3, weight_decay=0.0)])
     flat = torch.zeros(sum(p.numel() for p in params), device=gpu)            # one "bucket"
     for step in range(1, 5):
         scale = (1e-3, 1e-6, 1e-3, 1e-2)[step - 1]                             # step 2 stays under the bound
@@ -426,9 +428,11 @@ def test_shard_gnmt_adam_step_clips_like_clip_grad_norm_then_adam(gpu):
         off = 0
         for i, (p, rp) in enumerate(zip(params, ref.parameters())):
             n = p.numel()
-            O.opt_step(opt, 0, p_h[i], clipped[off:off + n], m_h[i], v_h[i], step, step == 1)
+            O.opt_step(opt, 0, p_h[i], clipped[off:off + n], m_h[i], v_h[i], step, step == 1, s3=x_h[i])
             off += n
             assert _same(p.data, p_h[i]), (step, i)
+            if amsgrad:
+                assert _same(mine.state[p]["max_exp_avg_sq"], x_h[i]), (step, i)
             assert torch.allclose(p.data, rp.data, rtol=1e-6, atol=1e-8), (step, i)
         # the gradients handed over are clipped in place, as clip_grad_norm_for_overlap leaves them
         # (examples/gnmt/seq2seq/train/shard_optimizer.py:75-76); untouched when the norm is under the bound
