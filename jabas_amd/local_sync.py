@@ -11,7 +11,14 @@ of that replica's backward on the autograd engine's device thread, which every r
 the GPU shares, so a Future that needed another replica's backward to make progress would
 deadlock. Ordering is by stream instead: the launch waits on an event from every VSW's
 stream, and ``finish_step`` makes every VSW stream wait for the launches (and reports
-anything that went wrong in them) before gradients and weights are reused.
+anything that went wrong in them) before gradients and weights are reused. The step ends by
+itself with the hand-over that completes the replicas' last bucket (``GradBucket.is_last()``),
+so a loop that only registers the hooks calls nothing else.
+
+Hooks that carry no state of ours (the reference registers ``dummy_hook`` with ``state=None``
+and builds the main state without any handle to IIDP's local machinery) find the object through
+the device it was installed for (``install``) and their VSW index through the replica a bucket's
+parameters belong to (``register_replicas``) or the stream they run on.
 
 The "overlap" weight-sync mode (jabas/train/trainer.py:327-333: an optimizer hook on VSW 0
 that updates the weights of a bucket as soon as its gradients are synchronised, on a stream
@@ -423,7 +430,8 @@ class LocalBucketSync:
         queued by whichever VSW hands its bucket over last. Returns a completed Future
         carrying ``value`` (default the tensor). ``bucket``: the bucket object itself, whose
         ``parameters()`` / ``gradients()`` place the weights when an optimizer is bound and whose
-        ``is_last()`` ends the step (``auto_finish``)."""
+        ``is_last()`` ends the step (``auto_finish``). ``_stream``: the VSW's stream when the hand-over is
+        repeated on its behalf by another thread (a bucket leaving the native meeting point)."""
         if not 0 <= k < self.K:
             raise ValueError(f"VSW index {k} outside 0..{self.K - 1}")
         if self._finishing:                    # an implied end of step is running on another thread: let it finish
