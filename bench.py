@@ -360,6 +360,21 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         res["step_without_statistics"] = rate(bytes_per_step, ms)
         ms, _ = timed_region(lambda i: engines[i % n].step(stats="full"), steps, warmup, torch)
         res["step_with_per_vsw_norms"] = rate(bytes_per_step, ms)
+        if cfg.K <= 4:
+            # the worker x worker Gram matrix ("between workers" statistics): out of the step's own launch (pair
+            # products beside the full rows, no byte read twice), against the step followed by a pass of its
+            # own over the K gradient arenas (K * gradient size more bytes per element read)
+            from jabas_amd import sync
+            ms, _ = timed_region(lambda i: engines[i % n].step(stats="gram"), steps, warmup, torch)
+            res["step_with_worker_gram_in_the_launch"] = rate(bytes_per_step, ms)
+            gws = torch.empty(1056 * 256, dtype=torch.float64, device=device)
+
+            def step_then_gram(i):
+                engines[i % n].step(stats="full")
+                sync.gram(engines[i % n].grads, workspace=gws)
+            ms, _ = timed_region(step_then_gram, steps, warmup, torch)
+            res["step_then_worker_gram_pass"] = dict(ms_per_step=ms)
+            del gws
     if extras:
         # the same step recorded once in a HIP graph and replayed with the scalars of the moment in a device
         # block (Adam's bias correction moves every step): one graph launch per step instead of the step's launches

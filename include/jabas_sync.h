@@ -41,6 +41,7 @@ extern "C" {
 #define JABAS_MAX_GROUPS 16     /* optimizer parameter groups per launch              */
 #define JABAS_STATS_STRIDE 20   /* doubles per span in stats_out: 4 + JABAS_MAX_K     */
 #define JABAS_GRAM_MAX_K 16     /* VSWs of one jabas_gram call                        */
+#define JABAS_STATS_GRAM_MAX_K 4 /* VSWs of a launch with JABAS_STATS_GRAM             */
 #define JABAS_GRAM_STRIDE 256   /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
 #define JABAS_STATIC_MAX_NUMEL (1ull << 26)  /* largest span of jabas_sync_bucket_static  */
 #define JABAS_STEP_SCALARS_BYTES 688         /* size of a step-scalar block (jabas_step_scalars_encode) */
@@ -75,8 +76,12 @@ enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAM
  * similarity between the halves and global-norm clipping read (slots DOT_AB .. NORM_AGG of a
  * row; the per-VSW slots are written as 0): the reference's adaptive batching consumes nothing
  * else (jabas/train/trainer.py:470-483), and the kernels that skip the K per-VSW norms keep more
- * loads in flight. FULL adds sum g_k^2 of every VSW. */
-enum { JABAS_STATS_NONE = 0, JABAS_STATS_FULL = 1, JABAS_STATS_SIMILARITY = 2 };
+ * loads in flight. FULL adds sum g_k^2 of every VSW. GRAM adds, to the full row, the products
+ * sum g_a*g_b of every pair of VSWs a < b, i.e. the whole worker x worker Gram matrix from the
+ * pass that aggregates and updates, with no byte read a second time; K <= JABAS_STATS_GRAM_MAX_K
+ * (JABAS_ERR_K beyond: the K*(K-1)/2 extra fp64 sums per thread fit the registers of the fused
+ * kernel up to there; more workers use jabas_gram, a pass of its own over the gradients). */
+enum { JABAS_STATS_NONE = 0, JABAS_STATS_FULL = 1, JABAS_STATS_SIMILARITY = 2, JABAS_STATS_GRAM = 3 };
 
 /* Slots of one stats_out row (JABAS_STATS_STRIDE doubles per span). A = VSWs with
  * half_id 0, B = VSWs with half_id 1; g_A = sum_{k in A} g_k*half_weight_k formed in
@@ -89,6 +94,9 @@ enum {
     JABAS_STAT_NORM_AGG = 3,    /* sum gbar^2 of the aggregate                         */
     JABAS_STAT_NORM_VSW0 = 4    /* + k: sum g_k^2 of VSW k                             */
 };
+/* JABAS_STATS_GRAM: slot of sum g_a*g_b, a < b < K (pairs in the order (0,1), (0,2), ..., (K-2,K-1),
+ * after the K norms); the diagonal of the Gram matrix is the norms. */
+#define JABAS_STAT_PAIR(K, a, b) (JABAS_STAT_NORM_VSW0 + (K) + (a) * (2 * (K) - (a) - 1) / 2 + ((b) - (a) - 1))
 
 /* One contiguous stretch of the flat layout. All buffers hold `numel` elements and are
  * indexed alike. Element e of every fp32 buffer must fall at the same position of a

@@ -16,14 +16,20 @@ MAX_GROUPS = 16
 STATS_STRIDE = 20
 GRAM_MAX_K = 16
 GRAM_STRIDE = 256
+STATS_GRAM_MAX_K = 4
 STATIC_MAX_NUMEL = 1 << 26
 STEP_SCALARS_BYTES = 688
 
 F32, BF16 = 0, 1
 OPT_NONE, OPT_SGD, OPT_ADAM, OPT_ADAMW, OPT_ADAM_AMSGRAD, OPT_ADAMW_AMSGRAD = 0, 1, 2, 3, 4, 5
-STATS_NONE, STATS_FULL, STATS_SIMILARITY = 0, 1, 2
+STATS_NONE, STATS_FULL, STATS_SIMILARITY, STATS_GRAM = 0, 1, 2, 3
 
 STAT_DOT_AB, STAT_NORM_A, STAT_NORM_B, STAT_NORM_AGG, STAT_NORM_VSW0 = 0, 1, 2, 3, 4
+
+
+def stat_pair(K, a, b):
+    """Slot of sum g_a*g_b (a < b < K) in a row of level STATS_GRAM: JABAS_STAT_PAIR of the header."""
+    return STAT_NORM_VSW0 + K + a * (2 * K - a - 1) // 2 + (b - a - 1)
 
 OK = 0
 ERR_NULL, ERR_K, ERR_ALIGN, ERR_DTYPE, ERR_OPT, ERR_GROUP = -1, -2, -3, -4, -5, -6

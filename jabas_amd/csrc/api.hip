@@ -205,7 +205,8 @@ int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
     if (s->grad_dtype != JABAS_F32 && s->grad_dtype != JABAS_BF16) return JABAS_ERR_DTYPE;
     const int oc = opt_class_of(s->opt_kind);
     if (oc < 0) return JABAS_ERR_OPT;
-    if (s->stats < JABAS_STATS_NONE || s->stats > JABAS_STATS_SIMILARITY) return JABAS_ERR_OPT;
+    if (s->stats < JABAS_STATS_NONE || s->stats > JABAS_STATS_GRAM) return JABAS_ERR_OPT;
+    if (s->stats == JABAS_STATS_GRAM && s->K > JABAS_STATS_GRAM_MAX_K) return JABAS_ERR_K;
     memset(a, 0, sizeof(*a));
     uint32_t mask = 0;
     for (int k = 0; k < s->K; ++k) {
@@ -296,7 +297,7 @@ __global__ void __launch_bounds__(kFinalizeBlock) finalize_stats_kernel(const ui
                                                                         uint32_t use_inline, uint32_t stripes,
                                                                         uint32_t in_stripes, uint32_t out_stride,
                                                                         const double* in, double* out) {
-    // input rows are compact (NS = 4 + K doubles each); output rows have out_stride slots, the unused ones 0
+    // input rows are compact (NS doubles each, the width of the level); output rows have out_stride slots, the unused ones 0
     __shared__ double red[kFinalizeBlock / 64][NS];
     const uint32_t s = blockIdx.y, j = blockIdx.x, t = threadIdx.x;
     uint32_t c0, c1, o;
@@ -345,7 +346,8 @@ hipError_t launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32
     return launch_kernel(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
                          a.use_inline, stripes, in_stripes, out_stride, in, out);
 }
-// One instantiation per row width: 4 (similarity sums) and 4 + K, K = 1..16.
+// One instantiation per row width: 4 (similarity sums), 4 + K, K = 1..16, and 4 + K + K(K-1)/2 for K <= 4
+// (7, 10, 14: among the widths of the full rows).
 hipError_t finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
                     uint32_t out_stride, const double* in, double* out) {
     switch (ns) {
@@ -392,7 +394,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
     }
     if (stats) {
         const uint32_t st = stripes_for(max_span_chunks);
-        const int ns = stats == JABAS_STATS_FULL ? 4 + s->K : 4;    // width of the partial rows
+        const int ns = stats_row_width(s->K, stats);                // width of the partial rows
         hipError_t err;
         if (st == 1) {
             err = finalize(ns, dim3(1, a.n_span), stream, a, 1u, 0u, kStatsStride, a.partials, stats_out);
@@ -412,7 +414,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
 
 using namespace jabas;
 
-JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.4 (gfx950)"; }
+JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.5 (gfx950)"; }
 
 JABAS_API const char* jabas_status_string(int status) {
     switch (status) {
@@ -616,8 +618,8 @@ JABAS_API int64_t jabas_plan_chunks(const void* host_blob, int32_t stats) {
     if (!host_blob) return JABAS_ERR_NULL;
     PlanHeader h;
     if (!read_plan_header(host_blob, &h)) return JABAS_ERR_PLAN;
-    if (stats < JABAS_STATS_NONE || stats > JABAS_STATS_SIMILARITY) return JABAS_ERR_OPT;
-    return h.shape[stats].n_chunks;
+    if (stats < JABAS_STATS_NONE || stats > JABAS_STATS_GRAM) return JABAS_ERR_OPT;
+    return h.shape[shape_level(stats)].n_chunks;
 }
 
 JABAS_API size_t jabas_plan_workspace_bytes(const void* host_blob) {
@@ -645,7 +647,7 @@ JABAS_API int jabas_sync_fused(const void* plan_host, const void* plan_dev, cons
     // were validated for that class only
     if (opt_class_of(h.opt_kind) != oc) return JABAS_ERR_PLAN;
     const int stats = args->stats;
-    const PlanShape& ps = h.shape[stats];
+    const PlanShape& ps = h.shape[shape_level(stats)];
     if (ps.block != static_cast<uint32_t>(launch_block(h.K, h.grad_dtype, oc, stats)) ||
         ps.chunk_tiles != static_cast<uint32_t>(launch_chunk_tiles(h.K, h.grad_dtype, oc, stats)))
         return JABAS_ERR_PLAN;

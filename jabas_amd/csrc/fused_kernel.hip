@@ -103,8 +103,10 @@ constexpr uint64_t kNarrowElems = 1ull << 30;
 __host__ __device__ constexpr bool narrow_addressing(int K, int SL) { return SL != 0 && K > 4; }
 
 // Statistics level of a launch: 0 none, 1 the full row (4 + K sums), 2 the four sums of the halves and of
-// the aggregate only (what the cosine similarity and global-norm clipping read).
-template <int K, int SL> struct NStats { static constexpr int value = SL == 1 ? 4 + K : (SL == 2 ? 4 : 1); };
+// the aggregate only (what the cosine similarity and global-norm clipping read), 3 the full row and the
+// products of every pair of workers (the Gram matrix; up to JABAS_STATS_GRAM_MAX_K workers).
+template <int K, int SL> struct NStats { static constexpr int value = stats_row_width(K, SL); };
+constexpr bool per_vsw_norms(int SL) { return SL == JABAS_STATS_FULL || SL == JABAS_STATS_GRAM; }
 
 // Per-thread running sums of the statistics. fp32 gradients: fp64 (a product of two fp32 values is exact
 // in fp64). bf16 gradients: fp32 within the thread's chunk (at most 16 elements), widened to fp64 when the
@@ -210,8 +212,13 @@ __device__ __forceinline__ void compute(const float (&g)[K][N], float (&p)[N], f
                     gb = in_b ? gb + t : gb;
                     ga = in_b ? ga : ga + t;
                 }
-                if constexpr (SL == 1)
+                if constexpr (per_vsw_norms(SL))
                     acc[JABAS_STAT_NORM_VSW0 + k] = stat_fma(g[k][i], g[k][i], acc[JABAS_STAT_NORM_VSW0 + k]);
+                if constexpr (SL == JABAS_STATS_GRAM) {
+#pragma unroll
+                    for (int b = k + 1; b < K; ++b)
+                        acc[JABAS_STAT_PAIR(K, k, b)] = stat_fma(g[k][i], g[b][i], acc[JABAS_STAT_PAIR(K, k, b)]);
+                }
             }
             // fp64 sums: fp32 x fp32 products are exact in fp64, so fma == mul followed by add there.
             acc[JABAS_STAT_DOT_AB] = stat_fma(ga, gb, acc[JABAS_STAT_DOT_AB]);
@@ -589,12 +596,16 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
 #endif
     constexpr unsigned idle = (OPT == OPT_ADAM && !SL && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
     const dim3 block(launch_block(K, DT, OPT, SL));
-    if constexpr (OPT == OPT_SGD || OPT == OPT_ADAM) {
-        if (dyn) return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, true>, dim3(grid), block, idle, stream, a));
+    if constexpr (SL == JABAS_STATS_GRAM && K > JABAS_STATS_GRAM_MAX_K) {
+        return static_cast<int>(hipErrorInvalidValue);              // refused by the front before it gets here
     } else {
-        if (dyn) return static_cast<int>(hipErrorInvalidValue);     // refused by the front before it gets here
+        if constexpr (OPT == OPT_SGD || OPT == OPT_ADAM) {
+            if (dyn) return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, true>, dim3(grid), block, idle, stream, a));
+        } else {
+            if (dyn) return static_cast<int>(hipErrorInvalidValue);     // refused by the front before it gets here
+        }
+        return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, false>, dim3(grid), block, idle, stream, a));
     }
-    return static_cast<int>(launch_kernel(fused_kernel<K, DT, OPT, SL, false>, dim3(grid), block, idle, stream, a));
 }
 
 }  // namespace
@@ -603,33 +614,40 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
 #define JABAS_CAT(a, b) JABAS_CAT_(a, b)
 
 #define JABAS_DISPATCH(FN, ...)                                                              \
-    const int key = opt_class == OPT_AMS ? 18 + (grad_dtype == JABAS_BF16 ? 3 : 0) + stats     \
-                                         : (grad_dtype == JABAS_BF16 ? 9 : 0) + opt_class * 3 + stats; \
+    const int key = (opt_class * 2 + (grad_dtype == JABAS_BF16 ? 1 : 0)) * 4 + stats;           \
     switch (key) {                                                                           \
-        case 0:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 0>(__VA_ARGS__);                    \
-        case 1:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 1>(__VA_ARGS__);                    \
-        case 2:  return FN<JABAS_K, JABAS_F32, OPT_NONE, 2>(__VA_ARGS__);                    \
-        case 3:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 0>(__VA_ARGS__);                     \
-        case 4:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 1>(__VA_ARGS__);                     \
-        case 5:  return FN<JABAS_K, JABAS_F32, OPT_SGD, 2>(__VA_ARGS__);                     \
-        case 6:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 0>(__VA_ARGS__);                    \
-        case 7:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 1>(__VA_ARGS__);                    \
-        case 8:  return FN<JABAS_K, JABAS_F32, OPT_ADAM, 2>(__VA_ARGS__);                    \
-        case 9:  return FN<JABAS_K, JABAS_BF16, OPT_NONE, 0>(__VA_ARGS__);                   \
-        case 10: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 1>(__VA_ARGS__);                   \
-        case 11: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 2>(__VA_ARGS__);                   \
+        case 0: return FN<JABAS_K, JABAS_F32, OPT_NONE, 0>(__VA_ARGS__);                     \
+        case 1: return FN<JABAS_K, JABAS_F32, OPT_NONE, 1>(__VA_ARGS__);                     \
+        case 2: return FN<JABAS_K, JABAS_F32, OPT_NONE, 2>(__VA_ARGS__);                     \
+        case 3: return FN<JABAS_K, JABAS_F32, OPT_NONE, 3>(__VA_ARGS__);                     \
+        case 4: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 0>(__VA_ARGS__);                    \
+        case 5: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 1>(__VA_ARGS__);                    \
+        case 6: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 2>(__VA_ARGS__);                    \
+        case 7: return FN<JABAS_K, JABAS_BF16, OPT_NONE, 3>(__VA_ARGS__);                    \
+        case 8: return FN<JABAS_K, JABAS_F32, OPT_SGD, 0>(__VA_ARGS__);                      \
+        case 9: return FN<JABAS_K, JABAS_F32, OPT_SGD, 1>(__VA_ARGS__);                      \
+        case 10: return FN<JABAS_K, JABAS_F32, OPT_SGD, 2>(__VA_ARGS__);                     \
+        case 11: return FN<JABAS_K, JABAS_F32, OPT_SGD, 3>(__VA_ARGS__);                     \
         case 12: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 0>(__VA_ARGS__);                    \
         case 13: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 1>(__VA_ARGS__);                    \
         case 14: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 2>(__VA_ARGS__);                    \
-        case 15: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 0>(__VA_ARGS__);                   \
-        case 16: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 1>(__VA_ARGS__);                   \
-        case 17: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 2>(__VA_ARGS__);                   \
-        case 18: return FN<JABAS_K, JABAS_F32, OPT_AMS, 0>(__VA_ARGS__);                     \
-        case 19: return FN<JABAS_K, JABAS_F32, OPT_AMS, 1>(__VA_ARGS__);                     \
-        case 20: return FN<JABAS_K, JABAS_F32, OPT_AMS, 2>(__VA_ARGS__);                     \
-        case 21: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 0>(__VA_ARGS__);                    \
-        case 22: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 1>(__VA_ARGS__);                    \
-        case 23: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 2>(__VA_ARGS__);                    \
+        case 15: return FN<JABAS_K, JABAS_BF16, OPT_SGD, 3>(__VA_ARGS__);                    \
+        case 16: return FN<JABAS_K, JABAS_F32, OPT_ADAM, 0>(__VA_ARGS__);                    \
+        case 17: return FN<JABAS_K, JABAS_F32, OPT_ADAM, 1>(__VA_ARGS__);                    \
+        case 18: return FN<JABAS_K, JABAS_F32, OPT_ADAM, 2>(__VA_ARGS__);                    \
+        case 19: return FN<JABAS_K, JABAS_F32, OPT_ADAM, 3>(__VA_ARGS__);                    \
+        case 20: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 0>(__VA_ARGS__);                   \
+        case 21: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 1>(__VA_ARGS__);                   \
+        case 22: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 2>(__VA_ARGS__);                   \
+        case 23: return FN<JABAS_K, JABAS_BF16, OPT_ADAM, 3>(__VA_ARGS__);                   \
+        case 24: return FN<JABAS_K, JABAS_F32, OPT_AMS, 0>(__VA_ARGS__);                     \
+        case 25: return FN<JABAS_K, JABAS_F32, OPT_AMS, 1>(__VA_ARGS__);                     \
+        case 26: return FN<JABAS_K, JABAS_F32, OPT_AMS, 2>(__VA_ARGS__);                     \
+        case 27: return FN<JABAS_K, JABAS_F32, OPT_AMS, 3>(__VA_ARGS__);                     \
+        case 28: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 0>(__VA_ARGS__);                    \
+        case 29: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 1>(__VA_ARGS__);                    \
+        case 30: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 2>(__VA_ARGS__);                    \
+        case 31: return FN<JABAS_K, JABAS_BF16, OPT_AMS, 3>(__VA_ARGS__);                    \
         default: return -1;                                                                  \
     }
 

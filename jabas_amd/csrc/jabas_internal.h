@@ -59,7 +59,8 @@ static_assert(block_ok(JABAS_BLOCK) && block_ok(JABAS_BLOCK_SGD) && block_ok(JAB
 constexpr int kMinChunkTiles = JABAS_CHUNK_TILES_LO;
 constexpr int kMaxChunkTiles = JABAS_CHUNK_TILES_HI;
 // opt_class: 0 none, 1 SGD, 2 Adam/AdamW, 3 Adam/AdamW with amsgrad (launch shapes of class 2);
-// stats: 0 none, 1 full rows, 2 similarity sums. The shape depends
+// stats: 0 none, 1 full rows, 2 similarity sums, 3 full rows + pair products (launch shapes and chunk
+// tables of level 1). The shape depends
 // on what a plan is encoded for (K, gradient dtype, optimizer class) and on the statistics level of the
 // launch; a plan holds one chunk table per shape, so it serves every step.
 __host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_class, int stats) {
@@ -72,6 +73,12 @@ __host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, 
     if (stats == 2) return K > 4 ? JABAS_CHUNK_TILES_SIM_MANYK : JABAS_CHUNK_TILES_SIM_LO;
     if (K > 4) return (stats || opt_class == 0) ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
     return kMinChunkTiles;
+}
+// Statistics level whose launch shape (and chunk table of a plan) a level uses.
+__host__ __device__ constexpr int shape_level(int stats) { return stats == JABAS_STATS_GRAM ? JABAS_STATS_FULL : stats; }
+// Width of the partial rows of a launch: 4 similarity sums, + K norms, + K(K-1)/2 pair products.
+__host__ __device__ constexpr int stats_row_width(int K, int stats) {
+    return stats == JABAS_STATS_FULL ? 4 + K : (stats == JABAS_STATS_GRAM ? 4 + K + K * (K - 1) / 2 : (stats ? 4 : 1));
 }
 constexpr int imin(int a, int b) { return a < b ? a : b; }
 // Fewest elements a chunk of a launch with statistics covers (one partial row per chunk): sizes workspaces.

@@ -12,7 +12,7 @@ import torch
 
 from . import _lib as L
 from .layout import FlatLayout
-from .sync import SpanSpec, SyncPlan, StepScalars, gradient_stats, make_step_args, opt_kind, cosine_from_stats, clip_coef
+from .sync import SpanSpec, SyncPlan, StepScalars, gradient_stats, make_step_args, opt_kind, cosine_from_stats, clip_coef, gram_from_stats
 
 
 class VSWFlatSync:
@@ -138,7 +138,8 @@ class VSWFlatSync:
     def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None, accumulations=1):
         """One sync step over the whole gradient set. Returns the per-span stats tensor
         when ``stats`` is set (True / "full": rows of 4 + K sums; "similarity": the four sums of the halves
-        and of the aggregate, per-VSW slots zero).
+        and of the aggregate, per-VSW slots zero; "gram", up to four VSWs: the full row plus the product of
+        every pair of VSWs' gradients, ``gram(rows)`` makes the matrix of them).
 
         Without ``clip_norm``: one fused launch. With it (global-norm clipping as
         examples/gnmt/seq2seq/train/trainer.py:157-161): aggregate + statistics, the
@@ -215,6 +216,11 @@ class VSWFlatSync:
     @staticmethod
     def cosine(stats):
         return cosine_from_stats(stats)
+
+    def gram(self, stats):
+        """K x K matrix of the products of the VSWs' gradients over the whole set, from the rows of a step with
+        ``stats="gram"`` (float64, on the device)."""
+        return gram_from_stats(stats, self.K)
 
 
 class GraphedStep:

@@ -51,6 +51,10 @@ int main(void) {
     SHOW_OFF(JabasStepArgs, grad_scale);
     SHOW_OFF(JabasStepArgs, scalars_dev);
 
+    /* slots of the pair products in a row of level JABAS_STATS_GRAM, as the header's macro places them */
+    printf("pairs4 %d,%d,%d,%d,%d,%d\n", JABAS_STAT_PAIR(4, 0, 1), JABAS_STAT_PAIR(4, 0, 2), JABAS_STAT_PAIR(4, 0, 3),
+           JABAS_STAT_PAIR(4, 1, 2), JABAS_STAT_PAIR(4, 1, 3), JABAS_STAT_PAIR(4, 2, 3));
+    printf("pairs3 %d,%d,%d\n", JABAS_STAT_PAIR(3, 0, 1), JABAS_STAT_PAIR(3, 0, 2), JABAS_STAT_PAIR(3, 1, 2));
     printf("version %s\n", jabas_sync_version());
     printf("status0 %s\n", jabas_status_string(JABAS_OK));
 

@@ -226,6 +226,13 @@ def test_entry_points_validate_before_launching():
     sp.state3 = 0x7f0000000000 + 21 * (1 << 32)
     ams.scalars_dev = 0x7f0000000000 + 22 * (1 << 32)
     assert lib.jabas_sync_bucket(C.byref(sp), None, C.byref(ams), None, None, 0, None) == L.ERR_OPT
+    # statistics level 'gram' (pair products in the fused launch): up to STATS_GRAM_MAX_K workers; no level beyond it
+    many = L.JabasStepArgs()
+    many.K, many.grad_dtype, many.stats = L.STATS_GRAM_MAX_K + 1, L.F32, L.STATS_GRAM
+    spk = _span(1000, K=L.STATS_GRAM_MAX_K + 1)
+    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
+    many.K, many.stats = 2, L.STATS_GRAM + 1
+    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_OPT
     hid = (C.c_uint8 * 2)(0, 1)
     assert lib.jabas_stats(g, 2, L.F32, w, hid, w, 100, 0x7f0400000000, None, 0, None) == L.ERR_ALIGN
     g[1] = 0x7f0100000000
@@ -277,6 +284,12 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
     assert seen[("chunks_stats", "8")] == ""                 # with statistics: 2048 per chunk -> 3 + 5
     assert int(next(n for (k, n) in seen if k == "workspace")) >= (8 + 2) * L.STATS_STRIDE * 8
     assert ("encode_misaligned", str(L.ERR_ALIGN)) in seen
+    # the ctypes mirror places the pair products of a 'gram' row where the header's macro does: behind the K norms,
+    # in the order (0,1), (0,2), ..., (K-2,K-1), and within the row's JABAS_STATS_STRIDE slots
+    for K, key in ((4, "pairs4"), (3, "pairs3")):
+        want = [L.stat_pair(K, a, b) for a in range(K) for b in range(a + 1, K)]
+        assert ("pairs%d" % K, ",".join(map(str, want))) in seen
+        assert want == list(range(4 + K, 4 + K + K * (K - 1) // 2)) and want[-1] < L.STATS_STRIDE
 
 
 def test_plan_encode_rejects_overlapping_written_buffers():
@@ -335,6 +348,9 @@ def test_launch_shape_follows_what_the_plan_is_encoded_for():
     assert lib.jabas_plan_chunks(blob8.ctypes.data, L.STATS_SIMILARITY) == n // 2048
     _, blob2 = chunks(2, L.F32, L.OPT_SGD)
     assert lib.jabas_plan_chunks(blob2.ctypes.data, L.STATS_SIMILARITY) == n // 2048
+    # the level with pair products launches in the shape of the full rows and uses their chunk table
+    assert lib.jabas_plan_chunks(blob2.ctypes.data, L.STATS_GRAM) == lib.jabas_plan_chunks(blob2.ctypes.data, L.STATS_FULL)
+    assert lib.jabas_plan_chunks(blob2.ctypes.data, L.STATS_GRAM + 1) == L.ERR_OPT
     _, blob = chunks(2, L.F32, L.OPT_SGD)
     assert lib.jabas_plan_workspace_bytes(blob.ctypes.data) >= (n // 2048 + 1) * L.STATS_STRIDE * 8
     args = L.JabasStepArgs()
@@ -479,7 +495,8 @@ def test_plan_encode_against_a_python_statement_of_the_chunking_rule(seed):
     assert lib.jabas_plan_chunks(blob.ctypes.data, 0) == want_chunks[0]
     assert lib.jabas_plan_chunks(blob.ctypes.data, 1) == want_chunks[1]
     assert lib.jabas_plan_chunks(blob.ctypes.data, 2) == want_chunks[2]
-    assert lib.jabas_plan_chunks(blob.ctypes.data, 3) == L.ERR_OPT
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 3) == want_chunks[1]        # pair products: the shape of the full rows
+    assert lib.jabas_plan_chunks(blob.ctypes.data, 4) == L.ERR_OPT
 
 
 def test_rendezvous_calls_validate_their_arguments():

@@ -180,11 +180,14 @@ def test_shard_optimizers_refresh_the_other_replicas_in_the_same_launch(gpu, kin
         mine.attach_replicas(list(main.parameters())[1:], list(rep1.parameters())[1:])
 
 
+@pytest.mark.parametrize("level", ["full", "gram"])
 @pytest.mark.parametrize("deferred", [False, True])
-def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
+def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred, level):
     """K hook threads on K streams hand their buckets over in different orders. Per-bucket mode: the
     last arrival queues that bucket's launch. Deferred mode: nothing is queued until finish_step, which
-    queues one planned launch over all buckets (built once, reused while DDP hands over the same buffers)."""
+    queues one planned launch over all buckets (built once, reused while DDP hands over the same buffers).
+    Level 'gram': the rows also carry the products of every pair of VSWs' gradients (the Gram matrix over
+    all buckets against the float64 oracle's)."""
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
 
@@ -199,7 +202,7 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
             return self._t
 
     K, batches, sizes = 3, (4, 2, 2), [40001, 7, 250000]
-    local = LocalBucketSync(batches, deferred=deferred, stats_level="full")
+    local = LocalBucketSync(batches, deferred=deferred, stats_level=level)
     st = H.GradientSimilarityState(None, 4, None, [], 1).attach_local(local)
     main_hook = H.similimarity_allreduce_hook(H.subgroup_allreduce_hook)
     streams = [torch.cuda.Stream(gpu) for _ in range(K)]
@@ -243,6 +246,14 @@ def test_k_vsw_rendezvous_with_streams_and_threads(gpu, deferred):
             assert _close(rows[b][:4 + K], want[:4 + K], 1e-6, 0.0)
         whole = O.cosine_from_rows(torch.stack([O.stats(host[b], batches) for b in range(len(sizes))]))
         assert H.cosine_similarity_from_placeholder(st.grad_placeholder) == pytest.approx(whole, rel=1e-9)
+        width = 4 + K + (K * (K - 1) // 2 if level == "gram" else 0)
+        assert all(torch.count_nonzero(r[width:]) == 0 for r in rows.values())
+        if level == "gram":
+            from jabas_amd import sync
+            got = sync.gram_from_stats(torch.stack([rows[b] for b in range(len(sizes))]), K)
+            want = O.gram([torch.cat([host[b][k] for b in range(len(sizes))]) for k in range(K)])
+            scale = torch.sqrt(torch.outer(torch.diagonal(want), torch.diagonal(want)))
+            assert bool(((got - want).abs() <= 1e-11 * scale).all())
         st.grad_placeholder.clear()
         st.step += 1
     if deferred:

@@ -155,6 +155,81 @@ def test_similarity_level_rows(gpu, K, dtype, rtol):
         assert torch.equal(_bits(m_d), _bits(m_h)) and torch.equal(_bits(v_d), _bits(v_h))
 
 
+@pytest.mark.parametrize("K", [1, 2, 3, 4])
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-11), (torch.bfloat16, 1e-5)])
+@pytest.mark.parametrize("opt", [None, SGD, ADAMW], ids=["aggregate", "sgd", "adamw"])
+def test_gram_level_rows(gpu, K, dtype, rtol, opt):
+    """Statistics level 3: the full row plus the product of every pair of workers, out of the launch that
+    aggregates and steps. Row against the float64 oracle (the four sums and the norms as at the full level,
+    the pair slots against the Gram matrix), pair order as the header's JABAS_STAT_PAIR, slots beyond the row
+    zero, and the aggregate and the optimizer step of the same launch bit-exact."""
+    from jabas_amd import sync, _lib as L
+    for n, skew in ((5, 0), (4099, 1), (300007, 0), (1 << 21, 2), (4099, 45)):
+        print(f"gram level K={K} {dtype} n={n} skew={skew}", flush=True)
+        hg = _host_grads(K, n, 90 + K, std=5e-4, dtype=dtype)
+        dg = [_dev(t, gpu, skew) for t in hg]
+        out = _dev(torch.zeros(n), gpu, skew)
+        p_h = torch.randn(n, generator=torch.Generator().manual_seed(3)) * 0.05
+        m_h, v_h = torch.zeros(n), torch.zeros(n)
+        if opt is None:
+            span = sync.SpanSpec(dg, agg_out=out)
+        else:
+            p_d, m_d, v_d = _dev(p_h, gpu, skew), _dev(m_h, gpu, skew), _dev(v_h, gpu, skew)
+            span = sync.SpanSpec(dg, agg_out=out, param=p_d, state1=m_d, state2=v_d if opt is ADAMW else None)
+        args = sync.make_step_args(BATCHES[K], dtype, stats="gram", opt=opt, step=1, first_step=True)
+        assert args.stats == L.STATS_GRAM
+        row = sync.sync_bucket(span, args).cpu()
+        torch.cuda.synchronize()
+        want = O.stats(hg, BATCHES[K])
+        G = O.gram(hg)
+        width = 4 + K + K * (K - 1) // 2
+        assert _close(row[1:4 + K], want[1:4 + K], rtol, 1e-30)[0], f"K={K} n={n}: {row} vs {want}"
+        assert abs(float(row[0] - want[0])) <= rtol * float(torch.sqrt(want[1] * want[2])) + 1e-30
+        slot = 4 + K
+        for a in range(K):
+            for b in range(a + 1, K):
+                assert L.stat_pair(K, a, b) == slot
+                # a pair product cancels: its error is measured against |g_a| |g_b|
+                assert abs(float(row[slot] - G[a, b])) <= rtol * float(torch.sqrt(G[a, a] * G[b, b])) + 1e-30, (K, n, a, b)
+                slot += 1
+        assert slot == width and torch.count_nonzero(row[width:]) == 0
+        got = sync.gram_from_stats(row, K)
+        assert torch.equal(got, got.t()) and torch.equal(torch.diagonal(got), row[4:4 + K])
+        if opt is None:
+            assert torch.equal(_bits(out), _bits(O.aggregate(hg, BATCHES[K])))
+        else:
+            agg_h, _ = O.sync_step(hg, BATCHES[K], [(0, n, ())], opt, p_h, m_h, v_h if opt is ADAMW else None,
+                                   step=1, first_step=True, want_stats=False)
+            assert torch.equal(_bits(out), _bits(agg_h)) and torch.equal(_bits(p_d), _bits(p_h))
+            assert torch.equal(_bits(m_d), _bits(m_h))
+            if opt is ADAMW:
+                assert torch.equal(_bits(v_d), _bits(v_h))
+
+
+def test_gram_level_limits_and_the_separate_pass(gpu):
+    """More than STATS_GRAM_MAX_K workers are refused before anything is launched; the fused sums agree with
+    jabas_gram's own pass over the same buffers (fp32 gradients: both exact products and fp64 sums)."""
+    from jabas_amd import sync, _lib as L
+    n = 1_000_003
+    hg = _host_grads(5, n, 97)
+    dg = [_dev(t, gpu, 3) for t in hg]
+    out = _dev(torch.zeros(n), gpu, 3)
+    before = out.clone()
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.sync_bucket(sync.SpanSpec(dg, agg_out=out), sync.make_step_args(BATCHES[5], torch.float32, stats="gram"))
+    assert e.value.status == L.ERR_K
+    assert torch.equal(out, before)
+    with pytest.raises(ValueError):
+        sync.gram_from_stats(torch.zeros(L.STATS_STRIDE, dtype=torch.float64), 5)
+    row = sync.sync_bucket(sync.SpanSpec(dg[:4], agg_out=out), sync.make_step_args(BATCHES[4], torch.float32, stats="gram"))
+    fused = sync.gram_from_stats(row, 4).cpu()
+    apart = sync.gram(dg[:4]).cpu()
+    scale = torch.sqrt(torch.outer(torch.diagonal(apart), torch.diagonal(apart)))
+    assert bool(((fused - apart).abs() <= 1e-12 * scale).all())
+    again = sync.sync_bucket(sync.SpanSpec(dg[:4], agg_out=out), sync.make_step_args(BATCHES[4], torch.float32, stats="gram"))
+    assert torch.equal(again.cpu().view(torch.int64), row.cpu().view(torch.int64))
+
+
 def test_stats_run_to_run_deterministic(gpu):
     from jabas_amd import sync
     hg = _host_grads(4, 3_000_001, 41)

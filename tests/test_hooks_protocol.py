@@ -270,8 +270,15 @@ def test_statistics_levels_and_their_names():
     assert [sync.stats_level(x) for x in (None, False, 0)] == [L.STATS_NONE] * 3
     assert [sync.stats_level(x) for x in (True, 1, "full")] == [L.STATS_FULL] * 3
     assert [sync.stats_level(x) for x in (2, "similarity")] == [L.STATS_SIMILARITY] * 2
+    assert [sync.stats_level(x) for x in (3, "gram")] == [L.STATS_GRAM] * 2
     with pytest.raises(ValueError):
         sync.stats_level("everything")
+    assert LocalBucketSync([1] * 4, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM
+    with pytest.raises(ValueError, match="up to 4"):
+        LocalBucketSync([1] * 5, launcher=Recorder(), stats_level="gram")
+    row = torch.arange(L.STATS_STRIDE, dtype=torch.float64)
+    G = sync.gram_from_stats(torch.stack([row, row]), 3)          # slots 4..6 the norms, 7, 8, 9 the pairs (0,1) (0,2) (1,2)
+    assert G.tolist() == [[8.0, 14.0, 16.0], [14.0, 10.0, 18.0], [16.0, 18.0, 12.0]]
     assert LocalBucketSync([1, 1], launcher=Recorder()).stats_level == L.STATS_SIMILARITY
     assert LocalBucketSync([1, 1], launcher=Recorder(), stats_level="full").stats_level == L.STATS_FULL
     args = sync.make_step_args((3, 1), torch.float32, stats="similarity")
