@@ -176,6 +176,28 @@ def test_full_size_configuration(gpu, name):
     agg1 = a.agg.clone()
     r2 = a.step(stats=True).cpu().clone()
     assert torch.equal(r1.view(torch.int64), r2.view(torch.int64))       # same plan, same bits
+    if cfg.K <= 4:
+        # the worker x worker products out of the same launch: the row's other slots keep their bits; the pair sums
+        # equal a float64 library reduction; and the sums of the halves and of the aggregate are the quadratic
+        # forms of the Gram matrix in the weights (up to the fp32 rounding of the aggregated elements)
+        K = cfg.K
+        r3 = a.step(stats="gram").cpu().clone()
+        assert torch.equal(r3[:, :4 + K].view(torch.int64), r1[:, :4 + K].view(torch.int64))
+        G = a.gram(r3).cpu()
+        for i in range(K):
+            for j in range(i + 1, K):
+                want = (a.grads[i].double() * a.grads[j].double()).sum().item()
+                assert abs(G[i, j].item() - want) <= stat_rel * (norms[i] * norms[j]) ** 0.5
+        wv, half, whv = O.batch_weights(cfg.batches)
+        wv = torch.tensor(wv, dtype=torch.float64)
+        wa = torch.tensor([x if h == 0 else 0.0 for x, h in zip(whv, half)], dtype=torch.float64)
+        wb = torch.tensor([x if h == 1 else 0.0 for x, h in zip(whv, half)], dtype=torch.float64)
+        tot = r3.sum(0)
+        assert float(wv @ G @ wv) == pytest.approx(tot[3].item(), rel=1e-5)
+        assert float(wa @ G @ wa) == pytest.approx(tot[1].item(), rel=1e-5)
+        if K > 1:
+            assert float(wb @ G @ wb) == pytest.approx(tot[2].item(), rel=1e-5)
+            assert abs(float(wa @ G @ wb) - tot[0].item()) <= 1e-5 * (tot[1].item() * tot[2].item()) ** 0.5
     for k in range(cfg.K):
         a.grads[k].mul_(4.0)
     a.step(stats=False)
