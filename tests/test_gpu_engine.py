@@ -271,6 +271,7 @@ ADAMW = dict(kind="adamw", betas=(0.9, 0.999), eps=1e-8,
     (ADAM, torch.float32, (3, 2, 1), True),
     (SGD, torch.float32, (4, 2, 2), False),
     (SGD, torch.bfloat16, (2,) * 9, True),
+    (ADAMW, torch.bfloat16, (5, 3, 2, 2), "gram"),
 ])
 def test_recorded_step_replays_with_the_scalars_of_the_moment(gpu, opt, dtype, batches, stats):
     """A step recorded ONCE in a HIP graph, replayed from the very first step on (SGD's first-step flag, Adam's
@@ -318,6 +319,10 @@ def test_recorded_step_replays_with_the_scalars_of_the_moment(gpu, opt, dtype, b
             rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
             width = 4 if stats == "similarity" else 4 + K
             assert _close(rows[:, :width], rows_h[:, :width], rtol, 1e-30)
+            if stats == "gram":                                    # the recorded launch leaves the pair products too
+                want = O.gram([torch.cat([g[o:o + n] for o, n, _ in spans]) for g in host["g"]])
+                scale = torch.sqrt(torch.outer(torch.diagonal(want), torch.diagonal(want)))
+                assert bool(((eng.gram(rows).cpu() - want).abs() <= 1e-5 * scale).all())
 
 
 def test_recorded_clipped_step_and_reconfigure(gpu):
