@@ -147,9 +147,8 @@ def hook_path(cfg, eng, device, steps, warmup, torch, deferred, batch_bytes=0, l
     for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
         sl = slice(off, off + numel)
         bucket_slices.append(sl)
-        pbs[b] = dict(param=eng.param[sl], state1=None if eng.state1 is None else eng.state1[sl],
-                      state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds,
-                      agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
+        pbs[b] = dict(param=eng.param[sl], bounds=bounds, agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl],
+                      **eng.state_of_span(off, numel))
     stream = torch.cuda.Stream(device)
     local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, deferred=deferred, stream=stream,
                             batch_bytes=batch_bytes, launch_streams=launch_streams)
@@ -191,9 +190,8 @@ def bucket_launches(cfg, eng, device, steps, warmup, torch, launch_streams):
     for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
         sl = slice(off, off + numel)
         calls.append(sync.BucketCall(sync.SpanSpec(
-            [g[sl] for g in eng.grads], agg_out=eng.agg[sl], param=eng.param[sl],
-            state1=None if eng.state1 is None else eng.state1[sl],
-            state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds)))
+            [g[sl] for g in eng.grads], agg_out=eng.agg[sl], param=eng.param[sl], bounds=bounds,
+            **eng.state_of_span(off, numel))))
     streams = [torch.cuda.Stream(device) for _ in range(launch_streams)]
     cur = torch.cuda.current_stream(device)
     level = "similarity" if cfg.stats else False
@@ -250,9 +248,8 @@ def hook_path_threads(cfg, eng, device, steps, warmup, torch, launch_streams, ba
     for b, (off, numel, bounds, _bucket) in enumerate(eng.layout.spans):
         sl = slice(off, off + numel)
         bucket_slices.append(sl)
-        pbs[b] = dict(param=eng.param[sl], state1=None if eng.state1 is None else eng.state1[sl],
-                      state2=None if eng.state2 is None else eng.state2[sl], bounds=bounds,
-                      agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl])
+        pbs[b] = dict(param=eng.param[sl], bounds=bounds, agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl],
+                      **eng.state_of_span(off, numel))
     local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, stream=torch.cuda.Stream(device),
                             launch_streams=launch_streams)
     local.step_count = eng.step_count

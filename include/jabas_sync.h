@@ -111,7 +111,23 @@ enum {
  * agg_out may be exactly one of the fp32 gradient buffers (in-place bucket update); apart
  * from that every written buffer (agg_out, param, state1, state2, state3, fanout) must be disjoint
  * from every other buffer of the span, else JABAS_ERR_ALIAS. Overlap between different
- * spans of one plan is the caller's responsibility. Unused pointers are NULL. */
+ * spans of one plan is the caller's responsibility. Unused pointers are NULL.
+ *
+ * Interleaved moments (state_block_log2 != 0; Adam kinds only, JABAS_ERR_OPT otherwise): Adam's moments are
+ * state only the optimizer touches, so where they live in HBM is this library's to choose, and one arena
+ * that alternates blocks of T = 2^state_block_log2 elements of exp_avg and of exp_avg_sq (then of
+ * max_exp_avg_sq for the ..._AMSGRAD kinds), [T of exp_avg][T of exp_avg_sq]..., streams 2-6 % faster than two
+ * (three) arrays of their own (measured with T = 8192 and 16384, 32 and 64 KiB blocks, on the K = 4 fp32 and
+ * K = 8 bf16 AdamW kernels): a workgroup's reads and writes of the moments then fall next to each other in
+ * memory instead of at unrelated addresses. The span names its place in such an arena: state1 = address of
+ * its first element's exp_avg, state_block_pos = that element's position inside its block (< T), state2 ==
+ * state1 + T floats, state3 == state1 + 2 T floats (amsgrad), and state1 - 4 * state_block_pos, the start of
+ * the block group, a multiple of 16 bytes (JABAS_ERR_ALIGN otherwise; a multiple of 256 for the fast element
+ * grid). T from 2^8 to 2^24. Element i of the span has its exp_avg at float index
+ * t + (ways - 1) * (t - t mod T), t = state_block_pos + i, from the start of the block group, ways = 2 or 3.
+ * The alias rule treats everything from state1 to the last element's last moment as one written buffer.
+ * No reference counterpart (torch keeps one tensor per parameter and moment,
+ * examples/gnmt/seq2seq/train/shard_optimizer.py:50-66). */
 typedef struct JabasSpan {
     const void* grads[JABAS_MAX_K];     /* K gradient buffers (fp32 or bf16)           */
     float*      agg_out;                /* aggregated fp32 gradient, or NULL           */
@@ -124,6 +140,8 @@ typedef struct JabasSpan {
     uint32_t    n_fanout;
     uint32_t    bound_begin;            /* first entry of this span in the bounds table*/
     uint32_t    bound_count;            /* 0: the whole span is parameter group 0      */
+    uint32_t    state_block_log2;       /* 0: state1/2/3 are arrays of their own; else interleaved moments */
+    uint32_t    state_block_pos;        /* interleaved moments: position of the first element in its block */
     uint32_t    reserved;
 } JabasSpan;
 

@@ -50,6 +50,8 @@ class JabasSpan(C.Structure):
         ("n_fanout", C.c_uint32),
         ("bound_begin", C.c_uint32),
         ("bound_count", C.c_uint32),
+        ("state_block_log2", C.c_uint32),
+        ("state_block_pos", C.c_uint32),
         ("reserved", C.c_uint32),
     ]
 

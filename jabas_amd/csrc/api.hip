@@ -23,7 +23,7 @@ namespace {
 #endif
 constexpr uint64_t kGramGrid = JABAS_GRAM_GRID;     // persistent workgroups of the Gram kernel
 constexpr uint32_t kPlanMagic = 0x4a425359u;  // "JBSY"
-constexpr uint32_t kPlanVersion = 7;
+constexpr uint32_t kPlanVersion = 8;
 
 // A plan holds one chunk table per launch shape, indexed by the statistics level of the launch (0 none,
 // 1 full rows, 2 similarity sums). Levels whose shapes are the same share one table.
@@ -100,6 +100,25 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     if (oc == 0 && in.n_fanout) return JABAS_ERR_OPT;
     for (uint32_t r = 0; r < in.n_fanout; ++r)
         if (!in.fanout[r]) return JABAS_ERR_NULL;
+    // interleaved moments: the span's place in an arena of alternating blocks of T elements per moment
+    const uint32_t il_log2 = in.state_block_log2;
+    const uint64_t il_T = il_log2 ? static_cast<uint64_t>(1) << (il_log2 & 31) : 0;
+    const uint64_t il_ways = oc == 3 ? 3 : 2;
+    if (il_log2) {
+        if (oc < 2) return JABAS_ERR_OPT;
+        if (il_log2 < 8 || il_log2 > 24 || in.state_block_pos >= il_T) return JABAS_ERR_SIZE;
+        const uintptr_t s1a = reinterpret_cast<uintptr_t>(in.state1);
+        if (reinterpret_cast<uintptr_t>(in.state2) != s1a + il_T * 4) return JABAS_ERR_ALIGN;
+        if (oc == 3 && reinterpret_cast<uintptr_t>(in.state3) != s1a + il_T * 8) return JABAS_ERR_ALIGN;
+        if (s1a < static_cast<uintptr_t>(in.state_block_pos) * 4 || (s1a - static_cast<uintptr_t>(in.state_block_pos) * 4) % 16)
+            return JABAS_ERR_ALIGN;
+    }
+    // bytes from state1 to the end of the last element's last moment (one written range when interleaved)
+    uint64_t il_bytes = 0;
+    if (il_log2) {
+        const uint64_t tl = in.state_block_pos + in.numel - 1;
+        il_bytes = 4 * (tl + (il_ways - 1) * (tl & ~(il_T - 1)) + (il_ways - 1) * il_T + 1 - in.state_block_pos);
+    }
 
     const uintptr_t g0 = reinterpret_cast<uintptr_t>(in.grads[0]);
     if (g0 % gs) return JABAS_ERR_ALIGN;
@@ -114,8 +133,10 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     if (oc != 0) {
         same_wide(in.param, 4);
         same_wide(in.state1, 4);
-        same_wide(in.state2, 4);
-        if (oc == 3) same_wide(in.state3, 4);
+        if (!il_log2) {                        // interleaved: state2 and state3 sit whole blocks behind state1
+            same_wide(in.state2, 4);
+            if (oc == 3) same_wide(in.state3, 4);
+        }
         for (uint32_t r = 0; r < in.n_fanout; ++r) same_wide(in.fanout[r], 4);
     }
     // elements before the line the grid starts at
@@ -138,9 +159,22 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
         if (!rebase_g(in.grads[k], &out->g[k])) return JABAS_ERR_ALIGN;
     if (!rebase_f(in.agg_out, &out->out)) return JABAS_ERR_ALIGN;
     if (oc != 0) {
-        if (!rebase_f(in.param, &out->p) || !rebase_f(in.state1, &out->s1) || !rebase_f(in.state2, &out->s2))
-            return JABAS_ERR_ALIGN;
-        if (oc == 3 && !rebase_f(in.state3, &out->s3)) return JABAS_ERR_ALIGN;
+        if (!rebase_f(in.param, &out->p) || !rebase_f(in.state1, &out->s1)) return JABAS_ERR_ALIGN;
+        if (il_log2) {
+            // the moment bases are the start of the span's first block group; a grid element finds its moments
+            // through its position in the arena (SpanDev::mom_*). state1 passed the congruence check above and
+            // the block group starts on a 16-byte line, so a thread's four elements never straddle a block.
+            float* group = in.state1 - in.state_block_pos;
+            out->s1 = group;
+            out->s2 = group + il_T;
+            out->s3 = oc == 3 ? group + 2 * il_T : nullptr;
+            out->mom_add = static_cast<uint64_t>(in.state_block_pos) - skew;
+            out->mom_mask = ~(il_T - 1);
+            out->mom_mult = static_cast<uint32_t>(il_ways - 1);
+        } else {
+            if (!rebase_f(in.state2, &out->s2)) return JABAS_ERR_ALIGN;
+            if (oc == 3 && !rebase_f(in.state3, &out->s3)) return JABAS_ERR_ALIGN;
+        }
         for (uint32_t r = 0; r < in.n_fanout; ++r)
             if (!rebase_f(in.fanout[r], &out->fan[r])) return JABAS_ERR_ALIGN;
         out->n_fan = in.n_fanout;
@@ -156,25 +190,33 @@ int encode_span(const JabasSpan& in, int K, int grad_dtype, int opt_kind, int bl
     // in-place aggregate above is the one exception): each element is read and written by a
     // different thread at a different time, so any overlap would be a silent race.
     const void* written[5 + JABAS_MAX_K - 1];
-    int nw = 0;
-    if (in.agg_out) written[nw++] = in.agg_out;
-    if (oc != 0) {
-        written[nw++] = in.param;
-        if (in.state1) written[nw++] = in.state1;
-        if (oc >= 2) written[nw++] = in.state2;
-        if (oc == 3) written[nw++] = in.state3;
-        for (uint32_t r = 0; r < in.n_fanout; ++r) written[nw++] = in.fanout[r];
-    }
+    size_t wbytes[5 + JABAS_MAX_K - 1];
     const size_t fb = in.numel * 4;
+    int nw = 0;
+    auto add_written = [&](const void* p, size_t bytes) { written[nw] = p; wbytes[nw++] = bytes; };
+    if (in.agg_out) add_written(in.agg_out, fb);
+    if (oc != 0) {
+        add_written(in.param, fb);
+        if (il_log2) {
+            add_written(in.state1, il_bytes);
+        } else {
+            if (in.state1) add_written(in.state1, fb);
+            if (oc >= 2) add_written(in.state2, fb);
+            if (oc == 3) add_written(in.state3, fb);
+        }
+        for (uint32_t r = 0; r < in.n_fanout; ++r) add_written(in.fanout[r], fb);
+    }
     for (int i = 0; i < nw; ++i) {
         for (int j = i + 1; j < nw; ++j)
-            if (ranges_overlap(written[i], fb, written[j], fb)) return JABAS_ERR_ALIAS;
+            if (ranges_overlap(written[i], wbytes[i], written[j], wbytes[j])) return JABAS_ERR_ALIAS;
         if (written[i] == static_cast<const void*>(in.agg_out)) continue;      // checked against the gradients above
         for (int k = 0; k < K; ++k)
-            if (ranges_overlap(written[i], fb, in.grads[k], in.numel * gs)) return JABAS_ERR_ALIAS;
+            if (ranges_overlap(written[i], wbytes[i], in.grads[k], in.numel * gs)) return JABAS_ERR_ALIAS;
     }
     out->lo = skew;
     out->hi = skew + in.numel;
+    out->narrow_ok = out->hi <= kNarrowElems &&
+                     (!il_log2 || il_ways * (in.state_block_pos + in.numel + il_T) <= kNarrowElems);
     out->bound_begin = in.bound_begin;
     out->bound_count = in.bound_count;
     const uint64_t nt = tiles_of(out->hi, block);

@@ -96,10 +96,9 @@ constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2, OPT_AMS = 3;    // OPT_AM
 __host__ __device__ constexpr bool is_adam(int opt) { return opt == OPT_ADAM || opt == OPT_AMS; }
 // Kernels with statistics over more than four gradient streams form the addresses of the vector path as
 // scalar base + 32-bit lane offset (measured on the ViT-L/16 set, K = 8 bf16: +0.5 % with full rows, +2 % with
-// similarity sums); their spans of more than kNarrowElems elements (over 4 GiB of fp32 per buffer) go
+// similarity sums); their spans that 32-bit byte offsets do not reach (over 4 GiB of fp32 per buffer) go
 // through the careful path tile by tile: correct but slower. Everywhere else 64-bit vector addresses are
 // faster (the scalar bases compete with the launch constants for scalar registers: -0.5 ... -2.5 %).
-constexpr uint64_t kNarrowElems = 1ull << 30;
 __host__ __device__ constexpr bool narrow_addressing(int K, int SL) { return SL != 0 && K > 4; }
 
 // Statistics level of a launch: 0 none, 1 the full row (4 + K sums), 2 the four sums of the halves and of
@@ -159,6 +158,13 @@ struct DynView {
         grad_scale = a.grad_scale;
     }
 };
+
+// Float index of grid element e's Adam moments from the span's moment bases: e itself when the moments are
+// arrays of their own, its place in the interleaved arena otherwise (SpanDev). Two integer operations.
+__device__ __forceinline__ uint64_t moment_index(const SpanDev& sp, uint64_t e) {
+    const uint64_t t = e + sp.mom_add;
+    return t + sp.mom_mult * (t & sp.mom_mask);
+}
 
 // One element of the optimizer step. g is the aggregated gradient.
 template <int OPT>
@@ -271,9 +277,10 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U, OPT>& r, const Sp
         for (int k = 0; k < K; ++k) r.g[u][k] = GR::template load<NARROW>(sp.g[k], eu);
         if constexpr (OPT != OPT_NONE) {
             load_vec<NV, NARROW>(r.p[u], sp.p, eu);
-            if (load_s1) load_vec<NV, NARROW>(r.s1[u], sp.s1, eu);
-            if constexpr (is_adam(OPT)) load_vec<NV, NARROW>(r.s2[u], sp.s2, eu);
-            if constexpr (OPT == OPT_AMS) load_vec<NV, NARROW>(r.s3[u], sp.s3, eu);
+            const uint64_t mu = is_adam(OPT) ? moment_index(sp, eu) : eu;
+            if (load_s1) load_vec<NV, NARROW>(r.s1[u], sp.s1, mu);
+            if constexpr (is_adam(OPT)) load_vec<NV, NARROW>(r.s2[u], sp.s2, mu);
+            if constexpr (OPT == OPT_AMS) load_vec<NV, NARROW>(r.s3[u], sp.s3, mu);
         }
     }
 }
@@ -306,9 +313,10 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U, OPT>& r, const 
         if (sp.out) store_vec<NV, NARROW>(agg, sp.out, eu);
         if constexpr (OPT != OPT_NONE) {
             store_vec<NV, NARROW>(p, sp.p, eu);
-            if (use_s1) store_vec<NV, NARROW>(s1, sp.s1, eu);
-            if constexpr (is_adam(OPT)) store_vec<NV, NARROW>(s2, sp.s2, eu);
-            if constexpr (OPT == OPT_AMS) store_vec<NV, NARROW>(s3, sp.s3, eu);
+            const uint64_t mu = is_adam(OPT) ? moment_index(sp, eu) : eu;
+            if (use_s1) store_vec<NV, NARROW>(s1, sp.s1, mu);
+            if constexpr (is_adam(OPT)) store_vec<NV, NARROW>(s2, sp.s2, mu);
+            if constexpr (OPT == OPT_AMS) store_vec<NV, NARROW>(s3, sp.s3, mu);
             for (uint32_t f = 0; f < sp.n_fan; ++f) store_vec<NV, NARROW>(p, sp.fan[f], eu);
         }
     }
@@ -380,19 +388,20 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
         float g[K][1], p[1] = {0.0f}, s1[1] = {0.0f}, s2[1] = {0.0f}, s3[1] = {0.0f}, agg[1];
 #pragma unroll
         for (int k = 0; k < K; ++k) g[k][0] = GR::load1(sp.g[k], e);
+        [[maybe_unused]] const uint64_t me = is_adam(OPT) ? moment_index(sp, e) : e;
         if constexpr (OPT != OPT_NONE) {
             p[0] = sp.p[e];
-            if (load_s1) s1[0] = sp.s1[e];
-            if constexpr (is_adam(OPT)) s2[0] = sp.s2[e];
-            if constexpr (OPT == OPT_AMS) s3[0] = sp.s3[e];
+            if (load_s1) s1[0] = sp.s1[me];
+            if constexpr (is_adam(OPT)) s2[0] = sp.s2[me];
+            if constexpr (OPT == OPT_AMS) s3[0] = sp.s3[me];
         }
         compute<K, 1, DT, OPT, SL, false>(g, p, s1, s2, s3, agg, a, G, clip, acc);
         if (sp.out) sp.out[e] = agg[0];
         if constexpr (OPT != OPT_NONE) {
             sp.p[e] = p[0];
-            if (use_s1) sp.s1[e] = s1[0];
-            if constexpr (is_adam(OPT)) sp.s2[e] = s2[0];
-            if constexpr (OPT == OPT_AMS) sp.s3[e] = s3[0];
+            if (use_s1) sp.s1[me] = s1[0];
+            if constexpr (is_adam(OPT)) sp.s2[me] = s2[0];
+            if constexpr (OPT == OPT_AMS) sp.s3[me] = s3[0];
             for (uint32_t r = 0; r < sp.n_fan; ++r) sp.fan[r][e] = p[0];
         }
     }
@@ -427,7 +436,7 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
         }
         uint32_t nfull = 0;
         // spans beyond 32-bit byte offsets take the careful path tile by tile (64-bit addresses there)
-        if (e0 >= sp.lo && stretch_end >= e0 + TE && (!narrow_addressing(K, SL) || sp.hi <= kNarrowElems)) {
+        if (e0 >= sp.lo && stretch_end >= e0 + TE && (!narrow_addressing(K, SL) || sp.narrow_ok)) {
             const uint64_t fit = (stretch_end - e0) / TE;
             const uint32_t left = lt1 - lt;
             nfull = fit < left ? static_cast<uint32_t>(fit) : left;

@@ -108,11 +108,21 @@ struct SpanDev {
     float* s3;
     float* fan[JABAS_MAX_K - 1];
     uint64_t lo, hi;
+    // Where the Adam moments of grid element e live: float index mom(e) = t + mom_mult * (t & mom_mask),
+    // t = e + mom_add, from s1 / s2 / s3. Arrays of their own: all three zero, mom(e) = e. Interleaved in
+    // blocks of T elements: s1 = start of the span's first block group, s2 = s1 + T, s3 = s1 + 2 T,
+    // mom_add = position of the first live element in its block minus lo (wraps; t >= 0 for every live e),
+    // mom_mask = ~(T - 1), mom_mult = arrays interleaved - 1.
+    uint64_t mom_add, mom_mask;
+    uint32_t mom_mult;
+    uint32_t narrow_ok;                      // 32-bit byte offsets reach every access of the span
     uint32_t n_fan;
     uint32_t bound_begin;
     uint32_t bound_count;
     uint32_t pad;
 };
+// Largest element index a 32-bit byte offset reaches in an fp32 buffer.
+constexpr uint64_t kNarrowElems = 1ull << 30;
 
 struct BoundDev {                            // same layout as JabasBound
     uint64_t start;                          // in un-rebased span coordinates

@@ -12,13 +12,19 @@ import torch
 
 from . import _lib as L
 from .layout import FlatLayout
-from .sync import SpanSpec, SyncPlan, StepScalars, gradient_stats, make_step_args, opt_kind, cosine_from_stats, clip_coef, gram_from_stats
+from .sync import SpanSpec, SyncPlan, StepScalars, MomentArena, MOMENT_BLOCK_LOG2, gradient_stats, make_step_args, opt_kind, cosine_from_stats, clip_coef, gram_from_stats
 
 
 class VSWFlatSync:
     def __init__(self, specs, batches, grad_dtype=torch.float32, opt=None, device="cuda", in_place=None,
-                 n_fanout=0, per_tensor_spans=False, caps=None, keep_clipped_grads=True, write_aggregate=True):
+                 n_fanout=0, per_tensor_spans=False, caps=None, keep_clipped_grads=True, write_aggregate=True,
+                 moment_block_log2=MOMENT_BLOCK_LOG2):
         self.K = len(batches)
+        # Adam's moments (exp_avg, exp_avg_sq, amsgrad's maximum) live in ONE arena that alternates blocks of
+        # 2**moment_block_log2 elements of each (sync.MomentArena): the kernels stream that 2-6 % faster than
+        # arenas of their own. ``state1`` / ``state2`` / ``state3`` then are flat COPIES made on access
+        # (``set_state`` writes one back); 0 or None: flat arenas as for SGD's momentum buffer.
+        self.moment_block_log2 = int(moment_block_log2 or 0)
         # False: the launch hands the aggregate to the optimizer in registers and writes it nowhere (4 of the
         # 44 bytes per element of an Adam step with four fp32 workers). For owners of the whole step who clear
         # or overwrite the buckets right after it, as the trainer does; a comm hook has to leave the
@@ -47,23 +53,78 @@ class VSWFlatSync:
         else:                                    # an arena of its own, unless nothing will ever be written to it
             self.agg = torch.zeros(n, dtype=torch.float32, device=self.device) if self.write_aggregate else None
         kind = opt_kind(opt)
-        self.param = self.state1 = self.state2 = self.state3 = None
+        self.param = self._state = None
+        self.moments = None
         self.fanout = []
         if kind != L.OPT_NONE:
             if len(opt["groups"]) < self.layout.n_groups:
                 raise ValueError(f"layout names {self.layout.n_groups} parameter groups, optimizer has "
                                  f"{len(opt['groups'])}")
             self.param = torch.zeros(n, dtype=torch.float32, device=self.device)
-            if kind != L.OPT_SGD or opt.get("momentum", 0.0) != 0.0:
-                self.state1 = torch.zeros(n, dtype=torch.float32, device=self.device)
-            if kind in (L.OPT_ADAM, L.OPT_ADAMW, L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD):
-                self.state2 = torch.zeros(n, dtype=torch.float32, device=self.device)
-            if kind in (L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD):       # amsgrad: max_exp_avg_sq
-                self.state3 = torch.zeros(n, dtype=torch.float32, device=self.device)
+            adam = kind in (L.OPT_ADAM, L.OPT_ADAMW, L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD)
+            ways = 3 if kind in (L.OPT_ADAM_AMSGRAD, L.OPT_ADAMW_AMSGRAD) else 2        # amsgrad: max_exp_avg_sq
+            if adam and self.moment_block_log2:
+                self.moments = MomentArena(n, ways, self.device, self.moment_block_log2)
+            elif adam:
+                self._state = [torch.zeros(n, dtype=torch.float32, device=self.device) for _ in range(ways)]
+            elif opt.get("momentum", 0.0) != 0.0:
+                self._state = [torch.zeros(n, dtype=torch.float32, device=self.device)]
             self.fanout = [torch.zeros(n, dtype=torch.float32, device=self.device) for _ in range(n_fanout)]
         self._fanout_wanted = n_fanout > 0
         self._build_plan()
         self.step_count = 0
+
+    # ---- optimizer state ---------------------------------------------------------
+    def _state_arena(self, j):
+        if self.moments is not None:
+            return self.moments.read(j) if j < self.moments.ways else None
+        return self._state[j] if self._state is not None and j < len(self._state) else None
+
+    @property
+    def state1(self):
+        """SGD's momentum buffer / Adam's exp_avg as a flat fp32 tensor laid out like ``param``: the arena itself
+        when the state is kept in flat arenas, a copy made now when the moments are interleaved."""
+        return self._state_arena(0)
+
+    @property
+    def state2(self):
+        return self._state_arena(1)
+
+    @property
+    def state3(self):
+        return self._state_arena(2)
+
+    def set_state(self, j, values, start=0):
+        """Writes the flat tensor ``values`` into elements [start, ...) of state j (0, 1, 2 as state1..3)."""
+        if self.moments is not None:
+            self.moments.write(j, values, start)
+        else:
+            self._state[j][start:start + values.numel()].copy_(values.reshape(-1))
+
+    def state_view(self, j, i):
+        """State j of parameter i in the parameter's flat order: a live view of a flat arena, a copy when the
+        moments are interleaved (``state_is_live`` tells which)."""
+        off, n = self.layout.param_offset[i], self.layout.specs[i].numel
+        if self.moments is not None:
+            return self.moments.read(j, off, n)
+        return self._state[j][off:off + n]
+
+    @property
+    def state_is_live(self):
+        return self.moments is None
+
+    @property
+    def n_state(self):
+        """State arrays the optimizer keeps per element: 0 (none, SGD without momentum), 1, 2 or 3 (amsgrad)."""
+        return self.moments.ways if self.moments is not None else len(self._state or [])
+
+    def state_of_span(self, off, numel):
+        """SpanSpec keywords naming the optimizer state of arena elements [off, off + numel)."""
+        if self.moments is not None:
+            return dict(moments=(self.moments, off))
+        st = self._state or []
+        names = ("state1", "state2", "state3")
+        return {names[j]: st[j][off:off + numel] for j in range(len(st))}
 
     def _build_plan(self):
         kind = opt_kind(self.opt)
@@ -73,11 +134,8 @@ class VSWFlatSync:
             spans.append(SpanSpec(
                 [g[sl] for g in self.grads], agg_out=self.agg[sl] if self.write_aggregate else None,
                 param=None if self.param is None else self.param[sl],
-                state1=None if self.state1 is None else self.state1[sl],
-                state2=None if self.state2 is None else self.state2[sl],
-                state3=None if self.state3 is None else self.state3[sl],
                 fanout=[f[sl] for f in self.fanout],
-                bounds=bounds if kind != L.OPT_NONE else ()))
+                bounds=bounds if kind != L.OPT_NONE else (), **self.state_of_span(off, numel)))
         self.span_bucket = [s[3] for s in self.layout.spans]
         self.plan = SyncPlan(spans, kind)
         self._plan_agg = self._plan_opt = self._coef = None
@@ -197,10 +255,8 @@ class VSWFlatSync:
             agg_spans.append(SpanSpec([g[sl] for g in self.grads], agg_out=self.agg[sl]))
             opt_spans.append(SpanSpec([self.agg[sl]], agg_out=self.agg[sl] if self.keep_clipped_grads else None,
                                       param=self.param[sl],
-                                      state1=None if self.state1 is None else self.state1[sl],
-                                      state2=None if self.state2 is None else self.state2[sl],
-                                      state3=None if self.state3 is None else self.state3[sl],
-                                      fanout=[f[sl] for f in self.fanout], bounds=bounds))
+                                      fanout=[f[sl] for f in self.fanout], bounds=bounds,
+                                      **self.state_of_span(off, numel)))
         self._plan_agg = SyncPlan(agg_spans, L.OPT_NONE)
         self._plan_opt = SyncPlan(opt_spans, opt_kind(self.opt))
         self._coef = torch.ones(1, dtype=torch.float32, device=self.device)

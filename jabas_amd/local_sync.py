@@ -155,7 +155,9 @@ class LocalBucketSync:
         under a norm bound (``grad_clip``) keep the write: their second launch reads the aggregate.
 
         opt + param_buckets: hyperparameter dictionary and, per bucket index, dict(param=, state1=,
-        state2=, state3=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket; the launch of
+        state2=, state3=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket (or, in place of
+        the state tensors of an Adam kind, moments=(sync.MomentArena, index of the bucket's first element in it):
+        the moments interleaved in one arena, the layout the kernels stream fastest); the launch of
         such a bucket also runs the optimizer. ``optimizer=`` (or ``bind_optimizer``) takes a
         torch.optim.SGD / Adam / AdamW or Shard* object instead and builds those arenas itself from the
         ``parameters()`` / ``gradients()`` of the bucket objects the hooks publish."""
@@ -681,7 +683,7 @@ class LocalBucketSync:
                 call = sync.BucketCall(agg_span)
                 call.update = sync.BucketCall(sync.SpanSpec(
                     [span.agg_out], agg_out=span.agg_out, param=span.param, state1=span.state1, state2=span.state2,
-                    state3=span.state3, fanout=span.fanout, bounds=span.bounds))
+                    state3=span.state3, fanout=span.fanout, bounds=span.bounds, moments=span.moments))
                 with torch.cuda.stream(main):
                     call.coef = torch.ones(1, dtype=torch.float32, device=tensors[0].device)
             else:
@@ -718,6 +720,7 @@ class LocalBucketSync:
         span = sync.SpanSpec(tensors, agg_out=agg_out,
                              param=pb and pb.get("param"), state1=pb and pb.get("state1"),
                              state2=pb and pb.get("state2"), state3=pb and pb.get("state3"),
+                             moments=pb and pb.get("moments"),
                              fanout=(pb or {}).get("fanout", ()),
                              bounds=(pb or {}).get("bounds", ()) if opt else ())
         return span, opt is not None

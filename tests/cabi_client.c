@@ -24,6 +24,8 @@ int main(void) {
     SHOW_OFF(JabasSpan, n_fanout);
     SHOW_OFF(JabasSpan, bound_begin);
     SHOW_OFF(JabasSpan, bound_count);
+    SHOW_OFF(JabasSpan, state_block_log2);
+    SHOW_OFF(JabasSpan, state_block_pos);
     SHOW_SIZE(JabasBound);
     SHOW_OFF(JabasBound, start);
     SHOW_OFF(JabasBound, group);

@@ -34,7 +34,7 @@ def test_struct_layouts_match_the_header():
     # sizes a C compiler gives the header's structs on x86-64 / amdgcn host ABI
     K = L.MAX_K
     assert K == 16 and L.STATS_STRIDE == 4 + K
-    assert C.sizeof(L.JabasSpan) == K * 8 + 5 * 8 + (K - 1) * 8 + 8 + 4 * 4
+    assert C.sizeof(L.JabasSpan) == K * 8 + 5 * 8 + (K - 1) * 8 + 8 + 6 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
     assert C.sizeof(L.JabasStepArgs) == 4 + 4 + 4 * K + 4 + K + 4 * K + 4 * 4 + 4 + 5 * 8 + 16 * 24 + 8 + 8
@@ -271,7 +271,7 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
             s, f = name.split(".")
             assert getattr(structs[s], f).offset == int(val), name
             checked += 1
-    assert checked == 38
+    assert checked == 40
     # every field of the ctypes mirror was reported by the C side (reserved words aside)
     for sname, st in structs.items():
         for f, _ in st._fields_:
@@ -290,6 +290,66 @@ def test_plain_c_client_sees_the_same_layout_and_drives_the_host_entry_points(tm
         want = [L.stat_pair(K, a, b) for a in range(K) for b in range(a + 1, K)]
         assert ("pairs%d" % K, ",".join(map(str, want))) in seen
         assert want == list(range(4 + K, 4 + K + K * (K - 1) // 2)) and want[-1] < L.STATS_STRIDE
+
+
+def test_plan_encode_checks_interleaved_moments():
+    """A span whose Adam moments sit interleaved in one arena (state_block_log2): the layout rules, and the
+    moments from the first element's exp_avg to the last element's last moment as ONE written range."""
+    T, n = 1 << 10, 5000
+    arena = 0x7f0000000000 + 40 * (1 << 32)
+
+    def span(pos=0, first_block=0, ways=2):
+        s = _span(n, opt=True)
+        s.state1 = arena + 4 * (first_block * ways * T + pos)
+        s.state2 = s.state1 + 4 * T
+        s.state3 = s.state1 + 8 * T if ways == 3 else None
+        s.state_block_log2, s.state_block_pos = 10, pos
+        return s
+    assert _encode([span()], opt=L.OPT_ADAM)[0] == L.OK
+    assert _encode([span()], opt=L.OPT_ADAMW)[0] == L.OK
+    assert _encode([span(ways=3)], opt=L.OPT_ADAM_AMSGRAD)[0] == L.OK
+    assert _encode([span()], opt=L.OPT_ADAM_AMSGRAD)[0] == L.ERR_NULL          # the maximum has no place in a two-way arena
+    assert _encode([span()], opt=L.OPT_SGD)[0] == L.ERR_OPT
+    s = span()
+    s.state_block_log2 = 7
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_SIZE
+    s = span()
+    s.state_block_log2 = 25
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_SIZE
+    s = span()
+    s.state_block_pos = T
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_SIZE
+    s = span()
+    s.state2 += 16
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIGN
+    s = span(ways=3)
+    s.state3 -= 4 * T
+    assert _encode([s], opt=L.OPT_ADAM_AMSGRAD)[0] == L.ERR_ALIGN
+    s = span()
+    s.state_block_pos = 2                                         # the block group would start 8 bytes off a 16-byte line
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIGN
+    # a span in the middle of a block, at the other buffers' element of a 16-byte line
+    s = _span(n, opt=True, skew=3)
+    s.state1 = arena + 4 * (2 * T + 64 * 3 + 3)
+    s.state2, s.state_block_log2, s.state_block_pos = s.state1 + 4 * T, 10, 64 * 3 + 3
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.OK
+    s.state_block_pos -= 1                                        # another element of the line than the weights'
+    s.state1 -= 4
+    s.state2 -= 4
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIGN
+    # 5000 elements from position 0: blocks 0..4 of exp_avg and of exp_avg_sq, the last ends 4 * (9 * T + 904) bytes in
+    end = arena + 4 * (9 * T + n - 4 * T)
+    s = span()
+    s.param = end                                                 # right behind the last second moment: fine
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.OK
+    s.param = end - 16
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIAS
+    s = span()
+    s.agg_out = arena + 4 * T + 256                               # inside the first block of second moments
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIAS
+    s = span()
+    s.grads[1] = arena + 4 * (3 * T)                              # a gradient buffer inside a block the span does not own
+    assert _encode([s], opt=L.OPT_ADAM)[0] == L.ERR_ALIAS         # ... but which lies inside the one written range
 
 
 def test_plan_encode_rejects_overlapping_written_buffers():

@@ -45,10 +45,14 @@ def _make(gpu, batches, opt, dtype=torch.float32, **kw):
 
 
 @pytest.mark.parametrize("per_tensor", [False, True])
-@pytest.mark.parametrize("opt,dtype", [(SGD, torch.float32), (ADAM, torch.float32), (ADAM, torch.bfloat16)])
-def test_engine_steps_match_oracle(gpu, opt, dtype, per_tensor):
+@pytest.mark.parametrize("opt,dtype,blocks", [(SGD, torch.float32, 13), (ADAM, torch.float32, 13), (ADAM, torch.bfloat16, 13),
+                                              (ADAM, torch.float32, 0), (ADAM, torch.bfloat16, 9)])
+def test_engine_steps_match_oracle(gpu, opt, dtype, per_tensor, blocks):
+    """blocks: log2 of the block size of the interleaved moment arena (the engine's default 13; 9: blocks smaller
+    than a tile; 0: flat state arenas)."""
     batches = (4, 2, 2)
-    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=2, per_tensor_spans=per_tensor)
+    eng, host, spans = _make(gpu, batches, opt, dtype, n_fanout=2, per_tensor_spans=per_tensor, moment_block_log2=blocks)
+    assert eng.state_is_live == (opt is SGD or blocks == 0)
     assert len(eng.layout.buckets) >= 3
     adam = opt["kind"] != "sgd"
     for step in (1, 2, 3):

@@ -26,6 +26,14 @@ def _mlp(seed):
                                torch.nn.ReLU(), torch.nn.Linear(33, 10))
 
 
+def _states(opt):
+    """id(parameter) -> its entry of ``opt.state_dict()["state"]``: what a checkpoint sees."""
+    sd = opt.state_dict()
+    params = [p for g in opt.param_groups for p in g["params"]]
+    index = [i for g in sd["param_groups"] for i in g["params"]]
+    return {id(p): sd["state"][i] for p, i in zip(params, index) if i in sd["state"]}
+
+
 def _groups(model):
     decay = [p for p in model.parameters() if p.dim() > 1]
     no_decay = [p for p in model.parameters() if p.dim() <= 1]
@@ -469,13 +477,16 @@ def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
     sd = mine.state_dict()
     assert len(sd["state"]) == len(list(trainer.main_model.parameters()))
     key = "momentum_buffer" if kind == "sgd" else "exp_avg"
+    seen = _states(mine)
     for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
-        assert _close(mine.state[p][key], ref_opt.state[rp][key], 1e-6, 1e-8)
+        assert _close(seen[id(p)][key], ref_opt.state[rp][key], 1e-6, 1e-8)
         if kind != "sgd":
             assert float(mine.state[p]["step"]) == 5.0
-            assert _close(mine.state[p]["exp_avg_sq"], ref_opt.state[rp]["exp_avg_sq"], 1e-6, 1e-12)
+            assert _close(seen[id(p)]["exp_avg_sq"], ref_opt.state[rp]["exp_avg_sq"], 1e-6, 1e-12)
+            # interleaved moments (the trainer's default): copies for state_dict() only, none kept in between
+            assert "exp_avg" not in mine.state[p] and not trainer.engine.state_is_live
         if kind.endswith("amsgrad"):
-            assert _close(mine.state[p]["max_exp_avg_sq"], ref_opt.state[rp]["max_exp_avg_sq"], 1e-6, 1e-12)
+            assert _close(seen[id(p)]["max_exp_avg_sq"], ref_opt.state[rp]["max_exp_avg_sq"], 1e-6, 1e-12)
 
 
 def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
@@ -533,17 +544,19 @@ def test_trainer_accumulates_micro_batches_between_steps(gpu):
             assert _close(p, rp, 1e-6, 1e-7), step
 
 
-@pytest.mark.parametrize("kind", ["sgd", "adamw", "adamw_amsgrad"])
-def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
+@pytest.mark.parametrize("kind,interleave", [("sgd", True), ("adamw", True), ("adamw_amsgrad", True), ("adamw", False),
+                                             ("adamw_amsgrad", False)])
+def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, interleave, tmp_path):
     """state_dict() after 3 steps, through a file, into a fresh trainer (other initial weights, another
     number of VSWs): the next 3 steps give the bits of the uninterrupted run. The optimizer entry is in
-    torch's own format: a stock torch optimizer loads it."""
+    torch's own format: a stock torch optimizer loads it. With Adam's moments interleaved in one arena (the
+    default) and with flat state arenas, whose views the optimizer object then holds at all times."""
     from jabas_amd.train import VSWSyncTrainer
     batches = (4, 4, 4)
     crit = torch.nn.MSELoss()
 
     def make(seed, n_vsw):
-        t = VSWSyncTrainer(gpu, (4,) * n_vsw, interval=2)
+        t = VSWSyncTrainer(gpu, (4,) * n_vsw, interval=2, interleave_moments=interleave)
         t.prepare_stream_parallel(_mlp(seed), crit)
         if kind == "sgd":
             o = torch.optim.SGD(_groups(t.main_model), lr=0.05, momentum=0.9, foreach=False)
@@ -581,13 +594,19 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
         for pm, pb in zip(m.parameters(), b.main_model.parameters()):
             assert torch.equal(pm, pb)
     keys = ("momentum_buffer",) if kind == "sgd" else ("exp_avg", "exp_avg_sq") + (("max_exp_avg_sq",) if kind.endswith("amsgrad") else ())
+    live = b.engine.state_is_live
+    assert live == (kind == "sgd" or not interleave)
     arenas = {"momentum_buffer": b.engine.state1, "exp_avg": b.engine.state1, "exp_avg_sq": b.engine.state2,
               "max_exp_avg_sq": b.engine.state3}
+    seen_a, seen_b = _states(opt_a), _states(opt_b)
     for pa, pb in zip(a.main_model.parameters(), b.main_model.parameters()):
         for key in keys:
-            assert torch.equal(opt_a.state[pa][key], opt_b.state[pb][key])
-            arena = arenas[key]                                                      # still views of the arenas
-            assert opt_b.state[pb][key].untyped_storage().data_ptr() == arena.untyped_storage().data_ptr()
+            assert torch.equal(seen_a[id(pa)][key], seen_b[id(pb)][key])
+            if live:                                                                 # still views of the arenas
+                assert torch.equal(opt_a.state[pa][key], opt_b.state[pb][key])
+                assert opt_b.state[pb][key].untyped_storage().data_ptr() == arenas[key].untyped_storage().data_ptr()
+            else:                                                                    # copies for state_dict() only
+                assert key not in opt_b.state[pb]
     assert opt_a.param_groups[0]["lr"] == opt_b.param_groups[0]["lr"]
 
     # a stock torch optimizer over a plain copy of the model takes the optimizer entry as it is
@@ -597,7 +616,7 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
              else torch.optim.AdamW(_groups(plain), lr=1e-3, amsgrad=kind.endswith("amsgrad")))
     stock.load_state_dict(b.state_dict()["optimizer"])
     for pp, pb in zip(plain.parameters(), b.main_model.parameters()):
-        assert torch.equal(stock.state[pp][keys[0]], opt_b.state[pb][keys[0]])
+        assert torch.equal(stock.state[pp][keys[0]], seen_b[id(pb)][keys[0]])
 
     # and the other way round: a checkpoint of a plain torch run (no trainer entries) resumes here
     c, opt_c = make(23, 3)
@@ -606,7 +625,7 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, tmp_path):
     for pc, pb in zip(c.main_model.parameters(), b.main_model.parameters()):
         assert torch.equal(pc, pb)
         for key in keys:
-            assert torch.equal(opt_c.state[pc][key], opt_b.state[pb][key])
+            assert torch.equal(_states(opt_c)[id(pc)][key], seen_b[id(pb)][key])
 
 
 def test_trainer_with_bf16_gradient_buckets(gpu):

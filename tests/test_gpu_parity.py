@@ -414,6 +414,102 @@ def test_sync_bucket_fused_amsgrad(gpu, K, dtype, kind, stats):
     assert float((s3_h > s2_h).float().mean()) > 0.1          # the maximum did part from the moment
 
 
+@pytest.mark.parametrize("K,dtype,kind,stats,amsgrad", [
+    (4, torch.float32, "adamw", "similarity", False), (8, torch.bfloat16, "adamw", "similarity", False),
+    (8, torch.bfloat16, "adamw", False, False), (2, torch.float32, "adam", "full", True),
+    (8, torch.bfloat16, "adam", "full", True), (3, torch.float32, "adamw", "gram", False),
+    (12, torch.float32, "adam", False, False), (1, torch.float32, "adamw", False, True)])
+@pytest.mark.parametrize("block_log2", [8, 11, 13])
+def test_interleaved_moments(gpu, K, dtype, kind, stats, amsgrad, block_log2):
+    """Adam's moments in one arena of alternating blocks (JabasSpan.state_block_log2): spans that start at
+    arbitrary elements of the arena, in the middle of a block, shorter than a block and across many blocks, with
+    parameter-group bounds and element skews; aggregate, weights and every moment bit-identical to the oracle's
+    flat arrays, nothing of the arena outside the span's own elements touched."""
+    from jabas_amd import sync
+    opt = dict(ADAMW if kind == "adamw" else ADAM, amsgrad=amsgrad)
+    ways, T = (3 if amsgrad else 2), 1 << block_log2
+    total = 5 * T + 70001
+    arena = sync.MomentArena(total, ways, gpu, block_log2)
+    marker = 7.25
+    arena.buf.fill_(marker)
+    cases = [(0, 4099, 0), (T - 64, 3 * T + 200, 0), (T + 320, 37, 0), (2 * T + 64 * 5 + 3, 70001, 3), (4 * T - 4 + 1, 2 * T, 1)]
+    for ci, (first, n, skew) in enumerate(cases):
+        skew = first % 64                          # every buffer of a span sits at the same element of a 256-byte line
+        print(f"interleaved K={K} {dtype} T={T} first={first} n={n}", flush=True)
+        bounds = ((0, 1), (5, 0), (min(1029, n - 1), 1)) if n > 1100 else ((0, 0),)
+        p_h = _host_state(n, 5 + ci)
+        m_h, v_h, x_h = torch.zeros(n), torch.zeros(n), torch.zeros(n)
+        for j in range(ways):
+            arena.write(j, torch.zeros(n, device=gpu), first)
+        agg_d = _dev(torch.zeros(n), gpu, skew)
+        p_d = _dev(p_h, gpu, skew)
+        dg = [_dev(torch.zeros(n, dtype=dtype), gpu, skew) for _ in range(K)]
+        span = sync.SpanSpec(dg, agg_out=agg_d, param=p_d, bounds=bounds, moments=(arena, first))
+        ws = sync.Workspace.for_span(n, dtype, gpu)
+        for step in (1, 2, 3):
+            hg = _host_grads(K, n, 700 + K + step + ci, std=5e-3 if step <= 2 else 2e-4, dtype=dtype)
+            for d, h in zip(dg, hg):
+                d.copy_(h)
+            row = sync.sync_bucket(span, sync.make_step_args(BATCHES[K], dtype, stats=stats, opt=opt, step=step), workspace=ws)
+            torch.cuda.synchronize()
+            agg_h, rows_h = O.sync_step(hg, BATCHES[K], [(0, n, bounds)], opt, p_h, m_h, v_h, step=step,
+                                        want_stats=bool(stats), state3=x_h if amsgrad else None)
+            assert torch.equal(_bits(agg_d), _bits(agg_h)), (first, step)
+            got = [arena.read(j, first, n) for j in range(ways)]
+            for name, a, b in (("p", p_d, p_h), ("m", got[0], m_h), ("v", got[1], v_h)) + ((("max", got[2], x_h),) if amsgrad else ()):
+                same, tot = _same_bits(a, b)
+                assert same == tot, (first, n, step, name, same, tot)
+            if stats:
+                rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
+                assert _close(row.cpu()[1:4], rows_h[0][1:4], rtol, 1e-30)[0]
+    # what the spans did not own still holds the marker
+    owned = torch.zeros(arena.blocks * T, dtype=torch.bool, device=gpu)
+    for first, n, _ in cases:
+        owned[first:first + n] = True
+    for j in range(ways):
+        rest = arena.way(j).reshape(-1)[~owned]
+        assert bool((rest == marker).all()), j
+
+
+def test_interleaved_moments_are_checked(gpu):
+    """Layout rules of interleaved moments: Adam kinds only, state2 / state3 whole blocks behind state1, the
+    block position inside the block, the block group on a 16-byte line; the moments count as one written range."""
+    import ctypes as C
+    from jabas_amd import sync, _lib as L
+    lib = L.lib()
+    n, b = 5000, 10
+    T = 1 << b
+    arena = sync.MomentArena(8 * T, 2, gpu, b)
+    g = [torch.zeros(n, device=gpu)]
+    p = torch.zeros(n, device=gpu)
+    adam = sync.make_step_args((1,), torch.float32, opt=ADAM, step=1)
+    sgd = sync.make_step_args((1,), torch.float32, opt=SGD, first_step=True)
+
+    def call(span, args=adam):
+        return lib.jabas_sync_bucket(C.byref(span), None, C.byref(args), None, None, 0, None)
+    good = sync.SpanSpec(g, param=p, moments=(arena, 0)).to_c()
+    assert call(good) == L.OK
+    assert call(good, sgd) == L.ERR_OPT
+    bad = sync.SpanSpec(g, param=p, moments=(arena, 0)).to_c()
+    bad.state2 = bad.state1 + 4 * T + 16
+    assert call(bad) == L.ERR_ALIGN
+    bad = sync.SpanSpec(g, param=p, moments=(arena, 0)).to_c()
+    bad.state_block_pos = T
+    assert call(bad) == L.ERR_SIZE
+    bad = sync.SpanSpec(g, param=p, moments=(arena, 0)).to_c()
+    bad.state_block_log2 = 7
+    assert call(bad) == L.ERR_SIZE
+    bad = sync.SpanSpec(g, param=p, moments=(arena, 0)).to_c()
+    bad.state_block_pos = 2                                   # the block group would start 8 bytes off a 16-byte line
+    assert call(bad) == L.ERR_ALIGN
+    # the weights inside the moments' range (the gap between two of the span's blocks is part of that range)
+    inside = arena.buf[2 * T:2 * T + n]
+    assert call(sync.SpanSpec(g, param=inside, moments=(arena, 0)).to_c()) == L.ERR_ALIAS
+    ams = sync.make_step_args((1,), torch.float32, opt=dict(ADAM, amsgrad=True), step=1)
+    assert call(good, ams) == L.ERR_NULL                      # two moments interleaved where the optimizer keeps three
+    torch.cuda.synchronize()
+
+
 def test_amsgrad_needs_its_maximum_and_is_not_replayed_from_a_block(gpu):
     from jabas_amd import sync, _lib as L
     n = 4096
