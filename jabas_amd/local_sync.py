@@ -104,7 +104,7 @@ class LocalBucketSync:
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
                  optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True,
-                 launch_streams=2, auto_finish=True):
+                 launch_streams=2, auto_finish=True, interleave_moments=False):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
@@ -154,6 +154,13 @@ class LocalBucketSync:
         default leaves the synchronised gradient in the main VSW's bucket, as the reference's hooks do. Buckets
         under a norm bound (``grad_clip``) keep the write: their second launch reads the aggregate.
 
+        interleave_moments (with ``optimizer=``, Adam kinds): the moments of a bucket's parameters are kept in
+        one arena of alternating blocks (``sync.MomentArena``: the layout the kernels stream 2-6 % faster) instead
+        of flat arenas. A moment then is no flat tensor: the optimizer object gets copies under torch's names
+        when its ``state_dict()`` runs (hooks on the optimizer) and holds only the step count in between; state
+        the optimizer carries in when a bucket is bound (a checkpoint loaded before the first step) is taken
+        over. Default: flat arenas whose views ``optimizer.state[p]`` holds at all times.
+
         opt + param_buckets: hyperparameter dictionary and, per bucket index, dict(param=, state1=,
         state2=, state3=, bounds=, fanout=, agg_out=) of flat fp32 tensors laid out like the bucket (or, in place of
         the state tensors of an Adam kind, moments=(sync.MomentArena, index of the bucket's first element in it):
@@ -199,6 +206,8 @@ class LocalBucketSync:
         self._sync_streams = []                # the launch streams; empty: VSW 0's own stream carries the launches
         self._sync_stream = stream
         self.auto_finish = bool(auto_finish)
+        self.interleave_moments = bool(interleave_moments)
+        self._moment_home = {}                 # id(parameter) -> (MomentArena, first element, parameter): interleaved moments
         self._step_open = False                # something was handed over since the last end of step
         self._finishing = False                # an implied end of step is running
         self._last_done = []                   # one event per launch stream behind the launches of the step finished last
@@ -317,6 +326,45 @@ class LocalBucketSync:
         self.grad_clip = float(getattr(optimizer, "grad_clip", float("inf")))
         return self
 
+    _MOMENT_NAMES = ("exp_avg", "exp_avg_sq", "max_exp_avg_sq")
+
+    def _hook_moments_into_state_dict(self):
+        """Interleaved moments: the optimizer object shows them when it is asked for its state. Before its
+        ``state_dict()`` packs ``optimizer.state`` every parameter gets copies of its moments under torch's names;
+        afterwards the result keeps them (in shallow copies of the per-parameter dictionaries: torch packs the
+        dictionaries themselves) and the optimizer's own dictionaries lose them again."""
+        opt = self.optimizer
+        if getattr(opt, "_jabas_moment_hooks", None) is not None:
+            opt._jabas_moment_hooks = weakref.ref(self)
+            return
+        opt._jabas_moment_hooks = weakref.ref(self)
+
+        def before(o):
+            me = o._jabas_moment_hooks()
+            if me is None or me.optimizer is not o:
+                return
+            homes = list(me._moment_home.values())
+            if homes:
+                torch.cuda.synchronize(homes[0][0].device)
+            for arena, start, prm in homes:
+                st = o.state[prm]
+                for j, name in enumerate(me._MOMENT_NAMES[:arena.ways]):
+                    st[name] = arena.read(j, start, prm.numel()).view(prm.shape)
+
+        def after(o, state_dict):
+            me = o._jabas_moment_hooks()
+            if me is None or me.optimizer is not o:
+                return state_dict
+            state_dict["state"] = {idx: dict(st) for idx, st in state_dict["state"].items()}
+            for _arena, _start, prm in list(me._moment_home.values()):
+                st = o.state[prm]
+                for name in me._MOMENT_NAMES:
+                    st.pop(name, None)
+            return state_dict
+
+        opt.register_state_dict_pre_hook(before)
+        opt.register_state_dict_post_hook(after)
+
     def _refresh_hyperparameters(self):
         if self.optimizer is None:
             return
@@ -354,14 +402,21 @@ class LocalBucketSync:
                 raise ValueError(f"bucket {bucket_index} carries a parameter no group of the optimizer holds")
         order = sorted(range(len(params)), key=lambda i: offs[i])
         sgd = self.opt["kind"] == "sgd"
+        interleaved = self.interleave_moments and not sgd
         with torch.no_grad(), torch.cuda.stream(self._launch_stream(bucket_index)):
             new = dict(_key=key, param=_arena_like(buf0), fanout=[])
-            if not sgd or self.opt.get("momentum", 0.0) != 0.0:
-                new["state1"] = _arena_like(buf0)
-            if not sgd:
-                new["state2"] = _arena_like(buf0)
-            if self.opt.get("amsgrad", False):
-                new["state3"] = _arena_like(buf0)
+            if interleaved:
+                # the bucket's first element at the element of a 256-byte line its other buffers start at
+                first = (buf0.data_ptr() // es) % 64
+                arena = sync.MomentArena(first + n, 3 if self.opt.get("amsgrad", False) else 2, buf0.device)
+                new["moments"] = (arena, first)
+            else:
+                if not sgd or self.opt.get("momentum", 0.0) != 0.0:
+                    new["state1"] = _arena_like(buf0)
+                if not sgd:
+                    new["state2"] = _arena_like(buf0)
+                if self.opt.get("amsgrad", False):
+                    new["state3"] = _arena_like(buf0)
             if buf0.dtype != torch.float32 and (self.write_aggregate or self.grad_clip != float("inf")):
                 new["agg_out"] = _arena_like(buf0)
             names = ("momentum_buffer",) if sgd else ("exp_avg", "exp_avg_sq", "max_exp_avg_sq")
@@ -371,6 +426,16 @@ class LocalBucketSync:
                 view.copy_(p.data)
                 p.data = view
                 st = self.optimizer.state[p]
+                if interleaved:
+                    arena, first = new["moments"]
+                    home = self._moment_home.get(id(p))
+                    for j, name in enumerate(names[:arena.ways]):
+                        if torch.is_tensor(st.get(name)):               # carried in by the optimizer object
+                            arena.write(j, st[name].to(buf0.device), first + o)
+                        elif home is not None:                          # kept by the bucket the parameter was in before
+                            arena.write(j, home[0].read(j, home[1], p.numel()), first + o)
+                        st.pop(name, None)
+                    self._moment_home[id(p)] = (arena, first + o, p)
                 for name, arena in zip(names, ("state1", "state2", "state3")):
                     if arena not in new:
                         continue
@@ -420,6 +485,8 @@ class LocalBucketSync:
         new["bounds"] = tuple(bounds)
         new["params"] = params
         self.param_buckets[bucket_index] = new
+        if interleaved:
+            self._hook_moments_into_state_dict()
         with self._lock:
             self._calls.pop(bucket_index, None)
             self._plans.clear()

@@ -93,6 +93,16 @@ def test_optimizer_in_the_hook_with_amsgrad(gpu, gdt, mode):
     _hooks_with_optimizer(gpu, "adamw_amsgrad", gdt, mode, (4, 2, 2))
 
 
+@pytest.mark.parametrize("kind", ["adamw", "adamw_amsgrad"])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["per_bucket", "deferred", "batched"])
+def test_optimizer_in_the_hook_with_interleaved_moments(gpu, kind, gdt, mode):
+    """``LocalBucketSync(interleave_moments=True)``: the moments of a bucket's parameters in one arena of alternating
+    blocks; weights bit-exact as with flat arenas, the moments bit-exact in what ``optimizer.state_dict()`` shows,
+    ``optimizer.state[p]`` without them in between."""
+    _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2), launch_streams=2, interleave=True)
+
+
 @pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
 def test_overlap_mode_that_writes_no_aggregate(gpu, gdt):
     """``write_aggregate=False``: weights, state and replicas as before, VSW 0's bucket left as backward filled
@@ -126,7 +136,15 @@ def test_eight_vsw_threads_with_bf16_buckets(gpu, mode):
     _hooks_with_optimizer(gpu, "adamw", torch.bfloat16, mode, (64, 56, 48, 40, 32, 24, 16, 8))
 
 
-def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPES=SHAPES):
+def _checkpointed(optimizer):
+    """id(parameter) -> its entry of ``optimizer.state_dict()["state"]``: the state as a checkpoint sees it."""
+    sd = optimizer.state_dict()
+    params = [p for g in optimizer.param_groups for p in g["params"]]
+    index = [i for g in sd["param_groups"] for i in g["params"]]
+    return {id(p): sd["state"][i] for p, i in zip(params, index) if i in sd["state"]}
+
+
+def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPES=SHAPES, interleave=False):
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
@@ -145,7 +163,8 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
     keep = not mode.endswith("no_aggregate")
     mode = mode.replace("_no_aggregate", "")
     local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=400_000 if mode == "batched" else 0,
-                            stream=create_stream_for_optimizer(gpu), write_aggregate=keep, launch_streams=launch_streams)
+                            stream=create_stream_for_optimizer(gpu), write_aggregate=keep, launch_streams=launch_streams,
+                            interleave_moments=interleave)
     assert len(local._sync_streams) == launch_streams
     st = H.GradientSimilarityState(None, K + K % 2, None, [], 2).attach_local(local)
     main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
@@ -192,6 +211,8 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
         local.finish_step()
         torch.cuda.synchronize()
         want_stats = st.step % st.interval == 0
+        # interleaved moments: the optimizer object holds them only while its state_dict() is made
+        seen = _checkpointed(optimizer) if interleave else None
         for b, (offs, bounds, n) in enumerate(layouts):
             agg_h, rows_h = O.sync_step(host[b], batches, [(0, n, bounds)], opt, p_h[b], s1_h[b], s2_h[b], step=step,
                                         first_step=(step == 1), want_stats=want_stats, lr_scale=local.lr_scale,
@@ -205,6 +226,9 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
                 sl = slice(o, o + p.numel())
                 assert _same(p.data, p_h[b][sl]), (step, b, i, "weights")
                 state = optimizer.state[p]
+                if interleave and kind != "sgd":
+                    assert "exp_avg" not in state and int(state["step"]) == step
+                    state = seen[id(p)]
                 if kind == "sgd":
                     assert _same(state["momentum_buffer"], s1_h[b][sl]), (step, b, i, "momentum")
                 else:
@@ -475,11 +499,13 @@ def test_batches_that_would_merge_nothing_fall_back_to_one_launch_per_bucket(gpu
     assert alone.launched > 3 * len(sizes) - 3 and alone.native_launches == 2 * len(sizes)
 
 
-def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
+@pytest.mark.parametrize("interleave", [False, True])
+def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu, interleave):
     """DDP's bucket rebuild can put the same parameters in another order (or other parameters) at the old buffer
     addresses. With an optimizer bound, the native meeting point must not launch the span it was described for
     the old order: VSW 0's bucket is checked against the parameters of the description, the arenas are laid out
-    again, and a peer that had already handed its (unchanged) buffer over natively is handed over again."""
+    again, and a peer that had already handed its (unchanged) buffer over natively is handed over again.
+    interleave: the moments live in the bucket's interleaved arena and move with their parameter into the new one."""
     from jabas_amd import ddp_comm_hooks as H
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import create_optimizer_hook, create_stream_for_optimizer
@@ -491,7 +517,7 @@ def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
     init = {n: torch.randn(s, generator=gen) * 0.05 for n, s in shapes.items()}
     replicas = [{n: torch.nn.Parameter(t.clone().to(gpu)) for n, t in init.items()} for _ in range(K)]
     optimizer = _torch_optimizer("adamw", list(replicas[0].values()))
-    local = LocalBucketSync(batches, stream=create_stream_for_optimizer(gpu))
+    local = LocalBucketSync(batches, stream=create_stream_for_optimizer(gpu), interleave_moments=interleave)
     st = H.GradientSimilarityState(None, 2, None, [], 10 ** 9).attach_local(local)
     main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
     bufs = [torch.zeros(8192, device=gpu) for _ in range(K)]
@@ -516,6 +542,7 @@ def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
                     H.dummy_hook(H.VSWPeerState(local, k), bucket).wait()
         local.finish_step()
         torch.cuda.synchronize()
+        seen = _checkpointed(optimizer) if interleave else {id(p): optimizer.state[p] for p in replicas[0].values()}
         for j, n in enumerate(order):
             sl = slice(4096 * j, 4096 * (j + 1))
             agg = O.aggregate([host[k][sl] for k in range(K)], batches)
@@ -523,8 +550,9 @@ def test_rebuilt_bucket_at_the_old_addresses_is_rebound(gpu):
             assert _same(bufs[0][sl], agg), (step, n, "aggregate")
             assert _same(replicas[0][n].data, p_h[n]), (step, n, "weights")
             assert _same(replicas[1][n].data, p_h[n]), (step, n, "replica")
-            assert _same(optimizer.state[replicas[0][n]]["exp_avg"], s1_h[n]), (step, n)
-            assert _same(optimizer.state[replicas[0][n]]["exp_avg_sq"], s2_h[n]), (step, n)
+            assert _same(seen[id(replicas[0][n])]["exp_avg"], s1_h[n]), (step, n)
+            assert _same(seen[id(replicas[0][n])]["exp_avg_sq"], s2_h[n]), (step, n)
+            assert ("exp_avg" in optimizer.state[replicas[0][n]]) == (not interleave)
         # natively launched: a step whose bucket came as the step before left it
         want_native = step >= 2 and plan[step - 2][0] == order
         assert local.native_launches - native_before == (1 if want_native else 0), step

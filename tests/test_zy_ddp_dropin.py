@@ -146,8 +146,10 @@ def test_stock_ddp_buckets_through_the_hooks(gpu, batches):
     dist.destroy_process_group()
 
 
-@pytest.mark.parametrize("mode", ["per_bucket", "batched", "deferred", "per_bucket_shared_weights"])
-@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+@pytest.mark.parametrize("kind,mode", [("sgd", "per_bucket"), ("sgd", "batched"), ("sgd", "deferred"), ("sgd", "per_bucket_shared_weights"),
+                                       ("adamw", "per_bucket"), ("adamw", "batched"), ("adamw", "deferred"),
+                                       ("adamw", "per_bucket_shared_weights"), ("adamw", "per_bucket_interleaved_moments"),
+                                       ("adamw", "deferred_interleaved_moments")])
 def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     """Overlap weight-sync mode end to end with stock DDP (jabas/train/trainer.py:327-333): the optimizer
     hook on VSW 0, a launch stream of its own, the weights of both replicas and the optimizer state
@@ -178,8 +180,10 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
     s1_h, s2_h = [torch.zeros_like(p) for p in p_h], [torch.zeros_like(p) for p in p_h]
 
     share = mode.endswith("shared_weights")              # the replica's parameters become views of the main weight arena
+    interleave = mode.endswith("interleaved_moments")    # Adam's moments of a bucket in one arena of alternating blocks
+    mode = mode.replace("_interleaved_moments", "")
     local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=250_000 if mode == "batched" else 0,
-                            share_weights=share)
+                            share_weights=share, interleave_moments=interleave)
     state = H.GradientSimilarityState(dist.group.WORLD, 2, None, [], 2).attach_local(local)
     rec = Recorder(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), main)
     prepare_overlap_optimizer_with_ddp(replicas, [state, H.VSWPeerState(local, 1)], [rec.hook, H.dummy_hook], optimizer, local)
@@ -196,6 +200,10 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
         torch.cuda.synchronize()
         per_vsw = _per_parameter_grads(rec, replicas)
         step_opt = dict(opt, groups=[dict(g, lr=g["lr"] * (0.9 ** (step - 1))) for g in opt["groups"]])
+        if interleave:                                    # the moments as a checkpoint of this moment holds them
+            sd_now = optimizer.state_dict()
+            index = dict(zip((id(q_) for g in optimizer.param_groups for q_ in g["params"]),
+                             (j for g in sd_now["param_groups"] for j in g["params"])))
         for i, (p, q) in enumerate(zip(main.parameters(), replicas[1].module.parameters())):
             agg = O.aggregate([per_vsw[0][i], per_vsw[1][i]], batches)
             O.opt_step(step_opt, group_of[i], p_h[i], agg, s1_h[i], s2_h[i], step, step == 1)
@@ -204,6 +212,9 @@ def test_stock_ddp_with_the_optimizer_in_the_hook(gpu, kind, mode):
             assert torch.equal(_bits(q.data), _bits(p_h[i])), (step, i, "replica weights")
             assert (q.data_ptr() == p.data_ptr()) == share and q is not p
             st = optimizer.state[p]
+            if interleave:
+                assert "exp_avg" not in st and int(st["step"]) == step
+                st = sd_now["state"][index[id(p)]]
             if kind == "sgd":
                 assert torch.equal(_bits(st["momentum_buffer"]), _bits(s1_h[i])), (step, i)
             else:
