@@ -2,7 +2,7 @@
 """Benchmark of the fused per-GPU gradient-sync step on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-all] [--no-cpu] [--no-extras]
-                    [--cpu-seconds S] [--calibrate-copy]
+                    [--cpu-seconds S] [--calibrate-copy] [--flat-moments]
 
 A step is one fused sync step (batch-weighted aggregate of the K VSW gradient buckets
 + the similarity statistics where the configuration asks for them + optimizer update) over
@@ -23,6 +23,7 @@ hook call per bucket and VSW: one launch per bucket, per 64 MiB of buckets, per 
 (without statistics, with full statistics rows).
 """
 import argparse
+import gc
 import json
 import math
 import os
@@ -76,8 +77,12 @@ def fill_engine(eng, cfg, device, torch, seed, independent_masks=False):
             v.copy_(torch.where(keep[:, None], v, torch.zeros((), device=device, dtype=v.dtype)))
 
 
+FLAT_MOMENTS = False     # --flat-moments: Adam's moments in arrays of their own instead of the interleaved arena
+
+
 def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0, write_aggregate=True):
     from jabas_amd.engine import VSWFlatSync
+    from jabas_amd.sync import MOMENT_BLOCK_LOG2
     gdt = torch.bfloat16 if cfg.grad_dtype == "bf16" else torch.float32
     numel = sum(s.numel for s in cfg.specs)
     ws = numel * algorithmic_bytes_per_elem(cfg)
@@ -85,7 +90,7 @@ def build_engines(cfg, device, torch, independent_masks=False, n_fanout=0, write
     engines = []
     for c in range(copies):
         eng = VSWFlatSync(cfg.specs, cfg.batches, grad_dtype=gdt, opt=cfg.opt, device=device, n_fanout=n_fanout,
-                          write_aggregate=write_aggregate)
+                          write_aggregate=write_aggregate, moment_block_log2=0 if FLAT_MOMENTS else MOMENT_BLOCK_LOG2)
         fill_engine(eng, cfg, device, torch, 1234 + 17 * c, independent_masks)
         engines.append(eng)
     return engines, numel, copies
@@ -99,18 +104,29 @@ def timed_region(fn, steps, warmup, torch):
     calls themselves took (queueing only: measured before the closing synchronisation) is left in
     ``host_us_of_last_region()``."""
     global _last_host_us
-    for i in range(warmup):
-        fn(i)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for i in range(steps):
-        fn(i)
-    e1.record()
-    _last_host_us = (time.perf_counter() - t0) * 1e6 / steps
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3
+    # The interpreter's cyclic garbage collector stays out of the timed region (as timeit keeps it out): a full
+    # collection over everything torch has imported takes tens of milliseconds, and one that falls between the
+    # opening event and the first launch leaves the GPU idle for that long (seen: 40 ms in a 120 ms region).
+    # Collected before the warm-up, so that the GPU is busy again when the timed region starts.
+    gc_was_on = gc.isenabled()
+    gc.collect()
+    gc.disable()
+    try:
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        _last_host_us = (time.perf_counter() - t0) * 1e6 / steps
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+    finally:
+        if gc_was_on:
+            gc.enable()
     return max(e0.elapsed_time(e1), 1e-6) / steps, wall_ms / steps
 
 
@@ -650,11 +666,16 @@ def main():
     ap.add_argument("--bucket-launches", type=int, default=0, metavar="S",
                     help="run only this: the headline workload's gradient set as one launch per bucket, bucket i on "
                          "launch stream i mod S, --steps steps after --warmup (for a kernel trace of the launches)")
+    ap.add_argument("--flat-moments", action="store_true",
+                    help="keep Adam's moments in flat arenas of their own (the layout before the interleaved moment "
+                         "arena, sync.MomentArena) in every engine this run builds: for A/B runs of the two layouts")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB copy 5 times before anything else (the K=1, weight-1 aggregate: "
                          "same 16-byte nontemporal loads and stores as the fused kernel, known traffic) for "
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
+    global FLAT_MOMENTS
+    FLAT_MOMENTS = bool(args.flat_moments)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this build measures the one-GPU share of the gradient-sync path; "
                  "run it with --gpus 1 (no collectives are part of the path)")
@@ -735,15 +756,16 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": head_cfg.name, "elements": head["elements"], "K": head["K"],
                    "batches": head["batches"], "grad_dtype": head["grad_dtype"], "optimizer": head["optimizer"],
-                   "stats": head["stats"], "bytes_per_elem": head["bytes_per_elem"]},
+                   "stats": head["stats"], "bytes_per_elem": head["bytes_per_elem"],
+                   "adam_moments": "flat arenas" if FLAT_MOMENTS else "one arena, interleaved in blocks of 8192 elements"},
         "pct_hbm_peak": head["pct_hbm_peak"],
         "roofline": roofline,
         "cpu_baseline": head.get("cpu_baseline"),
         "copy_GBps": copy_gbps,
         "workloads": list(results.values()),
         "reference_profile_metrics_resnet50": ref_metrics,
-        # the configuration the first round's headline was quoted on (ViT-B/16, K = 4, fp32 gradients, full statistics
-        # rows), so that figures stay comparable from round to round whatever the headline workload is
+        # the configuration an earlier headline was quoted on (ViT-B/16, K = 4, fp32 gradients, full statistics
+        # rows), so that figures stay comparable over time whatever the headline workload is
         "like_for_like": {"vit_b16_K4_f32_full_statistics_rows":
                           results.get("vit_b16", {}).get("step_with_per_vsw_norms")},
         "statistics_launches": stat_launches,
