@@ -161,7 +161,12 @@ struct DynView {
 
 // Float index of grid element e's Adam moments from the span's moment bases: e itself when the moments are
 // arrays of their own, its place in the interleaved arena otherwise (SpanDev). Two integer operations.
-__device__ __forceinline__ uint64_t moment_index(const SpanDev& sp, uint64_t e) {
+// The bound table of a launch is, like the plan's other tables, not written while the launch runs: read through
+// the constant address space (uniform loads the compiler is free to move or repeat).
+typedef const __attribute__((address_space(4))) BoundDev* ConstBounds;
+__device__ __forceinline__ ConstBounds const_bounds(const BoundDev* p) { return (ConstBounds)p; }
+
+template <class SP> __device__ __forceinline__ uint64_t moment_index(const SP& sp, uint64_t e) {
     const uint64_t t = e + sp.mom_add;
     return t + sp.mom_mult * (t & sp.mom_mask);
 }
@@ -265,8 +270,8 @@ template <int K, int DT, int U, int OPT = OPT_ADAM> struct TileRegs {
 
 // Issues every load of U consecutive full tiles. e is the (rebased) index of this
 // thread's first element in the first tile.
-template <int K, int DT, int OPT, int U, int BS, bool NARROW>
-__device__ __forceinline__ void issue_loads(TileRegs<K, DT, U, OPT>& r, const SpanDev& sp, uint64_t e, bool load_s1) {
+template <int K, int DT, int OPT, int U, int BS, bool NARROW, class SP>
+__device__ __forceinline__ void issue_loads(TileRegs<K, DT, U, OPT>& r, const SP& sp, uint64_t e, bool load_s1) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT, NV = EPT / 4;
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * EPT;
@@ -286,8 +291,8 @@ __device__ __forceinline__ void issue_loads(TileRegs<K, DT, U, OPT>& r, const Sp
 }
 
 // Arithmetic and stores of U tiles whose loads were issued by issue_loads.
-template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW, class A>
-__device__ __forceinline__ void consume(const TileRegs<K, DT, U, OPT>& r, const SpanDev& sp, uint64_t e, const A& a,
+template <int K, int DT, int OPT, int SL, bool HD, int U, bool NARROW, class A, class SP>
+__device__ __forceinline__ void consume(const TileRegs<K, DT, U, OPT>& r, const SP& sp, uint64_t e, const A& a,
                                         const GroupDev& G, float clip, bool use_s1, bool load_s1,
                                         typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
@@ -324,8 +329,8 @@ __device__ __forceinline__ void consume(const TileRegs<K, DT, U, OPT>& r, const 
 
 // Vector path over nfull consecutive full tiles of one parameter group: groups of U tiles,
 // then U/2, ... down to single tiles.
-template <int K, int DT, int OPT, int SL, bool HD, int U, class A>
-__device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t nfull, const A& a,
+template <int K, int DT, int OPT, int SL, bool HD, int U, class A, class SP>
+__device__ __forceinline__ void fast_run(const SP& sp, uint64_t e, uint32_t nfull, const A& a,
                                          const GroupDev& G, float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     constexpr int BS = launch_block(K, DT, OPT, SL);
     constexpr uint64_t TE = static_cast<uint64_t>(BS) * Grad<DT>::EPT;
@@ -347,15 +352,15 @@ __device__ __forceinline__ void fast_run(const SpanDev& sp, uint64_t e, uint32_t
 // vector straddles the span's first or last element or a bound take the slow way, so such a tile costs
 // little more than a full one (ResNet-50's batch-norm tensors and ViT's biases put a group change
 // into roughly every hundredth tile; one span per tensor puts an edge into every tensor).
-template <int K, int DT, int OPT, int SL, class A>
-__device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0, const A& a, uint32_t j,
+template <int K, int DT, int OPT, int SL, class A, class SP>
+__device__ __forceinline__ void careful_tile(const SP& sp, uint64_t tile_e0, const A& a, uint32_t j,
                                              float clip, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     using GR = Grad<DT>;
     constexpr int EPT = GR::EPT;
     constexpr int BS = launch_block(K, DT, OPT, SL);
     const bool use_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum);
     const bool load_s1 = is_adam(OPT) || (OPT == OPT_SGD && a.opt.has_momentum && !a.opt.first_step);
-    const BoundDev* bd = sp.bound_count ? a.bounds + sp.bound_begin : nullptr;
+    ConstBounds bd = sp.bound_count ? const_bounds(a.bounds + sp.bound_begin) : nullptr;
     const uint64_t e_first = tile_e0 + static_cast<uint64_t>(threadIdx.x) * EPT;
     const bool all_live = e_first >= sp.lo && e_first + EPT <= sp.hi;
     bool one_group = true;
@@ -408,8 +413,8 @@ __device__ __forceinline__ void careful_tile(const SpanDev& sp, uint64_t tile_e0
 }
 
 // Tiles [lt0, lt1) of one span (tile indices local to the span).
-template <int K, int DT, int OPT, int SL, bool HD, class A>
-__device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
+template <int K, int DT, int OPT, int SL, bool HD, class A, class SP>
+__device__ __forceinline__ void span_range(const SP& sp, uint32_t lt0, uint32_t lt1, uint32_t j0,
                                            const A& a, typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     const float clip = a.grad_scale ? *a.grad_scale : 1.0f;      // uniform: one scalar load per workgroup
     using GR = Grad<DT>;
@@ -421,7 +426,7 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
     constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
     const uint32_t nb = sp.bound_count;
-    const BoundDev* bd = nb ? a.bounds + sp.bound_begin : nullptr;
+    ConstBounds bd = nb ? const_bounds(a.bounds + sp.bound_begin) : nullptr;
     uint32_t lt = lt0, j = j0;
     while (lt < lt1) {
         const uint64_t e0 = static_cast<uint64_t>(lt) * TE;
@@ -454,8 +459,8 @@ __device__ __forceinline__ void span_range(const SpanDev& sp, uint32_t lt0, uint
 
 // Statistics kernels carry two copies of the arithmetic: one with the default halves
 // (even worker -> A, odd -> B) resolved at compile time, one driven by the half mask.
-template <int K, int DT, int OPT, int SL, class A>
-__device__ __forceinline__ void run_chunk(const SpanDev& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const A& a,
+template <int K, int DT, int OPT, int SL, class A, class SP>
+__device__ __forceinline__ void run_chunk(const SP& sp, uint32_t lt0, uint32_t lt1, uint32_t j0, const A& a,
                                           typename StatAcc<DT>::type (&acc)[NStats<K, SL>::value]) {
     if constexpr (SL) {
         constexpr uint32_t kDefaultMask = 0xAAAAu & ((1u << K) - 1u);
@@ -554,7 +559,7 @@ __device__ __forceinline__ void workgroup_chunk(const KArgs& a, const A& s, uint
         const uint32_t lt1 = lt0 + CT < tiles ? lt0 + CT : tiles;
         uint32_t j0 = 0;
         if (sp.bound_count) {                  // largest j with bounds[j].start <= first live element
-            const BoundDev* bd = a.bounds + sp.bound_begin;
+            ConstBounds bd = const_bounds(a.bounds + sp.bound_begin);
             const uint64_t e0 = static_cast<uint64_t>(lt0) * TE;
             const uint64_t rel = (e0 > sp.lo ? e0 : sp.lo) - sp.lo;
             uint32_t lo = 0, hi = sp.bound_count;
@@ -566,11 +571,17 @@ __device__ __forceinline__ void workgroup_chunk(const KArgs& a, const A& s, uint
         }
         run_chunk<K, DT, OPT, SL>(sp, lt0, lt1, j0, s, acc);
     } else {
-        const ChunkDesc c = a.chunks[b];
-        const SpanDev& sp = a.spans[c.span];
+        // The plan's tables are not written while a launch that names them runs: read through the constant
+        // address space, their fields are loaded like kernel arguments (uniform loads the compiler may move,
+        // repeat or keep as it likes) instead of being fetched again after every store that might alias them.
+        typedef const __attribute__((address_space(4))) ChunkDesc* ConstChunk;
+        typedef __attribute__((address_space(4))) SpanDev ConstSpan;
+        ConstChunk cp = (ConstChunk)(a.chunks + b);
+        const uint32_t c_span = cp->span, c_tile0 = cp->tile0, c_bound0 = cp->bound0;
+        const ConstSpan& sp = *(const ConstSpan*)(a.spans + c_span);
         const uint32_t tiles = static_cast<uint32_t>((sp.hi + TE - 1) / TE);
-        const uint32_t lt1 = c.tile0 + CT < tiles ? c.tile0 + CT : tiles;
-        run_chunk<K, DT, OPT, SL>(sp, c.tile0, lt1, c.bound0, s, acc);
+        const uint32_t lt1 = c_tile0 + CT < tiles ? c_tile0 + CT : tiles;
+        run_chunk<K, DT, OPT, SL>(sp, c_tile0, lt1, c_bound0, s, acc);
     }
 }
 
