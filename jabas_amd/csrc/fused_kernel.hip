@@ -6,7 +6,7 @@
 //   - one workgroup per chunk of consecutive tiles of one span; a tile is one 16-byte vector of
 //     every fp32 buffer (one 8-byte vector of a bf16 gradient buffer) per thread. Threads per
 //     workgroup and tiles per chunk depend on the kernel family (launch_block / launch_chunk_tiles):
-//     256 threads x 2 or 4 tiles with statistics, 128 x 2, 256 x 2 or 512 x 1 without. Small,
+//     256 threads x 2 or 4 tiles with statistics, 128 x 2, 256 x 2 or 256 x 4 without. Small,
 //     short-lived workgroups dispatched in order keep the part of every buffer that is being
 //     streamed at any moment compact, which on MI355X sustains a markedly higher HBM rate than a
 //     persistent grid that spreads over the whole buffers;

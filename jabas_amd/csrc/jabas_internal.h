@@ -19,10 +19,16 @@ namespace jabas {
 //                                 1024 threads were all slower (-2 ... -15 %)
 //   similarity sums only          256 threads x 2 tiles: with four sums the K > 4 kernels fit 4 waves per SIMD
 //                                 with two tiles of loads in flight
-//   plain with optimizer, K > 4   512 threads x 1 tile: +3 ... +8 % over 256 x 4 (bf16 and fp32, SGD and Adam);
-//                                 aggregate-only launches lose 20 % there and stay at 256 x 4
-//   plain, SGD, fp32, K <= 4      128 threads x 2 tiles: +2 ... +5 % over 256 x 2
-//   plain, everything else        256 threads x 2 tiles
+//   plain with optimizer, K > 4   256 threads x 2 tiles: +1 % over 512 x 1 and 512 x 2, +3 % over 256 x 4;
+//                                 aggregate-only launches stay at 256 x 4
+//   plain, Adam kinds, K <= 4     256 threads x 4 tiles, all loads of the chunk in flight at once: +0.5 ... +1.4 %
+//                                 over 256 x 2 (8 tiles: -4 %)
+//   plain, SGD, fp32, K <= 4      128 threads x 2 tiles: +2 ... +5 % over 256 x 2; 128 x 4 loses 5 % on the short
+//                                 ResNet-50 launch when the buffers rotate out of the last-level cache (and reads
+//                                 2 % faster than 128 x 2 when they do not: size sweeps over one buffer set mislead)
+//   plain, everything else K <= 4 256 threads x 2 tiles
+// (these figures are from after the planned launches began to read their tables through the constant address
+// space; before that the plain K > 4 kernels were best at 512 x 1 and the K <= 4 ones at 2 tiles).
 // The macros let a tuning build try other shapes without touching the sources.
 #ifndef JABAS_BLOCK
 #define JABAS_BLOCK 256
@@ -31,7 +37,7 @@ namespace jabas {
 #define JABAS_BLOCK_SGD 128
 #endif
 #ifndef JABAS_BLOCK_MANYK
-#define JABAS_BLOCK_MANYK 512
+#define JABAS_BLOCK_MANYK 256
 #endif
 #ifndef JABAS_BLOCK_SIM_MANYK
 #define JABAS_BLOCK_SIM_MANYK 256
@@ -43,13 +49,16 @@ namespace jabas {
 #define JABAS_CHUNK_TILES_HI 4
 #endif
 #ifndef JABAS_CHUNK_TILES_MANYK
-#define JABAS_CHUNK_TILES_MANYK 1
+#define JABAS_CHUNK_TILES_MANYK 2
 #endif
 #ifndef JABAS_CHUNK_TILES_SIM_MANYK
 #define JABAS_CHUNK_TILES_SIM_MANYK 2
 #endif
 #ifndef JABAS_CHUNK_TILES_SIM_LO
 #define JABAS_CHUNK_TILES_SIM_LO JABAS_CHUNK_TILES_LO
+#endif
+#ifndef JABAS_CHUNK_TILES_PLAIN_LO
+#define JABAS_CHUNK_TILES_PLAIN_LO 4
 #endif
 constexpr int kBlock = JABAS_BLOCK;         // default threads per workgroup (256 = 4 wave64)
 constexpr int kWaves = kBlock / 64;
@@ -72,6 +81,7 @@ __host__ __device__ constexpr int launch_block(int K, int grad_dtype, int opt_cl
 __host__ __device__ constexpr int launch_chunk_tiles(int K, int /*grad_dtype*/, int opt_class, int stats) {
     if (stats == 2) return K > 4 ? JABAS_CHUNK_TILES_SIM_MANYK : JABAS_CHUNK_TILES_SIM_LO;
     if (K > 4) return (stats || opt_class == 0) ? kMaxChunkTiles : JABAS_CHUNK_TILES_MANYK;
+    if (!stats && opt_class >= 2) return JABAS_CHUNK_TILES_PLAIN_LO;
     return kMinChunkTiles;
 }
 // Statistics level whose launch shape (and chunk table of a plan) a level uses.
@@ -85,8 +95,8 @@ constexpr int imin(int a, int b) { return a < b ? a : b; }
 constexpr int kMinStatsChunkElems = 4 * imin(imin(JABAS_BLOCK * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_SIM_LO),
                                              JABAS_BLOCK_SIM_MANYK * JABAS_CHUNK_TILES_SIM_MANYK);
 // Fewest elements any chunk covers, over all shapes: sizes blobs that must fit every launch.
-constexpr int kMinChunkElems = imin(kMinStatsChunkElems,
-                                    4 * imin(imin(JABAS_BLOCK_SGD * JABAS_CHUNK_TILES_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
+constexpr int kMinChunkElems = imin(imin(kMinStatsChunkElems, 4 * JABAS_BLOCK_SGD * JABAS_CHUNK_TILES_LO),
+                                    4 * imin(imin(JABAS_BLOCK * JABAS_CHUNK_TILES_PLAIN_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
                                              imin(JABAS_BLOCK_MANYK * JABAS_CHUNK_TILES_MANYK, JABAS_BLOCK * JABAS_CHUNK_TILES_HI)));
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
 

@@ -387,9 +387,9 @@ def test_plan_encode_rejects_overlapping_written_buffers():
 
 def test_launch_shape_follows_what_the_plan_is_encoded_for():
     """Launches with full statistics rows run 256-thread workgroups of 2 tiles (K <= 4) or 4 tiles, with
-    similarity sums only 2 tiles for every K; plain launches 512 threads x 1 tile for K > 4, 128 threads x
-    2 tiles for SGD with fp32 gradients and K <= 4, else 256 x 2. A plan holds a chunk table per shape and
-    serves launches of its own optimizer class only."""
+    similarity sums only 2 tiles for every K; plain launches with an optimizer 256 threads x 2 tiles for K > 4,
+    128 threads x 2 tiles for SGD with fp32 gradients and K <= 4, 256 x 4 for the Adam kinds and K <= 4, else 256 x 2;
+    aggregate-only launches 256 x 2 (K <= 4) or 256 x 4. A plan holds a chunk table per shape and serves launches of its own optimizer class only."""
     lib = L.lib()
     n = 10 * 4096
     def chunks(K, dtype, opt, gs=4):
@@ -400,7 +400,7 @@ def test_launch_shape_follows_what_the_plan_is_encoded_for():
     assert chunks(4, L.F32, L.OPT_SGD)[0] == (n // 1024, n // 2048)
     assert chunks(5, L.F32, L.OPT_SGD)[0] == (n // 2048, n // 4096)
     assert chunks(2, L.BF16, L.OPT_SGD, gs=2)[0] == (n // 2048, n // 2048)
-    assert chunks(2, L.F32, L.OPT_ADAM)[0] == (n // 2048, n // 2048)
+    assert chunks(2, L.F32, L.OPT_ADAM)[0] == (n // 4096, n // 2048)
     assert chunks(8, L.BF16, L.OPT_ADAMW, gs=2)[0] == (n // 2048, n // 4096)
     assert chunks(2, L.F32, L.OPT_NONE)[0] == (n // 2048, n // 2048)
     assert chunks(8, L.F32, L.OPT_NONE)[0] == (n // 4096, n // 4096)
@@ -479,16 +479,14 @@ def test_statistics_over_too_many_spans_are_refused_before_any_launch():
 
 def _shape_model(K, dtype, opt_class, stats):
     """(threads per workgroup, tiles per workgroup) as documented for the launch shapes."""
-    if stats or opt_class == 0:
+    if stats or opt_class == 0 or K > 4:
         block = 256
-    elif K > 4:
-        block = 512
     else:
         block = 128 if (opt_class == 1 and dtype == L.F32) else 256
     if K > 4:
-        tiles = 2 if stats == 2 else (4 if (stats or opt_class == 0) else 1)
+        tiles = 2 if stats == 2 else (4 if (stats or opt_class == 0) else 2)
     else:
-        tiles = 2
+        tiles = 4 if (not stats and opt_class >= 2) else 2
     return block, tiles
 
 
