@@ -293,18 +293,26 @@ class VSWSyncTrainer:
                         st[key] = eng.state_view(j, i).view(p.shape)
                     else:
                         st.pop(key, None)
-        if not sgd and not eng.state_is_live and not getattr(optimizer, "_jabas_moment_hooks", False):
-            trainer = weakref.ref(self)
+        if not sgd and not eng.state_is_live:
+            hooked = hasattr(optimizer, "_jabas_moment_owner")
+            optimizer._jabas_moment_owner = weakref.ref(self)      # the trainer whose arenas the hooks read
+            if hooked:
+                return
+
+            def owner(opt):
+                t = opt._jabas_moment_owner()
+                return t if t is not None and t.main_optimizer is opt and t.engine is not None \
+                    and not t.engine.state_is_live else None
 
             def before(opt):
-                t = trainer()
-                if t is not None and t.main_optimizer is opt and t.engine is not None:
+                t = owner(opt)
+                if t is not None:
                     torch.cuda.synchronize(t.gpu)
                     t._expose_state(opt, moments=True)
 
             def after(opt, state_dict):
-                t = trainer()
-                if t is not None and t.main_optimizer is opt and t.engine is not None:
+                t = owner(opt)
+                if t is not None:
                     # torch packs the per-parameter dictionaries themselves: the result keeps shallow copies of
                     # them (with the moments), the optimizer's own lose the moments again
                     state_dict["state"] = {idx: dict(st) for idx, st in state_dict["state"].items()}
@@ -313,7 +321,6 @@ class VSWSyncTrainer:
 
             optimizer.register_state_dict_pre_hook(before)
             optimizer.register_state_dict_post_hook(after)
-            optimizer._jabas_moment_hooks = True
 
     def _refresh_hyperparameters(self):
         """Learning rate and weight decay as the caller's optimizer object holds them now."""
