@@ -830,13 +830,20 @@ def test_random_plans_match_the_oracle(gpu, seed):
     fans = [_dev(torch.zeros(total), gpu, skew()) for _ in range(n_fan)]
     kind = sync.opt_kind(opt)
     adam = kind in (L.OPT_ADAM, L.OPT_ADAMW)
+    # every other Adam case keeps the moments interleaved in one arena (blocks of 256, 1024 or 8192 elements), the
+    # arena's element 0 at the weights' place of a 16-byte line (of a 256-byte line when all buffers share one)
+    arena = None
+    if adam and seed % 4 >= 2:
+        arena_first = skew()
+        arena = sync.MomentArena(arena_first + total, 2, gpu, (8, 10, 13)[seed % 3])
     spans_h, spans_d = [], []
     for o, s, b in zip(offs, sizes, bounds):
         sl = slice(o, o + s)
         spans_h.append((o, s, b))
+        state = dict(moments=(arena, arena_first + o)) if arena is not None else \
+            dict(state1=s1_d[sl] if opt else None, state2=s2_d[sl] if adam else None)
         spans_d.append(sync.SpanSpec([g[sl] for g in dg], agg_out=agg_d[sl], param=p_d[sl] if opt else None,
-                                     state1=s1_d[sl] if opt else None, state2=s2_d[sl] if adam else None,
-                                     fanout=[f[sl] for f in fans], bounds=b))
+                                     fanout=[f[sl] for f in fans], bounds=b, **state))
     plan = sync.SyncPlan(spans_d, kind)
     hg_work = [t.clone() for t in hg]
     block = sync.StepScalars(gpu) if opt and seed % 2 else None
@@ -862,6 +869,8 @@ def test_random_plans_match_the_oracle(gpu, seed):
             scale = want[:, 1:3].abs().max(dim=1, keepdim=True).values.clamp_min(1e-300)   # dot may cancel: bound it by the norms
             assert bool(((got - want).abs() <= rtol * want.abs() + 1e-9 * scale).all()), f"stats step {step}"
         if opt:
+            if arena is not None:
+                s1_d, s2_d = arena.read(0, arena_first, total), arena.read(1, arena_first, total)
             for i, (o, s, _) in enumerate(spans_h):
                 assert torch.equal(_bits(p_d[o:o + s]), _bits(p_h[o:o + s])), f"weights span {i} step {step}"
                 assert torch.equal(_bits(s1_d[o:o + s]), _bits(s1_h[o:o + s])), f"state1 span {i} step {step}"
@@ -878,6 +887,9 @@ def test_random_plans_match_the_oracle(gpu, seed):
         covered[o:o + s] = True
     if opt and (~covered).any():
         assert torch.equal(_bits(p_d)[~covered], _bits(_host_state(total, 40 + seed))[~covered])
+        if arena is not None:                                # the moments of elements no span owns stayed zero
+            assert torch.count_nonzero(arena.read(0, arena_first, total)[~covered.to(gpu)]) == 0
+            assert torch.count_nonzero(arena.read(1, arena_first, total)[~covered.to(gpu)]) == 0
         for f in fans:
             assert torch.count_nonzero(f.cpu()[~covered]) == 0
     if not in_place and (~covered).any():
