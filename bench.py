@@ -313,6 +313,9 @@ def hook_path_threads(cfg, eng, device, steps, warmup, torch, launch_streams, ba
     for t in threads:
         t.start()
     wall0 = 0.0
+    gc_was_on = gc.isenabled()            # as in timed_region: no collection pause inside a measured step
+    gc.collect()
+    gc.disable()
     try:
         for it in range(n_iter):
             if it == warmup:
@@ -326,6 +329,9 @@ def hook_path_threads(cfg, eng, device, steps, warmup, torch, launch_streams, ba
             state.grad_placeholder.clear()
     except threading.BrokenBarrierError:
         raise RuntimeError(f"hook threads failed: {errors}")
+    finally:
+        if gc_was_on:
+            gc.enable()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - wall0) * 1e3 / steps
     for t in threads:
