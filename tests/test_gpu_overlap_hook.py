@@ -262,11 +262,16 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
     assert local.native_launches == (2 * len(SHAPES) if mode == "per_bucket" else 0)
 
 
-@pytest.mark.parametrize("kind", ["sgd", "adam"])
+@pytest.mark.parametrize("kind", ["sgd", "adam", "adam_interleaved"])
 def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
     """The arenas handed over by the caller (``opt=`` + ``param_buckets=``) instead of built from bucket
-    objects: views into one weight arena, one state arena each, two parameter groups, one replica."""
+    objects: views into one weight arena, one state arena each (or, "adam_interleaved", the moments of all
+    buckets in ONE interleaved arena, every bucket naming its first element in it), two parameter groups, one
+    replica; through the native meeting point from the second step on."""
+    from jabas_amd import sync
     from jabas_amd.local_sync import LocalBucketSync
+    interleaved = kind == "adam_interleaved"
+    kind = kind.replace("_interleaved", "")
     K, batches, sizes = 2, (3, 1), [70001, 2049]
     opt = _opt_dict("sgd") if kind == "sgd" else dict(kind="adam", betas=(0.9, 0.999), eps=1e-8,
                                                      groups=[dict(lr=2e-3, weight_decay=0.0),
@@ -276,12 +281,14 @@ def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
     p_h = torch.randn(total, generator=gen) * 0.05
     s1_h, s2_h = torch.zeros(total), torch.zeros(total)
     p_d, s1_d, s2_d, fan = p_h.to(gpu), s1_h.to(gpu), s2_h.to(gpu), torch.zeros(total, device=gpu)
+    arena = sync.MomentArena(total, 2, gpu, 10) if interleaved else None
     spans, pbs, off = [], {}, 0
     for b, n in enumerate(sizes):
         bounds = ((0, 0), (n // 3, 1), (2 * n // 3 + 1, 0))
         sl = slice(off, off + n)
-        pbs[b] = dict(param=p_d[sl], state1=s1_d[sl], state2=None if kind == "sgd" else s2_d[sl], bounds=bounds,
-                      fanout=[fan[sl]])
+        state = dict(moments=(arena, off)) if interleaved else \
+            dict(state1=s1_d[sl], state2=None if kind == "sgd" else s2_d[sl])
+        pbs[b] = dict(param=p_d[sl], bounds=bounds, fanout=[fan[sl]], **state)
         spans.append((off, n, bounds))
         off += n
     local = LocalBucketSync(batches, opt=opt, param_buckets=pbs)
@@ -296,6 +303,8 @@ def test_explicit_param_buckets_with_two_groups_and_fan_out(gpu, kind):
         local.finish_step()
         torch.cuda.synchronize()
         agg_h, _ = O.sync_step(host, batches, spans, opt, p_h, s1_h, s2_h, step=step, first_step=(step == 1))
+        if interleaved:
+            s1_d, s2_d = arena.read(0), arena.read(1)
         assert _same(bufs[0], agg_h) and _same(p_d, p_h) and _same(s1_d, s1_h) and _same(fan, p_h), step
         if kind != "sgd":
             assert _same(s2_d, s2_h), step
