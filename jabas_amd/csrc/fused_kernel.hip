@@ -94,12 +94,13 @@ template <> struct Grad<JABAS_BF16> {
 
 constexpr int OPT_NONE = 0, OPT_SGD = 1, OPT_ADAM = 2, OPT_AMS = 3;    // OPT_AMS: Adam / AdamW with amsgrad
 __host__ __device__ constexpr bool is_adam(int opt) { return opt == OPT_ADAM || opt == OPT_AMS; }
-// Kernels with statistics over more than four gradient streams form the addresses of the vector path as
-// scalar base + 32-bit lane offset (measured on the ViT-L/16 set, K = 8 bf16: +0.5 % with full rows, +2 % with
-// similarity sums); their spans that 32-bit byte offsets do not reach (over 4 GiB of fp32 per buffer) go
-// through the careful path tile by tile: correct but slower. Everywhere else 64-bit vector addresses are
-// faster (the scalar bases compete with the launch constants for scalar registers: -0.5 ... -2.5 %).
-__host__ __device__ constexpr bool narrow_addressing(int K, int SL) { return SL != 0 && K > 4; }
+// Kernels with statistics form the addresses of the vector path as scalar base + 32-bit lane offset (measured
+// on the ViT-L/16 set, K = 8 bf16: +0.5 % with full rows, +2 % with similarity sums; K = 4 fp32 Adam: 8-9 fewer
+// VGPRs, full rows 131 -> 123 and 4 waves per SIMD instead of 3, ViT-B/16 +1.2 % with similarity sums, +0.4 % with
+// full rows, GNMT +-0.3 %); their spans that 32-bit byte offsets do not reach (over 4 GiB of fp32 per buffer)
+// go through the careful path tile by tile: correct but slower. The plain kernels keep 64-bit vector addresses
+// (no gain there: their registers are not what limits them).
+__host__ __device__ constexpr bool narrow_addressing(int /*K*/, int SL) { return SL != 0; }
 
 // Statistics level of a launch: 0 none, 1 the full row (4 + K sums), 2 the four sums of the halves and of
 // the aggregate only (what the cosine similarity and global-norm clipping read), 3 the full row and the
