@@ -610,12 +610,20 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
     // Residency cap through idle dynamic LDS (160 KB per CU). Fewer resident workgroups keep the
     // streamed window of every buffer more compact, which the memory system rewards on write-heavy
     // mixes as long as the kernel does not need the waves to hide its own arithmetic. Measured (A/B in
-    // one process): Adam/AdamW without statistics at K <= 4, fp32 gradients, gains 1-4 % at 5 workgroups
-    // per CU instead of the 6 its registers allow; SGD kernels and every statistics kernel lose.
+    // one process, and over whole bench runs with rotating buffers): Adam/AdamW at K <= 4 with fp32
+    // gradients gains 0-4 % without statistics at 5 workgroups per CU instead of the 6 its registers
+    // allow, and 0.2-2.4 % with statistics at 3 workgroups per CU instead of 4 (more with replica
+    // weights to refresh); SGD kernels, bf16 gradients and K > 4 lose or stay flat.
 #ifndef JABAS_IDLE_LDS_BYTES
 #define JABAS_IDLE_LDS_BYTES 32768u
 #endif
-    constexpr unsigned idle = (OPT == OPT_ADAM && !SL && K <= 4 && DT == JABAS_F32) ? JABAS_IDLE_LDS_BYTES : 0u;
+#ifndef JABAS_STATS_LDS_BYTES
+#define JABAS_STATS_LDS_BYTES 53248u      // per workgroup, flush_stats' own table included: three workgroups per CU
+#endif
+    constexpr bool capped = OPT == OPT_ADAM && K <= 4 && DT == JABAS_F32;
+    constexpr unsigned flush_bytes = NStats<K, SL>::value * launch_block(K, DT, OPT, SL) * 8u;   // fp64 [value][thread]
+    static_assert(!capped || !SL || flush_bytes < JABAS_STATS_LDS_BYTES, "the cap is what is left beside the table");
+    constexpr unsigned idle = !capped ? 0u : SL ? JABAS_STATS_LDS_BYTES - flush_bytes : JABAS_IDLE_LDS_BYTES;
     const dim3 block(launch_block(K, DT, OPT, SL));
     if constexpr (SL == JABAS_STATS_GRAM && K > JABAS_STATS_GRAM_MAX_K) {
         return static_cast<int>(hipErrorInvalidValue);              // refused by the front before it gets here
