@@ -266,8 +266,10 @@ def hook_path_threads(cfg, eng, device, steps, warmup, torch, launch_streams, ba
         bucket_slices.append(sl)
         pbs[b] = dict(param=eng.param[sl], bounds=bounds, agg_out=None if eng.agg is eng.grads[0] else eng.agg[sl],
                       **eng.state_of_span(off, numel))
-    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs, stream=torch.cuda.Stream(device),
-                            launch_streams=launch_streams)
+    # launch_streams = 0: no launch stream, a bucket's launch on the stream of the VSW that handed it over last
+    local = LocalBucketSync(cfg.batches, opt=cfg.opt, param_buckets=pbs,
+                            stream=torch.cuda.Stream(device) if launch_streams else None,
+                            launch_streams=launch_streams, launch_on_last_vsw=not launch_streams)
     local.step_count = eng.step_count
     local._momentum_ready = eng.step_count > 0
     state = H.GradientSimilarityState(None, K + K % 2, None, [], 1 if cfg.stats else 10 ** 9).attach_local(local)
@@ -416,8 +418,8 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
             str(ls): bucket_launches(cfg, engines[0], device, hsteps, hwarm, torch, ls) for ls in (1, 2, 3)}
         # the same hooks as training calls them: K threads on K streams with backward-like work between the buckets
         # (a leg of K host threads: whatever goes wrong in it is reported in its place, not instead of the line)
-        for ls in (1, 2):
-            key = f"hook_path_threads_{ls}_launch_stream{'s' if ls > 1 else ''}"
+        for ls in (1, 2, 0):
+            key = f"hook_path_threads_{ls}_launch_stream{'s' if ls > 1 else ''}" if ls else "hook_path_threads_launch_on_last_vsw"
             try:
                 res[key] = hook_path_threads(cfg, engines[0], device, hsteps, max(3, hwarm // 3), torch, ls,
                                              engine_ms=ms_per_step)

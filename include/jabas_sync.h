@@ -395,8 +395,11 @@ int jabas_rdv_drop_bucket(JabasRendezvous* r, uint32_t bucket);
 
 /* VSW k hands bucket `bucket` over on vsw_stream. want_stats counts from VSW 0 only (its hook knows
  * whether this is a statistics step); args: this step's arguments (args->stats is replaced by
- * stats_level or JABAS_STATS_NONE accordingly). Returns a JABAS_RDV_* code or a negative JabasStatus
- * (JABAS_ERR_STATE: handed over twice). */
+ * stats_level or JABAS_STATS_NONE accordingly). launch_stream: where the launch goes if this
+ * hand-over completes the bucket (only the completing call's word is used, so it may differ from
+ * call to call: a launch stream of the caller's, VSW 0's stream, or vsw_stream itself to put the
+ * launch behind the work of whichever VSW comes last; that VSW then records no event).
+ * Returns a JABAS_RDV_* code or a negative JabasStatus (JABAS_ERR_STATE: handed over twice). */
 int jabas_rdv_publish(JabasRendezvous* r, int32_t k, uint32_t bucket, int32_t want_stats,
                       jabas_stream_t vsw_stream, jabas_stream_t launch_stream,
                       const JabasStepArgs* args, int32_t stats_level);

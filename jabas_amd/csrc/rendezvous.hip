@@ -128,16 +128,18 @@ JABAS_API int jabas_rdv_publish(JabasRendezvous* r, int32_t k, uint32_t bucket, 
         const uint32_t bit = 1u << k;
         if (b->arrived & bit) return JABAS_ERR_STATE;
         hipStream_t mine = static_cast<hipStream_t>(vsw_stream);
-        // VSW 0's own stream needs no event when the launch is queued on it; a peer cannot know yet which
-        // stream the launch will take (VSW 0 may hand its bucket over later) and always records one
-        if (k != 0 || vsw_stream != launch_stream) {
+        const bool complete = (b->arrived | bit) == (r->K >= 32 ? 0xffffffffu : (1u << r->K) - 1u);
+        // The launch goes on the stream the completing hand-over names: only that hand-over knows it (callers
+        // may put a bucket's launch on the stream of whichever VSW comes last), so every other one records an
+        // event, and the completing one does unless the launch follows its own work on its own stream.
+        if (!complete || vsw_stream != launch_stream) {
             if (hipEventRecord(b->events[k], mine) != hipSuccess) return JABAS_ERR_LAUNCH;
             b->recorded |= bit;
         }
         b->streams[k] = mine;
         b->arrived |= bit;
         if (k == 0) b->want_stats = want_stats != 0;
-        if (b->arrived != (r->K >= 32 ? 0xffffffffu : (1u << r->K) - 1u)) return JABAS_RDV_WAITING;
+        if (!complete) return JABAS_RDV_WAITING;
         // complete: this call launches. The bucket is free for the next step from here on (its events are
         // waited for below, before any thread can record them again: the VSW streams are held back by the
         // caller's end-of-step event, which is queued after this launch).

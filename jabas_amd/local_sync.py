@@ -104,7 +104,7 @@ class LocalBucketSync:
 
     def __init__(self, batches, launcher=None, opt=None, param_buckets=None, deferred=False, stream=None,
                  optimizer=None, stats_level="similarity", batch_bytes=0, share_weights=False, write_aggregate=True,
-                 launch_streams=2, auto_finish=True, interleave_moments=False):
+                 launch_streams=2, auto_finish=True, interleave_moments=False, launch_on_last_vsw=False):
         """deferred: collect the buckets of a step and queue ONE planned launch over all of them in
         ``finish_step`` instead of one launch per bucket as each becomes complete. The per-bucket mode
         overlaps the sync with the rest of the backward pass; the deferred mode spends less GPU time
@@ -135,6 +135,14 @@ class LocalBucketSync:
         38 buckets: 2.61 ms a step on one stream, 6 us of idle queue between launches, 2.37 ms on two, which is
         what one launch over all buckets takes; a third stream gains nothing). ``finish_step`` orders the VSW
         streams behind every one of them.
+
+        launch_on_last_vsw (without ``stream=``): a bucket's launch goes on the stream of the VSW whose hand-over
+        completed the bucket, behind an event from every other VSW's stream, instead of on VSW 0's stream or on
+        launch streams of its own. No stream beyond the K the VSWs run on is needed (a GPU serves a process
+        through a handful of hardware queues; streams beyond them share one and run in submission order, which
+        launch streams on top of three or more VSW streams run into), consecutive buckets completed by
+        different VSWs still overlap their ramp-up and drain, and the VSW that came last finds the launch ahead
+        of the rest of its own backward pass, which nobody else waits for.
 
         auto_finish: when the bucket objects tell which bucket is a replica's last (``GradBucket.is_last()``),
         the hand-over that completes that bucket also ends the step (``finish_step`` with the streams the hooks
@@ -205,6 +213,10 @@ class LocalBucketSync:
         self._n_launch_streams = max(1, int(launch_streams))
         self._sync_streams = []                # the launch streams; empty: VSW 0's own stream carries the launches
         self._sync_stream = stream
+        self.launch_on_last_vsw = bool(launch_on_last_vsw)
+        if self.launch_on_last_vsw and stream is not None:
+            raise ValueError("launch_on_last_vsw puts the launches on the VSWs' own streams: no stream= beside it")
+        self._bucket_stream = {}               # launch_on_last_vsw: bucket index -> stream of the VSW that completed it
         self.auto_finish = bool(auto_finish)
         self.interleave_moments = bool(interleave_moments)
         self._moment_home = {}                 # id(parameter) -> (MomentArena, first element, parameter): interleaved moments
@@ -251,6 +263,10 @@ class LocalBucketSync:
     def _launch_stream(self, bucket_index=0):
         if self._sync_streams:
             return self._sync_streams[bucket_index % len(self._sync_streams)]
+        if self.launch_on_last_vsw:
+            own = self._bucket_stream.get(bucket_index)
+            if own is not None:
+                return own
         return self._main_stream
 
     # ------------------------------------------------------------------ who hands over what
@@ -524,7 +540,8 @@ class LocalBucketSync:
         event = stream = None
         if tensor.is_cuda:
             stream = self._current_stream(tensor) if _stream is None else _stream
-            if not self.deferred and not self.batch_bytes and (k != 0 or self._sync_stream is not None):
+            if not self.deferred and not self.batch_bytes and (k != 0 or self._sync_stream is not None
+                                                                or self.launch_on_last_vsw):
                 # VSW 0's own stream needs none when the launch is queued on it. A fresh event every time:
                 # recording one event again step after step (to save its creation) made the waits on it
                 # three times as expensive on this runtime. (Batched and deferred launches order themselves
@@ -549,6 +566,9 @@ class LocalBucketSync:
             complete = ready = slot.count == self.K
             if ready:
                 del self._slots[bucket_index]
+                if self.launch_on_last_vsw and stream is not None and not self._sync_streams:
+                    self._bucket_stream[bucket_index] = stream     # the launch follows this VSW's own work
+                    slot.events[k] = None
                 if self._batch_bytes_asked and stream is not None:
                     self._bucket_bytes[bucket_index] = tensor.numel() * tensor.element_size()
                 if self.deferred or (self.batch_bytes and stream is not None):
@@ -656,8 +676,13 @@ class LocalBucketSync:
         if k == 0:
             self._main_stream, self._main_ptr = stream, ptr
             self._native_on_done[bucket_index] = on_done
-        launch = self._launch_stream(bucket_index)
-        main_ptr = launch.cuda_stream if self._sync_streams else self._main_ptr
+        if self._sync_streams:
+            launch = self._launch_stream(bucket_index)
+            main_ptr = launch.cuda_stream
+        elif self.launch_on_last_vsw:
+            launch, main_ptr = stream, ptr                      # used only if this hand-over completes the bucket
+        else:
+            launch, main_ptr = self._main_stream, self._main_ptr
         call = known[2]
         stamp = (self.step_count, self.lr_scale, self.accumulations)
         ent = self._native_args.get((known[3], call.with_opt))
@@ -676,7 +701,9 @@ class LocalBucketSync:
         row = call._rows[rc - L.RDV_LAUNCHED_ROW0] if rc >= L.RDV_LAUNCHED_ROW0 else None
         with self._lock:
             self._native_seen.pop(bucket_index, None)
-            self._launch_streams.add(self._launch_stream(bucket_index))
+            if self.launch_on_last_vsw and not self._sync_streams:
+                self._bucket_stream[bucket_index] = launch
+            self._launch_streams.add(launch)
             self.launched += 1
             self.native_launches += 1
             if call.with_opt:
@@ -825,8 +852,16 @@ class LocalBucketSync:
             return
         with_opt = [self.opt is not None and i in self.param_buckets for i in order]
         if (any(with_opt) and not all(with_opt)) or (with_opt[0] and self.grad_clip != float("inf")):
+            gate, gated = None, {main}
             for i, slot in zip(order, slots):          # buckets with and without weights behind them, or a norm
                 slot.events = [None] * self.K          # per bucket to wait for: one launch each after all
+                own = self._launch_stream(i)           # the VSW streams were ordered ahead of `main` only
+                if own not in gated:
+                    if gate is None:
+                        gate = torch.cuda.Event()
+                        gate.record(main)
+                    own.wait_event(gate)
+                    gated.add(own)
                 self._fire(i, slot)
             return
         try:

@@ -118,11 +118,21 @@ def test_launches_alternating_between_launch_streams(gpu, kind, gdt, mode, launc
     _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2), launch_streams=launch_streams)
 
 
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+@pytest.mark.parametrize("gdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["per_bucket", "batched", "deferred"])
+def test_launches_on_the_stream_of_the_vsw_that_came_last(gpu, kind, gdt, mode):
+    """``launch_on_last_vsw``: no stream beside the VSWs' own; VSW 0 always hands over first here, so every
+    launch sits on a peer's stream behind an event from VSW 0's. The same bits, and the second and third step
+    through the native meeting point."""
+    _hooks_with_optimizer(gpu, kind, gdt, mode, (4, 2, 2), launch_streams=0)
+
+
 # buckets of 8, 12 and 17 MB: a bucket's launch is still running when the next bucket is handed over
 BIG_SHAPES = [[(1024, 2048), (2048,)], [(1536, 2048), (7,)], [(2048, 1024), (1024,), (1100, 2000)]]
 
 
-@pytest.mark.parametrize("gdt,launch_streams", [(torch.float32, 1), (torch.bfloat16, 2)])
+@pytest.mark.parametrize("gdt,launch_streams", [(torch.float32, 1), (torch.bfloat16, 2), (torch.float32, 0)])
 def test_multi_megabyte_buckets_through_the_native_meeting_point(gpu, gdt, launch_streams):
     """K = 4 hook threads, buckets large enough that launches are in flight at the following hand-overs; the
     second and third step go through the native meeting point."""
@@ -130,10 +140,11 @@ def test_multi_megabyte_buckets_through_the_native_meeting_point(gpu, gdt, launc
                           SHAPES=BIG_SHAPES)
 
 
-@pytest.mark.parametrize("mode", ["per_bucket", "batched"])
-def test_eight_vsw_threads_with_bf16_buckets(gpu, mode):
+@pytest.mark.parametrize("mode,launch_streams", [("per_bucket", 1), ("batched", 1), ("per_bucket", 0)])
+def test_eight_vsw_threads_with_bf16_buckets(gpu, mode, launch_streams):
     """The largest configuration's shape: eight VSWs with batches 64..8, bf16 buckets, AdamW."""
-    _hooks_with_optimizer(gpu, "adamw", torch.bfloat16, mode, (64, 56, 48, 40, 32, 24, 16, 8))
+    _hooks_with_optimizer(gpu, "adamw", torch.bfloat16, mode, (64, 56, 48, 40, 32, 24, 16, 8),
+                          launch_streams=launch_streams)
 
 
 def _checkpointed(optimizer):
@@ -162,9 +173,11 @@ def _hooks_with_optimizer(gpu, kind, gdt, mode, batches, launch_streams=1, SHAPE
     # batched: complete buckets wait until 400 kB of them are ready, then go out as one planned launch
     keep = not mode.endswith("no_aggregate")
     mode = mode.replace("_no_aggregate", "")
+    # launch_streams=0: no launch stream at all, a bucket's launch on the stream of the VSW that completed it
     local = LocalBucketSync(batches, deferred=(mode == "deferred"), batch_bytes=400_000 if mode == "batched" else 0,
-                            stream=create_stream_for_optimizer(gpu), write_aggregate=keep, launch_streams=launch_streams,
-                            interleave_moments=interleave)
+                            stream=create_stream_for_optimizer(gpu) if launch_streams else None, write_aggregate=keep,
+                            launch_streams=launch_streams, interleave_moments=interleave,
+                            launch_on_last_vsw=not launch_streams)
     assert len(local._sync_streams) == launch_streams
     st = H.GradientSimilarityState(None, K + K % 2, None, [], 2).attach_local(local)
     main_hook = create_optimizer_hook(H.similimarity_allreduce_hook(H.subgroup_allreduce_hook), optimizer)
@@ -376,10 +389,13 @@ def test_native_meeting_point_errors_and_new_buffers(gpu):
     assert local.native_launches == before + len(sizes)
 
 
-def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
+@pytest.mark.parametrize("how", ["vsw0_stream", "batched_two_launch_streams", "last_vsw_stream"])
+def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu, how):
     """ShardGNMTAdam(grad_clip=) in the hook (examples/gnmt/seq2seq/train/shard_optimizer.py:8-29,75-76):
     every bucket's aggregate is scaled to norm <= grad_clip before Adam sees it. Oracle: the aggregate,
-    torch.nn.utils.clip_grad_norm_'s coefficient from its float64 norm, one fp32 product, Adam."""
+    torch.nn.utils.clip_grad_norm_'s coefficient from its float64 norm, one fp32 product, Adam. Also out of a
+    batch of buckets (each bucket still takes launches of its own, on its own launch stream, behind the batch's
+    stream waits) and on the stream of the VSW that came last."""
     from jabas_amd import ddp_comm_hooks as H, optim
     from jabas_amd.local_sync import LocalBucketSync
     from jabas_amd.train import create_optimizer_hook
@@ -393,7 +409,9 @@ def test_per_bucket_clipping_of_the_gnmt_shard_optimizer(gpu):
     clip = 0.05
     optimizer = optim.ShardGNMTAdam([p for bucket in replicas[0] for p in bucket], lr=2e-3, grad_clip=clip)
     opt = dict(kind="adam", betas=(0.9, 0.999), eps=1e-8, groups=[dict(lr=2e-3, weight_decay=0.0)])
-    local = LocalBucketSync(batches)
+    local = LocalBucketSync(batches, **dict(
+        vsw0_stream={}, last_vsw_stream=dict(launch_on_last_vsw=True),
+        batched_two_launch_streams=dict(stream=torch.cuda.Stream(gpu), launch_streams=2, batch_bytes=1 << 20))[how])
     st = H.IIDPState(None, 2).attach_local(local)
     main_hook = create_optimizer_hook(H.iidp_allreduce_hook, optimizer)
     p_h = [torch.cat([t.reshape(-1) for t in bucket]) for bucket in init]
