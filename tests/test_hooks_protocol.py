@@ -474,3 +474,19 @@ def test_auto_finish_can_be_switched_off():
     assert local.step_count == 0 and local.launched == 1
     local.finish_step()
     assert local.step_count == 1
+
+
+def test_launch_on_last_vsw_is_a_mode_without_launch_streams():
+    """The option puts launches on the VSWs' own streams: it excludes ``stream=`` (checked before any stream is
+    touched), and with host tensors (no streams at all) the protocol is what it is without it."""
+    with pytest.raises(ValueError, match="launch_on_last_vsw"):
+        LocalBucketSync([1, 1], launcher=Recorder(), stream=object(), launch_streams=1, launch_on_last_vsw=True)
+    rec = Recorder()
+    local = LocalBucketSync([1, 1], launcher=rec, launch_on_last_vsw=True)
+    g = [torch.full((3,), 1.0), torch.full((3,), 2.0)]
+    local.publish(1, 0, g[1])
+    assert rec.calls == []
+    local.publish(0, 0, g[0])
+    assert [c[0] for c in rec.calls] == [0] and float(g[0][0]) == 3.0
+    local.finish_step()
+    assert local.step_count == 1
