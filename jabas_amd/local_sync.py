@@ -340,7 +340,74 @@ class LocalBucketSync:
         self.optimizer = optimizer
         self._group_of = {id(p): gi for gi, g in enumerate(optimizer.param_groups) for p in g["params"]}
         self.grad_clip = float(getattr(optimizer, "grad_clip", float("inf")))
+        if hasattr(optimizer, "register_load_state_dict_post_hook"):
+            me = weakref.ref(self)
+
+            def adopt(o):
+                local = me()
+                if local is not None and local.optimizer is o:
+                    local._adopt_loaded_state()
+
+            optimizer.register_load_state_dict_post_hook(adopt)
         return self
+
+    def _adopt_loaded_state(self):
+        """``optimizer.load_state_dict`` puts fresh tensors into ``optimizer.state``; the launches read the
+        arenas. For every bucket already laid out the loaded moments are copied into its arenas (a parameter
+        the checkpoint holds no state for starts from zeros, as it would in torch) and the optimizer's
+        dictionaries show the arenas again; the step count follows the checkpoint's. Buckets laid out later
+        take the loaded tensors over when they are bound."""
+        bound = [pb for pb in self.param_buckets.values() if pb.get("params") is not None]
+        if not bound:
+            return
+        device = bound[0]["param"].device
+        torch.cuda.synchronize(device)
+        sgd = self.opt["kind"] == "sgd"
+        names = ("momentum_buffer",) if sgd else self._MOMENT_NAMES
+        steps, loaded_momentum = set(), False
+        self._bound_steps = {}
+        with torch.no_grad():
+            for pb in bound:
+                for prm in pb["params"]:
+                    st = self.optimizer.state[prm]
+                    n = prm.numel()
+                    home = self._moment_home.get(id(prm))
+                    if home is not None:
+                        arena, start, _ = home
+                        for j, name in enumerate(names[:arena.ways]):
+                            loaded = st.pop(name, None)
+                            flat = (loaded.to(device=device, dtype=torch.float32).reshape(-1) if torch.is_tensor(loaded)
+                                    else torch.zeros(n, dtype=torch.float32, device=device))
+                            arena.write(j, flat, start)
+                    else:
+                        o = (prm.data_ptr() - pb["param"].data_ptr()) // 4
+                        for name, key in zip(names, ("state1", "state2", "state3")):
+                            if key not in pb:
+                                continue
+                            view = pb[key][o:o + n].view(prm.shape)
+                            loaded = st.get(name)
+                            if torch.is_tensor(loaded):
+                                view.copy_(loaded)
+                                loaded_momentum = loaded_momentum or name == "momentum_buffer"
+                            else:
+                                view.zero_()
+                            st[name] = view
+                    if not sgd:
+                        if "step" in st:
+                            steps.add(int(float(st["step"])))
+                        self._bound_steps[id(st)] = st
+        if len(steps) > 1:
+            raise ValueError(f"parameters at different step counts {sorted(steps)}: one fused launch cannot mirror that")
+        if sgd:
+            self._momentum_ready = loaded_momentum
+        else:
+            self.step_count = steps.pop() if steps else 0
+            for st in self._bound_steps.values():
+                st["step"] = self.step_count
+        self._refresh_hyperparameters()
+        self._args_cache.clear()
+        self._native_args.clear()
+        torch.cuda.synchronize(device)
 
     _MOMENT_NAMES = ("exp_avg", "exp_avg_sq", "max_exp_avg_sq")
 

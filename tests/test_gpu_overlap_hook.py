@@ -617,3 +617,75 @@ def test_statistics_rows_keep_alternating_when_a_bucket_moves_to_the_native_meet
         if step >= 2:
             assert handed[step].row.data_ptr() == handed[step - 2].row.data_ptr()
             assert handed[step].row.data_ptr() != handed[step - 1].row.data_ptr()
+
+
+@pytest.mark.parametrize("kind,interleave", [("sgd", False), ("adamw", False), ("adamw", True), ("adamw_amsgrad", True)])
+def test_optimizer_load_state_dict_after_the_buckets_are_bound(gpu, kind, interleave):
+    """``optimizer.load_state_dict`` replaces the tensors in ``optimizer.state``; the launches read the arenas.
+    Two steps, a checkpoint (weights + ``optimizer.state_dict()``), two more steps, then the checkpoint is loaded
+    back and steps 3 and 4 are taken again: weights and state must be the oracle's after four steps, bit for bit
+    (a launch that kept using what its arenas held would apply steps 5 and 6 to them)."""
+    import copy
+    from jabas_amd import ddp_comm_hooks as H
+    from jabas_amd.local_sync import LocalBucketSync
+    from jabas_amd.train import create_optimizer_hook
+    K, batches, shapes = 2, (6, 2), SHAPES[:2]
+    opt = _opt_dict(kind)
+    gen = torch.Generator().manual_seed(11)
+    init = [[torch.randn(s, generator=gen) * 0.05 for s in bucket] for bucket in shapes]
+    replicas = [[[torch.nn.Parameter(t.clone().to(gpu)) for t in bucket] for bucket in init] for _ in range(K)]
+    layouts = [_layout(bucket) for bucket in shapes]
+    bufs = [[torch.zeros(n, device=gpu) for _ in range(K)] for (_, _, n) in layouts]
+    optimizer = _torch_optimizer(kind, [p for bucket in replicas[0] for p in bucket])
+    local = LocalBucketSync(batches, interleave_moments=interleave)
+    st = H.IIDPState(None, 2).attach_local(local)
+    main_hook = create_optimizer_hook(H.iidp_allreduce_hook, optimizer)
+    host = {step: [[torch.randn(n, generator=torch.Generator().manual_seed(31 * step + 7 * b + k)) * 1e-3
+                    for k in range(K)] for b, (_, _, n) in enumerate(layouts)] for step in range(1, 5)}
+
+    def take(step):
+        for b in range(len(shapes)):
+            for k in range(K):
+                bufs[b][k].copy_(host[step][b][k])
+                bucket = ParamBucket(b, bufs[b][k], replicas[k][b], layouts[b][0])
+                (main_hook(st, bucket) if k == 0 else H.dummy_hook(H.VSWPeerState(local, k), bucket)).wait()
+        local.finish_step()
+
+    take(1)
+    take(2)
+    torch.cuda.synchronize()
+    saved_w = [[p.detach().clone() for p in bucket] for bucket in replicas[0]]
+    saved_o = copy.deepcopy(optimizer.state_dict())
+    take(3)
+    take(4)
+    torch.cuda.synchronize()
+    with torch.no_grad():
+        for model in replicas:
+            for bucket, saved in zip(model, saved_w):
+                for p, w in zip(bucket, saved):
+                    p.copy_(w)                                                  # in place: the views stay
+    optimizer.load_state_dict(saved_o)
+    assert kind == "sgd" or local.step_count == 2            # Adam's t follows the checkpoint; SGD keeps no count
+    take(3)
+    take(4)
+    torch.cuda.synchronize()
+    seen = _checkpointed(optimizer)
+    for b, (offs, bounds, n) in enumerate(layouts):
+        p_h = torch.cat([t.reshape(-1) for t in init[b]])
+        s1_h, s2_h = torch.zeros_like(p_h), torch.zeros_like(p_h)
+        s3_h = torch.zeros_like(p_h) if kind.endswith("amsgrad") else None
+        for step in range(1, 5):
+            O.sync_step(host[step][b], batches, [(0, n, bounds)], opt, p_h, s1_h, s2_h, step=step,
+                        first_step=(step == 1), want_stats=False, state3=s3_h)
+        for i, (p, o) in enumerate(zip(replicas[0][b], offs)):
+            sl = slice(o, o + p.numel())
+            assert _same(p.data, p_h[sl]), (b, i, "weights")
+            assert _same(replicas[1][b][i].data, p.data), (b, i, "replica")
+            state = seen[id(p)]
+            if kind == "sgd":
+                assert _same(state["momentum_buffer"], s1_h[sl]), (b, i, "momentum")
+            else:
+                assert int(state["step"]) == 4
+                assert _same(state["exp_avg"], s1_h[sl]) and _same(state["exp_avg_sq"], s2_h[sl]), (b, i, "moments")
+                if s3_h is not None:
+                    assert _same(state["max_exp_avg_sq"], s3_h[sl]), (b, i, "maximum")
