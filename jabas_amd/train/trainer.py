@@ -269,6 +269,16 @@ class VSWSyncTrainer:
             self._bind_model(k, m, copy_weights=True)
         if optimizer is not None:
             self._expose_state(optimizer, moments=self.engine.state_is_live)
+            if hasattr(optimizer, "register_load_state_dict_post_hook"):
+                fresh = not hasattr(optimizer, "_jabas_load_owner")
+                optimizer._jabas_load_owner = weakref.ref(self)        # the trainer whose arenas take a loaded state
+                if fresh:
+                    def adopt(opt):
+                        t = opt._jabas_load_owner()
+                        if t is not None and t.main_optimizer is opt:
+                            t._adopt_optimizer_state()
+
+                    optimizer.register_load_state_dict_post_hook(adopt)
         torch.cuda.synchronize(self.gpu)
 
     _MOMENT_KEYS = ("exp_avg", "exp_avg_sq", "max_exp_avg_sq")
@@ -321,6 +331,45 @@ class VSWSyncTrainer:
 
             optimizer.register_state_dict_pre_hook(before)
             optimizer.register_state_dict_post_hook(after)
+
+    _adoptions = 0
+
+    def _adopt_optimizer_state(self):
+        """After ``main_optimizer.load_state_dict``: the fresh tensors it put into ``optimizer.state`` are copied
+        into the arenas the fused launch reads (a parameter the checkpoint holds no state for starts from zeros,
+        as it would in torch), the step count follows the checkpoint's (Adam's own count; SGD keeps none, but a
+        stored momentum buffer means a step was taken) and the optimizer's dictionaries show the arenas again.
+        Runs as a hook on the optimizer, so loading a checkpoint into the caller's optimizer object is enough."""
+        eng = self.engine
+        if eng is None or self.main_optimizer is None:
+            return
+        self._adoptions += 1
+        torch.cuda.synchronize(self.gpu)
+        sgd = self.opt["kind"] == "sgd"
+        keys = (("momentum_buffer", 0),) if sgd else tuple((k, j) for j, k in enumerate(self._MOMENT_KEYS))
+        steps, has_momentum = set(), False
+        for i, p in enumerate(self.main_model.parameters()):
+            st = self.main_optimizer.state.get(p, {})
+            for key, j in keys:
+                if j >= eng.n_state:
+                    continue
+                loaded = st.get(key)
+                if torch.is_tensor(loaded):
+                    eng.set_state(j, loaded.to(self.gpu), start=eng.layout.param_offset[i])
+                    has_momentum = has_momentum or key == "momentum_buffer"
+                else:
+                    eng.set_state(j, torch.zeros(p.numel(), dtype=torch.float32, device=self.gpu),
+                                  start=eng.layout.param_offset[i])
+            if "step" in st:
+                steps.add(int(float(st["step"])))
+        if len(steps) > 1:
+            raise ValueError(f"parameters at different step counts {sorted(steps)}: one fused launch cannot mirror that")
+        eng.step_count = steps.pop() if steps else (1 if has_momentum else 0)
+        self.opt["groups"] = [dict(lr=float(g["lr"]), weight_decay=float(g.get("weight_decay", 0.0)))
+                              for g in self.main_optimizer.param_groups]
+        self._step_tensor = torch.full((), float(eng.step_count), dtype=torch.float32)
+        self._expose_state(self.main_optimizer, moments=eng.state_is_live)
+        torch.cuda.synchronize(self.gpu)
 
     def _refresh_hyperparameters(self):
         """Learning rate and weight decay as the caller's optimizer object holds them now."""
@@ -421,26 +470,14 @@ class VSWSyncTrainer:
             if self.main_optimizer is None:
                 raise ValueError("the checkpoint holds a torch optimizer's state; hand the optimizer over through "
                                  "prepare_weight_sync_method first")
+            adopted = self._adoptions
             self.main_optimizer.load_state_dict(state["optimizer"])     # fresh tensors in optimizer.state ...
-            steps, has_momentum = set(), False
-            for i, p in enumerate(self.main_model.parameters()):        # ... copied into the arenas
-                st = self.main_optimizer.state.get(p, {})
-                for key, j in (("momentum_buffer", 0), ("exp_avg", 0), ("exp_avg_sq", 1), ("max_exp_avg_sq", 2)):
-                    if j < eng.n_state and st.get(key) is not None:
-                        eng.set_state(j, st[key].to(self.gpu), start=eng.layout.param_offset[i])
-                        has_momentum = has_momentum or key == "momentum_buffer"
-                if "step" in st:
-                    steps.add(int(float(st["step"])))
-            if len(steps) > 1:
-                raise ValueError(f"parameters at different step counts {sorted(steps)}: one fused launch cannot mirror that")
-            if "engine_step" in state:
+            if self._adoptions == adopted:                              # ... copied into the arenas (by the hook on
+                self._adopt_optimizer_state()                           # the optimizer where torch has such hooks)
+            if "engine_step" in state and int(state["engine_step"]) != eng.step_count:
                 eng.step_count = int(state["engine_step"])
-            else:       # a plain torch checkpoint: Adam's own count; SGD keeps none, but a stored momentum buffer means a step was taken
-                eng.step_count = steps.pop() if steps else (1 if has_momentum else 0)
-            self.opt["groups"] = [dict(lr=float(g["lr"]), weight_decay=float(g.get("weight_decay", 0.0)))
-                                  for g in self.main_optimizer.param_groups]
-            self._step_tensor = torch.full((), float(eng.step_count), dtype=torch.float32)
-            self._expose_state(self.main_optimizer, moments=eng.state_is_live)
+                self._step_tensor = torch.full((), float(eng.step_count), dtype=torch.float32)
+                self._expose_state(self.main_optimizer, moments=eng.state_is_live)
         elif "optimizer_arenas" in state:
             arenas = state["optimizer_arenas"]
             if arenas["numel"] != eng.layout.total:

@@ -627,6 +627,27 @@ def test_trainer_resumes_bit_for_bit_from_its_checkpoint(gpu, kind, interleave, 
         for key in keys:
             assert torch.equal(_states(opt_c)[id(pc)][key], seen_b[id(pb)][key])
 
+    # loading into the caller's own optimizer object is enough: the loaded tensors reach the arenas (a hook on the
+    # optimizer), so with the weights put back a run continues as the one that was saved did
+    d, opt_d = make(21, 3)
+    run(d, 1, 5)                                          # somewhere else: its state must be replaced, not kept
+    saved = torch.load(path, map_location=gpu, weights_only=True)
+    with torch.no_grad():
+        for m in d.local_models:
+            m.load_state_dict(saved["model"])
+    opt_d.load_state_dict(saved["optimizer"])
+    assert d.engine.step_count == (1 if kind == "sgd" else 3)
+    d.sync_step, d.similarity_state.step = saved["sync_step"], saved["similarity_step"]
+    for sch, sd in zip(d.local_schedulers, saved["schedulers"]):
+        sch.load_state_dict(sd)
+    run(d, 4, 6)
+    for pa, pd in zip(a.main_model.parameters(), d.main_model.parameters()):
+        assert torch.equal(pa.detach().view(torch.int32), pd.detach().view(torch.int32))
+    seen_d = _states(opt_d)
+    for pa, pd in zip(a.main_model.parameters(), d.main_model.parameters()):
+        for key in keys:
+            assert torch.equal(seen_a[id(pa)][key], seen_d[id(pd)][key])
+
 
 def test_trainer_with_bf16_gradient_buckets(gpu):
     """Reduced-precision buckets (the ViT-L/16 configuration): every VSW's gradient is rounded to bf16
