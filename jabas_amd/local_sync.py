@@ -451,9 +451,8 @@ class LocalBucketSync:
     def _refresh_hyperparameters(self):
         if self.optimizer is None:
             return
-        for mine, theirs in zip(self.opt["groups"], self.optimizer.param_groups):
-            mine["lr"] = float(theirs["lr"])
-            mine["weight_decay"] = float(theirs.get("weight_decay", 0.0))
+        from .train.trainer import refresh_opt_from_torch_optimizer
+        refresh_opt_from_torch_optimizer(self.opt, self.optimizer)
 
     def _bind_bucket(self, bucket_index, slot):
         """Arenas for the weights and optimizer state of one bucket's parameters, laid out like the

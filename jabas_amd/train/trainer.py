@@ -152,6 +152,38 @@ def opt_from_torch_optimizer(optimizer):
     return opt
 
 
+def refresh_opt_from_torch_optimizer(opt, optimizer):
+    """Brings the hyperparameter dictionary ``opt`` (made by ``opt_from_torch_optimizer``) up to what the optimizer
+    object's ``param_groups`` hold now: learning rate and weight decay per group, and the values a launch takes
+    once (momentum / dampening / nesterov, betas / eps), which schedulers that cycle the momentum move from step
+    to step. Groups that have come to differ in one of the latter, and a momentum that appears or disappears (the
+    momentum buffer exists or it does not), are errors."""
+    groups = optimizer.param_groups
+    for mine, theirs in zip(opt["groups"], groups):
+        mine["lr"] = float(theirs["lr"])
+        mine["weight_decay"] = float(theirs.get("weight_decay", 0.0))
+    g0 = groups[0]
+    keys = ("momentum", "dampening", "nesterov") if opt["kind"] == "sgd" else ("betas", "eps")
+    for key in keys:
+        if key not in g0:
+            continue
+        for g in groups[1:]:
+            if g[key] != g0[key]:
+                raise ValueError(f"parameter groups differ in {key!r}: one value per launch is supported")
+    if opt["kind"] == "sgd":
+        momentum = float(g0.get("momentum", opt.get("momentum", 0.0)))
+        if (momentum != 0.0) != (opt.get("momentum", 0.0) != 0.0):
+            raise ValueError("the momentum became zero or non-zero after the state arenas were laid out")
+        opt["momentum"] = momentum
+        opt["dampening"] = float(g0.get("dampening", opt.get("dampening", 0.0)))
+        opt["nesterov"] = bool(g0.get("nesterov", opt.get("nesterov", False)))
+    else:
+        if "betas" in g0:
+            opt["betas"] = (float(g0["betas"][0]), float(g0["betas"][1]))
+        if "eps" in g0:
+            opt["eps"] = float(g0["eps"])
+
+
 class VSWSyncTrainer:
     def __init__(self, gpu, local_batch_sizes, opt=None, interval=100, grad_dtype=torch.float32,
                  param_groups_func=None, similarity_target=None, controller=None, clip_norm=None,
@@ -372,12 +404,9 @@ class VSWSyncTrainer:
         torch.cuda.synchronize(self.gpu)
 
     def _refresh_hyperparameters(self):
-        """Learning rate and weight decay as the caller's optimizer object holds them now."""
-        if self.main_optimizer is None:
-            return
-        for mine, theirs in zip(self.opt["groups"], self.main_optimizer.param_groups):
-            mine["lr"] = float(theirs["lr"])
-            mine["weight_decay"] = float(theirs.get("weight_decay", 0.0))
+        """The hyperparameters as the caller's optimizer object holds them now."""
+        if self.main_optimizer is not None:
+            refresh_opt_from_torch_optimizer(self.opt, self.main_optimizer)
 
     def _bind_model(self, k, m, copy_weights):
         """Points replica k's parameters and gradients at its arenas."""

@@ -489,6 +489,60 @@ def test_trainer_takes_the_callers_optimizer_and_scheduler(gpu, kind):
             assert _close(seen[id(p)]["max_exp_avg_sq"], ref_opt.state[rp]["max_exp_avg_sq"], 1e-6, 1e-12)
 
 
+@pytest.mark.parametrize("kind", ["sgd", "adamw"])
+def test_trainer_follows_a_scheduler_that_cycles_the_momentum(gpu, kind):
+    """torch's OneCycleLR moves the momentum (SGD) or beta1 (Adam kinds) of every group along with the learning
+    rate: the launch takes them from the optimizer object at every step, like the learning rate."""
+    from jabas_amd.train import VSWSyncTrainer
+    batches = (5, 3)
+    crit = torch.nn.MSELoss()
+    trainer = VSWSyncTrainer(gpu, batches, interval=100)
+    trainer.prepare_stream_parallel(_mlp(12), crit)
+    ref_model = _mlp(12).to(gpu)
+
+    def build(model):
+        if kind == "sgd":
+            return torch.optim.SGD(_groups(model), lr=0.05, momentum=0.9, foreach=False)
+        return torch.optim.AdamW(_groups(model), lr=1e-3, foreach=False)
+
+    def cycle(o):
+        return torch.optim.lr_scheduler.OneCycleLR(o, max_lr=0.08 if kind == "sgd" else 4e-3, total_steps=8,
+                                                   base_momentum=0.6, max_momentum=0.95)
+
+    mine, ref_opt = build(trainer.main_model), build(ref_model)
+    sched, ref_sched = cycle(mine), cycle(ref_opt)
+    trainer.prepare_weight_sync_method(mine, sched, _groups)
+    w, _, _ = O.batch_weights(batches)
+    seen = set()
+    for step in range(1, 7):
+        gen = torch.Generator().manual_seed(170 + step)
+        data = [(torch.randn(b, 37, generator=gen).to(gpu), torch.randn(b, 10, generator=gen).to(gpu)) for b in batches]
+        trainer.compute(data)
+        per_vsw = []
+        for x, y in data:
+            ref_model.zero_grad(set_to_none=True)
+            crit(ref_model(x), y).backward()
+            per_vsw.append([p.grad.detach().clone() for p in ref_model.parameters()])
+        for i, p in enumerate(ref_model.parameters()):
+            p.grad = torch.add(torch.mul(per_vsw[0][i], w[0]), torch.mul(per_vsw[1][i], w[1]))
+        seen.add(mine.param_groups[0]["momentum"] if kind == "sgd" else mine.param_groups[0]["betas"][0])
+        ref_opt.step()
+        ref_sched.step()
+        trainer.step()
+        torch.cuda.synchronize()
+        for p, rp in zip(trainer.main_model.parameters(), ref_model.parameters()):
+            assert _close(p, rp, 1e-6, 1e-7), f"{kind} step {step}"
+    assert len(seen) >= 5                                   # the momentum did move
+    # groups that come to differ in it cannot share a launch
+    if kind == "sgd":
+        mine.param_groups[1]["momentum"] = 0.5
+    else:
+        mine.param_groups[1]["betas"] = (0.5, 0.999)
+    trainer.compute(data)
+    with pytest.raises(ValueError, match="parameter groups differ"):
+        trainer.step()
+
+
 def test_trainer_rejects_optimizers_it_cannot_mirror(gpu):
     from jabas_amd.train import VSWSyncTrainer
     trainer = VSWSyncTrainer(gpu, (2, 2))
