@@ -13,10 +13,11 @@ LIB_PATH = os.environ.get("JABAS_SYNC_LIB") or os.path.join(_HERE, "csrc", "libj
 
 MAX_K = 16
 MAX_GROUPS = 16
-STATS_STRIDE = 20
+STATS_STRIDE = 40
 GRAM_MAX_K = 16
 GRAM_STRIDE = 256
-STATS_GRAM_MAX_K = 4
+STATS_GRAM_MAX_K = 4            # fp32 gradients
+STATS_GRAM_MAX_K_BF16 = 8       # bf16 gradients
 STATIC_MAX_NUMEL = 1 << 26
 STEP_SCALARS_BYTES = 688
 

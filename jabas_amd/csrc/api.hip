@@ -248,7 +248,7 @@ int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
     const int oc = opt_class_of(s->opt_kind);
     if (oc < 0) return JABAS_ERR_OPT;
     if (s->stats < JABAS_STATS_NONE || s->stats > JABAS_STATS_GRAM) return JABAS_ERR_OPT;
-    if (s->stats == JABAS_STATS_GRAM && s->K > JABAS_STATS_GRAM_MAX_K) return JABAS_ERR_K;
+    if (s->stats == JABAS_STATS_GRAM && s->K > stats_gram_max_k(s->grad_dtype)) return JABAS_ERR_K;
     memset(a, 0, sizeof(*a));
     uint32_t mask = 0;
     for (int k = 0; k < s->K; ++k) {
@@ -388,14 +388,15 @@ hipError_t launch_finalize(dim3 grid, hipStream_t stream, const KArgs& a, uint32
     return launch_kernel(finalize_stats_kernel<NS>, grid, dim3(kFinalizeBlock), 0, stream, a.chunk_prefix, a.n_chunks,
                          a.use_inline, stripes, in_stripes, out_stride, in, out);
 }
-// One instantiation per row width: 4 (similarity sums), 4 + K, K = 1..16, and 4 + K + K(K-1)/2 for K <= 4
-// (7, 10, 14: among the widths of the full rows).
+// One instantiation per row width: 4 (similarity sums), 4 + K, K = 1..16, and 4 + K + K(K-1)/2 for K <= 8
+// (7, 10, 14, 19: among the widths of the full rows; 25, 32, 40).
 hipError_t finalize(int ns, dim3 grid, hipStream_t stream, const KArgs& a, uint32_t stripes, uint32_t in_stripes,
                     uint32_t out_stride, const double* in, double* out) {
     switch (ns) {
 #define JABAS_FIN(n) case n: return launch_finalize<n>(grid, stream, a, stripes, in_stripes, out_stride, in, out);
         JABAS_FIN(4) JABAS_FIN(5) JABAS_FIN(6) JABAS_FIN(7) JABAS_FIN(8) JABAS_FIN(9) JABAS_FIN(10) JABAS_FIN(11) JABAS_FIN(12)
-        JABAS_FIN(13) JABAS_FIN(14) JABAS_FIN(15) JABAS_FIN(16) JABAS_FIN(17) JABAS_FIN(18) JABAS_FIN(19) JABAS_FIN(20)
+        JABAS_FIN(13) JABAS_FIN(14) JABAS_FIN(15) JABAS_FIN(16) JABAS_FIN(17) JABAS_FIN(18) JABAS_FIN(19) JABAS_FIN(20) JABAS_FIN(25)
+        JABAS_FIN(32) JABAS_FIN(40)
 #undef JABAS_FIN
         default: return hipErrorInvalidValue;
     }
@@ -426,7 +427,9 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
         if (!stats_out) return JABAS_ERR_NULL;
         if (a.n_span > kMaxStatsSpans) return JABAS_ERR_SIZE;     // before anything is launched: no half-done step
         if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 8) return JABAS_ERR_WORKSPACE;
-        if (workspace_bytes < workspace_rows(a.n_chunks, a.n_span) * kStatsStride * sizeof(double)) return JABAS_ERR_WORKSPACE;
+        // one compact partial row per chunk and per (span, stripe), as wide as the level's rows are
+        if (workspace_bytes < workspace_rows(a.n_chunks, a.n_span) * stats_row_width(s->K, stats) * sizeof(double))
+            return JABAS_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(stats_out) % 8) return JABAS_ERR_ALIGN;
     }
     a.partials = static_cast<double*>(workspace);
@@ -745,9 +748,10 @@ JABAS_API int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_
 namespace {
 constexpr uint64_t kStaticMaxNumel = JABAS_STATIC_MAX_NUMEL;
 constexpr uint64_t kStaticMinChunkElems = kMinStatsChunkElems;    // one partial row per chunk of a statistics launch
+constexpr int kStaticRowDoubles = 4 + JABAS_MAX_K;            // the widest rows it serves: full rows of 16 VSWs
 constexpr size_t kStaticScratchBytes =
     workspace_rows((kStaticMaxNumel + kWideElems - 1 + kStaticMinChunkElems - 1) / kStaticMinChunkElems, 1) *
-    kStatsStride * sizeof(double);
+    kStaticRowDoubles * sizeof(double);
 static_assert(kStaticScratchBytes <= (6u << 20), "static scratch stays modest");
 constexpr int kMaxDevices = 64;
 }  // namespace
@@ -776,6 +780,9 @@ JABAS_API int jabas_sync_bucket_static(const JabasSpan* span, const JabasBound* 
     if (span->numel > kStaticMaxNumel) return JABAS_ERR_SIZE;
     void* ws = nullptr;
     if (args->stats) {
+        if (args->K >= 1 && args->K <= JABAS_MAX_K && args->stats <= JABAS_STATS_GRAM &&
+            stats_row_width(args->K, args->stats) > kStaticRowDoubles)
+            return JABAS_ERR_SIZE;                    // pair products of more than four VSWs: rows wider than the array holds
         const int rc = static_scratch(&ws);
         if (rc != JABAS_OK) return rc;
     }

@@ -625,7 +625,7 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
     static_assert(!capped || !SL || flush_bytes < JABAS_STATS_LDS_BYTES, "the cap is what is left beside the table");
     constexpr unsigned idle = !capped ? 0u : SL ? JABAS_STATS_LDS_BYTES - flush_bytes : JABAS_IDLE_LDS_BYTES;
     const dim3 block(launch_block(K, DT, OPT, SL));
-    if constexpr (SL == JABAS_STATS_GRAM && K > JABAS_STATS_GRAM_MAX_K) {
+    if constexpr (SL == JABAS_STATS_GRAM && K > stats_gram_max_k(DT)) {
         return static_cast<int>(hipErrorInvalidValue);              // refused by the front before it gets here
     } else {
         if constexpr (OPT == OPT_SGD || OPT == OPT_ADAM) {

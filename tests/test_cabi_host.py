@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_the_header():
     # sizes a C compiler gives the header's structs on x86-64 / amdgcn host ABI
     K = L.MAX_K
-    assert K == 16 and L.STATS_STRIDE == 4 + K
+    assert K == 16 and L.STATS_STRIDE == 40 >= max(4 + K, 4 + 8 + 28)     # full rows of 16 VSWs, pair products of 8
     assert C.sizeof(L.JabasSpan) == K * 8 + 5 * 8 + (K - 1) * 8 + 8 + 6 * 4
     assert C.sizeof(L.JabasBound) == 16
     assert C.sizeof(L.JabasGroup) == 24
@@ -231,6 +231,16 @@ def test_entry_points_validate_before_launching():
     many.K, many.grad_dtype, many.stats = L.STATS_GRAM_MAX_K + 1, L.F32, L.STATS_GRAM
     spk = _span(1000, K=L.STATS_GRAM_MAX_K + 1)
     assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
+    # bf16 gradients: up to STATS_GRAM_MAX_K_BF16 (the pair sums of a thread are fp32 there); the static entry point's
+    # array holds rows of up to 4 + 16 sums and refuses the wider ones
+    many.K, many.grad_dtype = L.STATS_GRAM_MAX_K_BF16 + 1, L.BF16
+    spk = _span(1000, K=L.STATS_GRAM_MAX_K_BF16 + 1, gs=2)
+    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
+    many.K = L.STATS_GRAM_MAX_K_BF16
+    spk = _span(1000, K=L.STATS_GRAM_MAX_K_BF16, gs=2)
+    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 8, None) == L.ERR_WORKSPACE
+    assert lib.jabas_sync_bucket_static(C.byref(spk), None, C.byref(many), 0x7f0400000000, None) == L.ERR_SIZE
+    assert L.STAT_NORM_VSW0 + 8 + 28 == L.STATS_STRIDE == L.stat_pair(8, 6, 7) + 1
     many.K, many.stats = 2, L.STATS_GRAM + 1
     assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_OPT
     hid = (C.c_uint8 * 2)(0, 1)

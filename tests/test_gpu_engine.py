@@ -112,12 +112,14 @@ def test_global_norm_clipping(gpu, opt, clip_norm, keep):
         assert norm == pytest.approx(clip_norm, rel=1e-4)
 
 
-@pytest.mark.parametrize("opt,dtype", [(SGD, torch.float32), (ADAM, torch.bfloat16)])
+@pytest.mark.parametrize("opt,dtype,batches", [(SGD, torch.float32, (4, 2, 1, 1)), (ADAM, torch.bfloat16, (4, 2, 1, 1)),
+                                               (ADAM, torch.bfloat16, (64, 56, 48, 40, 32, 24, 16, 8))])
 @pytest.mark.parametrize("clip", [None, 0.05])
-def test_engine_gram_rows_out_of_the_step(gpu, opt, dtype, clip):
+def test_engine_gram_rows_out_of_the_step(gpu, opt, dtype, batches, clip):
     """stats="gram": the planned launch over every span leaves the pair products beside the full rows (with
-    clipping: the aggregate launch does), and the step itself stays what it is without them."""
-    batches = (4, 2, 1, 1)
+    clipping: the aggregate launch does), and the step itself stays what it is without them. Four workers, and
+    the eight bf16 ones of the largest configuration."""
+    K = len(batches)
     eng, host, spans = _make(gpu, batches, opt, dtype, per_tensor_spans=True)
     plain, host2, _ = _make(gpu, batches, opt, dtype, per_tensor_spans=True)
     for step in (1, 2):
@@ -128,13 +130,13 @@ def test_engine_gram_rows_out_of_the_step(gpu, opt, dtype, clip):
         plain.step(stats=False, clip_norm=clip)
         torch.cuda.synchronize()
         assert rows.shape == (len(spans), L.STATS_STRIDE)
-        assert torch.count_nonzero(rows[:, 4 + 4 + 6:]) == 0
+        assert torch.count_nonzero(rows[:, 4 + K + K * (K - 1) // 2:]) == 0
         want = O.gram([torch.cat([g[o:o + n] for o, n, _ in spans]) for g in host["g"]])
         scale = torch.sqrt(torch.outer(torch.diagonal(want), torch.diagonal(want)))
         tol = 1e-11 if dtype == torch.float32 else 1e-5
         assert bool(((eng.gram(rows).cpu() - want).abs() <= tol * scale).all())
         rows_h = torch.stack([O.stats([g[o:o + n] for g in host["g"]], batches) for o, n, _ in spans])
-        assert _close(rows[:, 1:8], rows_h[:, 1:8], tol, 1e-30)
+        assert _close(rows[:, 1:4 + K], rows_h[:, 1:4 + K], tol, 1e-30)
         assert torch.equal(eng.param.view(torch.int32), plain.param.view(torch.int32))
         assert torch.equal(eng.state1.view(torch.int32), plain.state1.view(torch.int32))
 

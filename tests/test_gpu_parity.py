@@ -155,14 +155,15 @@ def test_similarity_level_rows(gpu, K, dtype, rtol):
         assert torch.equal(_bits(m_d), _bits(m_h)) and torch.equal(_bits(v_d), _bits(v_h))
 
 
-@pytest.mark.parametrize("K", [1, 2, 3, 4])
-@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-11), (torch.bfloat16, 1e-5)])
+@pytest.mark.parametrize("K,dtype,rtol", [(K, torch.float32, 1e-11) for K in (1, 2, 3, 4)] +
+                         [(K, torch.bfloat16, 1e-5) for K in (1, 2, 3, 4, 5, 6, 7, 8)])
 @pytest.mark.parametrize("opt", [None, SGD, ADAMW], ids=["aggregate", "sgd", "adamw"])
 def test_gram_level_rows(gpu, K, dtype, rtol, opt):
     """Statistics level 3: the full row plus the product of every pair of workers, out of the launch that
-    aggregates and steps. Row against the float64 oracle (the four sums and the norms as at the full level,
-    the pair slots against the Gram matrix), pair order as the header's JABAS_STAT_PAIR, slots beyond the row
-    zero, and the aggregate and the optimizer step of the same launch bit-exact."""
+    aggregates and steps (up to four workers with fp32 gradients, eight with bf16 ones). Row against the float64
+    oracle (the four sums and the norms as at the full level, the pair slots against the Gram matrix), pair order
+    as the header's JABAS_STAT_PAIR, slots beyond the row zero, and the aggregate and the optimizer step of the
+    same launch bit-exact."""
     from jabas_amd import sync, _lib as L
     for n, skew in ((5, 0), (4099, 1), (300007, 0), (1 << 21, 2), (4099, 45)):
         print(f"gram level K={K} {dtype} n={n} skew={skew}", flush=True)
@@ -220,7 +221,23 @@ def test_gram_level_limits_and_the_separate_pass(gpu):
     assert e.value.status == L.ERR_K
     assert torch.equal(out, before)
     with pytest.raises(ValueError):
-        sync.gram_from_stats(torch.zeros(L.STATS_STRIDE, dtype=torch.float64), 5)
+        sync.gram_from_stats(torch.zeros(L.STATS_STRIDE, dtype=torch.float64), 9)
+    # bf16 gradients: eight workers at most; the entry point that allocates nothing stops at four (its array holds
+    # rows of 4 + 16 sums)
+    hb = _host_grads(9, 70001, 98, std=5e-4, dtype=torch.bfloat16)
+    db = [_dev(t, gpu, 3) for t in hb]
+    outb = _dev(torch.zeros(70001), gpu, 3)
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.sync_bucket(sync.SpanSpec(db, agg_out=outb), sync.make_step_args(BATCHES[9], torch.bfloat16, stats="gram"))
+    assert e.value.status == L.ERR_K and torch.count_nonzero(outb) == 0
+    with pytest.raises(L.JabasSyncError) as e:
+        sync.sync_bucket_static(sync.SpanSpec(db[:8], agg_out=outb), sync.make_step_args(BATCHES[8], torch.bfloat16, stats="gram"),
+                                stats_out=torch.zeros(L.STATS_STRIDE, dtype=torch.float64, device=gpu))
+    assert e.value.status == L.ERR_SIZE and torch.count_nonzero(outb) == 0
+    rowb = sync.sync_bucket(sync.SpanSpec(db[:8], agg_out=outb), sync.make_step_args(BATCHES[8], torch.bfloat16, stats="gram"))
+    fusedb, apartb = sync.gram_from_stats(rowb, 8).cpu(), sync.gram(db[:8]).cpu()
+    scaleb = torch.sqrt(torch.outer(torch.diagonal(apartb), torch.diagonal(apartb)))
+    assert bool(((fusedb - apartb).abs() <= 2e-5 * scaleb).all())
     row = sync.sync_bucket(sync.SpanSpec(dg[:4], agg_out=out), sync.make_step_args(BATCHES[4], torch.float32, stats="gram"))
     fused = sync.gram_from_stats(row, 4).cpu()
     apart = sync.gram(dg[:4]).cpu()

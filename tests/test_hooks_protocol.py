@@ -274,8 +274,9 @@ def test_statistics_levels_and_their_names():
     with pytest.raises(ValueError):
         sync.stats_level("everything")
     assert LocalBucketSync([1] * 4, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM
-    with pytest.raises(ValueError, match="up to 4"):
-        LocalBucketSync([1] * 5, launcher=Recorder(), stats_level="gram")
+    assert LocalBucketSync([1] * 8, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM   # bf16 buckets
+    with pytest.raises(ValueError, match="up to 8"):
+        LocalBucketSync([1] * 9, launcher=Recorder(), stats_level="gram")
     row = torch.arange(L.STATS_STRIDE, dtype=torch.float64)
     G = sync.gram_from_stats(torch.stack([row, row]), 3)          # slots 4..6 the norms, 7, 8, 9 the pairs (0,1) (0,2) (1,2)
     assert G.tolist() == [[8.0, 14.0, 16.0], [14.0, 10.0, 18.0], [16.0, 18.0, 12.0]]
