@@ -459,7 +459,7 @@ int run_fused(KArgs& a, const JabasStepArgs* s, uint32_t max_span_chunks, double
 
 using namespace jabas;
 
-JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.5 (gfx950)"; }
+JABAS_API const char* jabas_sync_version(void) { return "jabas_sync 0.6 (gfx950)"; }
 
 JABAS_API const char* jabas_status_string(int status) {
     switch (status) {

@@ -54,7 +54,7 @@ def aggregate(grads, w):
 def stats(grads, w, half_id, hw):
     arr, bf16, keep = _grad_ptrs(grads)
     n, K = keep[0].numel(), len(keep)
-    row = torch.zeros(20, dtype=torch.float64)          # 4 + 16 slots, as the library's rows
+    row = torch.zeros(20, dtype=torch.float64)          # 4 + 16 slots: the oracle's own rows (four sums, one norm per worker)
     lib().oc_stats(arr, K, bf16, (C.c_float * K)(*[float(x) for x in w]), (C.c_uint8 * K)(*[int(x) for x in half_id]),
                    (C.c_float * K)(*[float(x) for x in hw]), C.c_size_t(n), C.c_void_p(row.data_ptr()))
     return row

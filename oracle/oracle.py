@@ -33,7 +33,7 @@ import math
 import numpy as np
 import torch
 
-STATS_STRIDE = 20
+STATS_STRIDE = 20          # the four sums and up to 16 per-worker norms (the library's rows are wider: pair products too)
 DOT_AB, NORM_A, NORM_B, NORM_AGG, NORM_VSW0 = 0, 1, 2, 3, 4
 
 
