@@ -381,7 +381,7 @@ def time_config(cfg, device, steps, warmup, torch, extras=True):
         res["step_without_statistics"] = rate(bytes_per_step, ms)
         ms, _ = timed_region(lambda i: engines[i % n].step(stats="full"), steps, warmup, torch)
         res["step_with_per_vsw_norms"] = rate(bytes_per_step, ms)
-        if cfg.K <= (8 if cfg.grad_dtype == "bf16" else 4):
+        if cfg.K <= 8:
             # the worker x worker Gram matrix ("between workers" statistics): out of the step's own launch (pair
             # products beside the full rows, no byte read twice), against the step followed by a pass of its
             # own over the K gradient arenas (K * gradient size more bytes per element read)

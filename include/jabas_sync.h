@@ -41,8 +41,7 @@ extern "C" {
 #define JABAS_MAX_GROUPS 16     /* optimizer parameter groups per launch              */
 #define JABAS_STATS_STRIDE 40   /* doubles per span in stats_out: the widest row, 4 + 8 + 28 (GRAM, 8 VSWs) */
 #define JABAS_GRAM_MAX_K 16     /* VSWs of one jabas_gram call                        */
-#define JABAS_STATS_GRAM_MAX_K 4 /* VSWs of a launch with JABAS_STATS_GRAM, fp32 gradients */
-#define JABAS_STATS_GRAM_MAX_K_BF16 8 /* ... with bf16 gradients                       */
+#define JABAS_STATS_GRAM_MAX_K 8 /* VSWs of a launch with JABAS_STATS_GRAM             */
 #define JABAS_GRAM_STRIDE 256   /* doubles per call in gram_out: JABAS_GRAM_MAX_K squared */
 #define JABAS_STATIC_MAX_NUMEL (1ull << 26)  /* largest span of jabas_sync_bucket_static  */
 #define JABAS_STEP_SCALARS_BYTES 688         /* size of a step-scalar block (jabas_step_scalars_encode) */
@@ -80,10 +79,9 @@ enum { JABAS_OPT_NONE = 0, JABAS_OPT_SGD = 1, JABAS_OPT_ADAM = 2, JABAS_OPT_ADAM
  * loads in flight. FULL adds sum g_k^2 of every VSW. GRAM adds, to the full row, the products
  * sum g_a*g_b of every pair of VSWs a < b, i.e. the whole worker x worker Gram matrix from the
  * pass that aggregates and updates, with no byte read a second time; K <= JABAS_STATS_GRAM_MAX_K
- * for fp32 gradients, K <= JABAS_STATS_GRAM_MAX_K_BF16 for bf16 gradients (JABAS_ERR_K beyond:
- * the K*(K-1)/2 extra sums per thread, fp64 for fp32 gradients and fp32 for bf16 ones, fit the
- * registers of the fused kernel up to there; more workers use jabas_gram, a pass of its own
- * over the gradients). */
+ * (JABAS_ERR_K beyond: the K*(K-1)/2 extra sums per thread, fp64 for fp32 gradients and fp32
+ * for bf16 ones, fit the registers of the fused kernel up to there; more workers use jabas_gram,
+ * a pass of its own over the gradients). */
 enum { JABAS_STATS_NONE = 0, JABAS_STATS_FULL = 1, JABAS_STATS_SIMILARITY = 2, JABAS_STATS_GRAM = 3 };
 
 /* Slots of one stats_out row (JABAS_STATS_STRIDE doubles per span). A = VSWs with
@@ -295,7 +293,7 @@ int jabas_sync_bucket(const JabasSpan* span, const JabasBound* bounds_dev,
  * Calls neither allocate nor free anything.
  * span->numel above JABAS_STATIC_MAX_NUMEL (64 Mi elements, a 256 MB fp32 bucket) is refused
  * with JABAS_ERR_SIZE before anything is launched, and so is JABAS_STATS_GRAM with more than
- * JABAS_STATS_GRAM_MAX_K VSWs (rows wider than the array is sized for). All calls on one GPU share that GPU's
+ * five VSWs (rows of more than 4 + JABAS_MAX_K sums, wider than the array is sized for). All calls on one GPU share that GPU's
  * array: calls with statistics that overlap in time on one GPU (different streams or
  * threads) race on it and must be serialised by the caller; calls without statistics do
  * not touch it. Results are those of jabas_sync_bucket, bit for bit. */

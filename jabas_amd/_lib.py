@@ -16,8 +16,7 @@ MAX_GROUPS = 16
 STATS_STRIDE = 40
 GRAM_MAX_K = 16
 GRAM_STRIDE = 256
-STATS_GRAM_MAX_K = 4            # fp32 gradients
-STATS_GRAM_MAX_K_BF16 = 8       # bf16 gradients
+STATS_GRAM_MAX_K = 8
 STATIC_MAX_NUMEL = 1 << 26
 STEP_SCALARS_BYTES = 688
 

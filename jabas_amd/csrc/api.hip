@@ -248,7 +248,7 @@ int fill_step_scal(const JabasStepArgs* s, StepScal* a) {
     const int oc = opt_class_of(s->opt_kind);
     if (oc < 0) return JABAS_ERR_OPT;
     if (s->stats < JABAS_STATS_NONE || s->stats > JABAS_STATS_GRAM) return JABAS_ERR_OPT;
-    if (s->stats == JABAS_STATS_GRAM && s->K > stats_gram_max_k(s->grad_dtype)) return JABAS_ERR_K;
+    if (s->stats == JABAS_STATS_GRAM && s->K > JABAS_STATS_GRAM_MAX_K) return JABAS_ERR_K;
     memset(a, 0, sizeof(*a));
     uint32_t mask = 0;
     for (int k = 0; k < s->K; ++k) {
@@ -782,7 +782,7 @@ JABAS_API int jabas_sync_bucket_static(const JabasSpan* span, const JabasBound* 
     if (args->stats) {
         if (args->K >= 1 && args->K <= JABAS_MAX_K && args->stats <= JABAS_STATS_GRAM &&
             stats_row_width(args->K, args->stats) > kStaticRowDoubles)
-            return JABAS_ERR_SIZE;                    // pair products of more than four VSWs: rows wider than the array holds
+            return JABAS_ERR_SIZE;                    // pair products of more than five VSWs: rows wider than the array holds
         const int rc = static_scratch(&ws);
         if (rc != JABAS_OK) return rc;
     }

@@ -477,20 +477,25 @@ __device__ __forceinline__ void run_chunk(const SP& sp, uint32_t lt0, uint32_t l
 // instructions per value, which matters because a workgroup only covers a few thousand elements.
 //   stage 1  thread (v, part) adds entries part, part+16, ..., part+240 of value v (in order);
 //   stage 2  the 16 parts of a value sit in one 16-lane row: DPP row reduction.
+// BS / 16 values go through the table at a time (16 with 256 threads), so rows wider than that take several
+// passes over a table of 32 KB instead of one of up to 80 (pair products of eight workers: 40 values).
 // The order is fixed, so the row is bit-identical from run to run.
 template <int NS, int BS>
 __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
     constexpr int kParts = 16;                       // lanes of one DPP row
-    constexpr int kPerPass = BS / kParts;            // values reduced per pass (16 with 256 threads)
-    __shared__ double buf[NS][BS];
+    constexpr int kPerPass = BS / kParts;            // values reduced per pass
+    constexpr int kBuf = NS < kPerPass ? NS : kPerPass;
+    __shared__ double buf[kBuf][BS];
     const int tid = threadIdx.x;
 #pragma unroll
-    for (int i = 0; i < NS; ++i) buf[i][tid] = acc[i];
-    __syncthreads();
+    for (int v0 = 0; v0 < NS; v0 += kPerPass) {
+        if (v0) __syncthreads();                     // the table is read out before it is filled again
 #pragma unroll
-    for (int v0 = 0; v0 < NS; v0 += kPerPass) {      // K > 12 needs a second pass at 256 threads
-        if (tid < (NS - v0) * kParts) {
-            const int v = v0 + (tid >> 4), part = tid & 15;
+        for (int i = 0; i < kPerPass; ++i)
+            if (v0 + i < NS) buf[i][tid] = acc[v0 + i];
+        __syncthreads();
+        if (tid < (NS - v0) * kParts) {              // at most kPerPass * 16 = BS threads
+            const int v = tid >> 4, part = tid & 15;
             double s = buf[v][part];
 #pragma unroll
             for (int i = 1; i < BS / kParts; ++i) s += buf[v][i * kParts + part];
@@ -498,7 +503,7 @@ __device__ __forceinline__ void flush_stats(double (&acc)[NS], double* row) {
             s += dpp_move<0x4E, 0xf>(s);     // quad_perm [2,3,0,1]
             s += dpp_move<0x141, 0xf>(s);    // row_half_mirror
             s += dpp_move<0x140, 0xf>(s);    // row_mirror
-            if (part == 0) row[v] = s;
+            if (part == 0) row[v0 + v] = s;
         }
     }
 }
@@ -621,11 +626,11 @@ int launch_one(const KArgs& a, unsigned grid, hipStream_t stream, bool dyn) {
 #define JABAS_STATS_LDS_BYTES 53248u      // per workgroup, flush_stats' own table included: three workgroups per CU
 #endif
     constexpr bool capped = OPT == OPT_ADAM && K <= 4 && DT == JABAS_F32;
-    constexpr unsigned flush_bytes = NStats<K, SL>::value * launch_block(K, DT, OPT, SL) * 8u;   // fp64 [value][thread]
+    constexpr unsigned flush_bytes = imin(NStats<K, SL>::value, launch_block(K, DT, OPT, SL) / 16) * launch_block(K, DT, OPT, SL) * 8u;   // flush_stats' fp64 table
     static_assert(!capped || !SL || flush_bytes < JABAS_STATS_LDS_BYTES, "the cap is what is left beside the table");
     constexpr unsigned idle = !capped ? 0u : SL ? JABAS_STATS_LDS_BYTES - flush_bytes : JABAS_IDLE_LDS_BYTES;
     const dim3 block(launch_block(K, DT, OPT, SL));
-    if constexpr (SL == JABAS_STATS_GRAM && K > stats_gram_max_k(DT)) {
+    if constexpr (SL == JABAS_STATS_GRAM && K > JABAS_STATS_GRAM_MAX_K) {
         return static_cast<int>(hipErrorInvalidValue);              // refused by the front before it gets here
     } else {
         if constexpr (OPT == OPT_SGD || OPT == OPT_ADAM) {

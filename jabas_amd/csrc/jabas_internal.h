@@ -99,12 +99,7 @@ constexpr int kMinChunkElems = imin(imin(kMinStatsChunkElems, 4 * JABAS_BLOCK_SG
                                     4 * imin(imin(JABAS_BLOCK * JABAS_CHUNK_TILES_PLAIN_LO, JABAS_BLOCK * JABAS_CHUNK_TILES_LO),
                                              imin(JABAS_BLOCK_MANYK * JABAS_CHUNK_TILES_MANYK, JABAS_BLOCK * JABAS_CHUNK_TILES_HI)));
 constexpr int kStatsStride = JABAS_STATS_STRIDE;
-// Most workers a launch with JABAS_STATS_GRAM serves: the pair sums are fp64 per thread for fp32 gradients and
-// fp32 for bf16 ones.
-__host__ __device__ constexpr int stats_gram_max_k(int grad_dtype) {
-    return grad_dtype == JABAS_BF16 ? JABAS_STATS_GRAM_MAX_K_BF16 : JABAS_STATS_GRAM_MAX_K;
-}
-static_assert(stats_row_width(JABAS_STATS_GRAM_MAX_K_BF16, JABAS_STATS_GRAM) <= JABAS_STATS_STRIDE &&
+static_assert(stats_row_width(JABAS_STATS_GRAM_MAX_K, JABAS_STATS_GRAM) <= JABAS_STATS_STRIDE &&
               stats_row_width(JABAS_MAX_K, JABAS_STATS_FULL) <= JABAS_STATS_STRIDE, "every row fits the stride");
 
 // Elements one thread handles per tile: one 16-byte fp32 vector of every fp32 buffer

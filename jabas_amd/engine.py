@@ -196,7 +196,7 @@ class VSWFlatSync:
     def step(self, stats=False, lr_scale=1.0, stream=None, clip_norm=None, accumulations=1):
         """One sync step over the whole gradient set. Returns the per-span stats tensor
         when ``stats`` is set (True / "full": rows of 4 + K sums; "similarity": the four sums of the halves
-        and of the aggregate, per-VSW slots zero; "gram", up to four VSWs (eight with bf16 gradients): the full row plus the product of
+        and of the aggregate, per-VSW slots zero; "gram", up to eight VSWs: the full row plus the product of
         every pair of VSWs' gradients, ``gram(rows)`` makes the matrix of them).
 
         Without ``clip_norm``: one fused launch. With it (global-norm clipping as

@@ -122,7 +122,7 @@ class LocalBucketSync:
         the halves and norm clipping read: all the reference's adaptive batching consumes,
         jabas/train/trainer.py:470-483), "full" (plus the squared norm of every VSW's gradient) or "gram" (plus
         the product of every pair of VSWs' gradients, the worker x worker Gram matrix, out of the same launch:
-        up to four VSWs with fp32 buckets, eight with bf16 ones; ``sync.gram_from_stats`` reads it from the rows).
+        up to eight VSWs; ``sync.gram_from_stats`` reads it from the rows).
 
         stream: the stream the fused launches are queued on (the reference's dedicated optimizer
         stream, jabas/train/trainer.py:328); default: the stream VSW 0's hooks run on.
@@ -191,8 +191,8 @@ class LocalBucketSync:
         self._plans = {}                       # batched mode: group of buckets -> its plan
         self._stream_cache = {}
         self.stats_level = sync.stats_level(stats_level) or L.STATS_SIMILARITY
-        if self.stats_level == L.STATS_GRAM and len(batches) > L.STATS_GRAM_MAX_K_BF16:
-            raise ValueError(f"statistics level 'gram' serves up to {L.STATS_GRAM_MAX_K_BF16} VSWs, not {len(batches)}: "
+        if self.stats_level == L.STATS_GRAM and len(batches) > L.STATS_GRAM_MAX_K:
+            raise ValueError(f"statistics level 'gram' serves up to {L.STATS_GRAM_MAX_K} VSWs, not {len(batches)}: "
                              f"use 'full' and sync.gram() over the gradient buffers")
         self._ready = {}                       # deferred / batched mode: bucket index -> complete _Slot not launched yet
         self._vsw_streams = {}                 # VSW index -> the stream its hooks ran on in this step

@@ -75,8 +75,8 @@ def stats_level(stats):
     """JABAS_STATS_* level of a launch: False / None / 0 none; True / 1 / 'full' the full row (4 + K sums);
     2 / 'similarity' the four sums of the halves and of the aggregate only (what the cosine similarity and
     global-norm clipping read; the per-VSW norm slots of the row are 0); 3 / 'gram' the full row plus the
-    products of every pair of workers (the Gram matrix out of the same pass; up to STATS_GRAM_MAX_K workers with
-    fp32 gradients, STATS_GRAM_MAX_K_BF16 with bf16 ones; read it with :func:`gram_from_stats`)."""
+    products of every pair of workers (the Gram matrix out of the same pass; up to STATS_GRAM_MAX_K workers;
+    read it with :func:`gram_from_stats`)."""
     if stats is None or stats is False or stats == 0:
         return L.STATS_NONE
     if stats is True or stats == 1 or stats == "full":
@@ -554,8 +554,8 @@ def gram_from_stats(stats_rows, K):
     """K x K Gram matrix (float64, on the rows' device) of the worker gradients from statistics rows of level
     'gram', summed over the rows (one row per span or bucket): the diagonal from the per-VSW norms, the rest
     from the pair slots. No launch of its own: the sums came out of the pass that aggregated the gradients."""
-    if not 1 <= K <= L.STATS_GRAM_MAX_K_BF16:
-        raise ValueError(f"rows of level 'gram' exist for 1..{L.STATS_GRAM_MAX_K_BF16} workers, not {K}")
+    if not 1 <= K <= L.STATS_GRAM_MAX_K:
+        raise ValueError(f"rows of level 'gram' exist for 1..{L.STATS_GRAM_MAX_K} workers, not {K}")
     total = stats_rows.detach().reshape(-1, L.STATS_STRIDE).to(torch.float64).sum(dim=0)
     out = torch.empty(K, K, dtype=torch.float64, device=total.device)
     for a in range(K):

@@ -226,20 +226,19 @@ def test_entry_points_validate_before_launching():
     sp.state3 = 0x7f0000000000 + 21 * (1 << 32)
     ams.scalars_dev = 0x7f0000000000 + 22 * (1 << 32)
     assert lib.jabas_sync_bucket(C.byref(sp), None, C.byref(ams), None, None, 0, None) == L.ERR_OPT
-    # statistics level 'gram' (pair products in the fused launch): up to STATS_GRAM_MAX_K workers; no level beyond it
+    # statistics level 'gram' (pair products in the fused launch): up to STATS_GRAM_MAX_K workers; no level beyond it;
+    # the static entry point's array holds rows of up to 4 + 16 sums and refuses the wider ones (six workers and more)
     many = L.JabasStepArgs()
-    many.K, many.grad_dtype, many.stats = L.STATS_GRAM_MAX_K + 1, L.F32, L.STATS_GRAM
-    spk = _span(1000, K=L.STATS_GRAM_MAX_K + 1)
-    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
-    # bf16 gradients: up to STATS_GRAM_MAX_K_BF16 (the pair sums of a thread are fp32 there); the static entry point's
-    # array holds rows of up to 4 + 16 sums and refuses the wider ones
-    many.K, many.grad_dtype = L.STATS_GRAM_MAX_K_BF16 + 1, L.BF16
-    spk = _span(1000, K=L.STATS_GRAM_MAX_K_BF16 + 1, gs=2)
-    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
-    many.K = L.STATS_GRAM_MAX_K_BF16
-    spk = _span(1000, K=L.STATS_GRAM_MAX_K_BF16, gs=2)
-    assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 8, None) == L.ERR_WORKSPACE
-    assert lib.jabas_sync_bucket_static(C.byref(spk), None, C.byref(many), 0x7f0400000000, None) == L.ERR_SIZE
+    for dt, gs in ((L.F32, 4), (L.BF16, 2)):
+        many.K, many.grad_dtype, many.stats = L.STATS_GRAM_MAX_K + 1, dt, L.STATS_GRAM
+        spk = _span(1000, K=L.STATS_GRAM_MAX_K + 1, gs=gs)
+        assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_K
+        many.K = L.STATS_GRAM_MAX_K
+        spk = _span(1000, K=L.STATS_GRAM_MAX_K, gs=gs)
+        assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 8, None) == L.ERR_WORKSPACE
+        assert lib.jabas_sync_bucket_static(C.byref(spk), None, C.byref(many), 0x7f0400000000, None) == L.ERR_SIZE
+        many.K = 6
+        assert lib.jabas_sync_bucket_static(C.byref(_span(1000, K=6, gs=gs)), None, C.byref(many), 0x7f0400000000, None) == L.ERR_SIZE
     assert L.STAT_NORM_VSW0 + 8 + 28 == L.STATS_STRIDE == L.stat_pair(8, 6, 7) + 1
     many.K, many.stats = 2, L.STATS_GRAM + 1
     assert lib.jabas_sync_bucket(C.byref(spk), None, C.byref(many), 0x7f0400000000, 0x7f0500000000, 1 << 20, None) == L.ERR_OPT

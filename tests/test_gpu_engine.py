@@ -113,7 +113,8 @@ def test_global_norm_clipping(gpu, opt, clip_norm, keep):
 
 
 @pytest.mark.parametrize("opt,dtype,batches", [(SGD, torch.float32, (4, 2, 1, 1)), (ADAM, torch.bfloat16, (4, 2, 1, 1)),
-                                               (ADAM, torch.bfloat16, (64, 56, 48, 40, 32, 24, 16, 8))])
+                                               (ADAM, torch.bfloat16, (64, 56, 48, 40, 32, 24, 16, 8)),
+                                               (ADAM, torch.float32, (7, 7, 5, 3, 2, 1))])
 @pytest.mark.parametrize("clip", [None, 0.05])
 def test_engine_gram_rows_out_of_the_step(gpu, opt, dtype, batches, clip):
     """stats="gram": the planned launch over every span leaves the pair products beside the full rows (with

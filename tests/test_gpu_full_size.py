@@ -177,7 +177,7 @@ def test_full_size_configuration(gpu, name):
     agg1 = a.agg.clone()
     r2 = a.step(stats=True).cpu().clone()
     assert torch.equal(r1.view(torch.int64), r2.view(torch.int64))       # same plan, same bits
-    if cfg.K <= (L.STATS_GRAM_MAX_K_BF16 if gdt == torch.bfloat16 else L.STATS_GRAM_MAX_K):
+    if cfg.K <= L.STATS_GRAM_MAX_K:
         # the worker x worker products out of the same launch: the row's other slots keep their bits; the pair sums
         # equal a float64 library reduction; and the sums of the halves and of the aggregate are the quadratic
         # forms of the Gram matrix in the weights (up to the fp32 rounding of the aggregated elements)

@@ -274,7 +274,7 @@ def test_statistics_levels_and_their_names():
     with pytest.raises(ValueError):
         sync.stats_level("everything")
     assert LocalBucketSync([1] * 4, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM
-    assert LocalBucketSync([1] * 8, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM   # bf16 buckets
+    assert LocalBucketSync([1] * 8, launcher=Recorder(), stats_level="gram").stats_level == L.STATS_GRAM
     with pytest.raises(ValueError, match="up to 8"):
         LocalBucketSync([1] * 9, launcher=Recorder(), stats_level="gram")
     row = torch.arange(L.STATS_STRIDE, dtype=torch.float64)
