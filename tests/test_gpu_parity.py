@@ -873,7 +873,9 @@ def test_random_plans_match_the_oracle(gpu, seed):
     hg_work = [t.clone() for t in hg]
     block = sync.StepScalars(gpu) if opt and seed % 2 else None
     for step in (1, 2, 3):
-        stats = step != 2
+        # full rows on the first step, none on the second; on the third the similarity sums or, up to eight
+        # workers, the full rows with the pair products
+        stats = (True, False, "gram" if K <= L.STATS_GRAM_MAX_K and seed % 3 else "similarity")[step - 1]
         args = sync.make_step_args(batches, dtype, stats=stats, opt=opt, step=step, first_step=(step == 1),
                                    half_id=half_id)
         if block is not None:
@@ -884,15 +886,27 @@ def test_random_plans_match_the_oracle(gpu, seed):
                                                     half_id=half_id, lr_scale=3.0))
         rows = plan.run(args)
         torch.cuda.synchronize()
+        hg_in = [t.clone() for t in hg_work]            # what this step's launch read (the in-place aggregate moves worker 0's)
         agg_h, rows_h = O.sync_step(hg_work, batches, spans_h, opt, p_h, s1_h, s2_h if adam else None, step=step,
-                                    first_step=(step == 1), want_stats=stats, half_id=half_id)
+                                    first_step=(step == 1), want_stats=bool(stats), half_id=half_id)
         for i, (o, s, _) in enumerate(spans_h):
             assert torch.equal(_bits(agg_d[o:o + s]), _bits(agg_h[o:o + s])), f"span {i} step {step}"
         if stats:
             rtol = 1e-2 if dtype == torch.bfloat16 else 1e-6
-            got, want = rows.cpu()[:, :4 + K], rows_h[:, :4 + K]
+            width = 4 if stats == "similarity" else 4 + K
+            got, want = rows.cpu()[:, :width], rows_h[:, :width]
             scale = want[:, 1:3].abs().max(dim=1, keepdim=True).values.clamp_min(1e-300)   # dot may cancel: bound it by the norms
             assert bool(((got - want).abs() <= rtol * want.abs() + 1e-9 * scale).all()), f"stats step {step}"
+            pairs = K * (K - 1) // 2 if stats == "gram" else 0
+            assert torch.count_nonzero(rows[:, width + pairs:]) == 0
+            if pairs:
+                for i, (o, sz, _) in enumerate(spans_h):
+                    G = O.gram([t[o:o + sz] for t in hg_in])
+                    for a in range(K):
+                        for b in range(a + 1, K):
+                            err = abs(float(rows[i, L.stat_pair(K, a, b)]) - float(G[a, b]))
+                            assert err <= (1e-5 if dtype == torch.bfloat16 else 1e-11) * float(torch.sqrt(G[a, a] * G[b, b])) + 1e-300, \
+                                f"pair ({a}, {b}) span {i}"
         if opt:
             if arena is not None:
                 s1_d, s2_d = arena.read(0, arena_first, total), arena.read(1, arena_first, total)
