@@ -424,7 +424,9 @@ __device__ __forceinline__ void span_range(const SP& sp, uint32_t lt0, uint32_t 
     constexpr int UW = SL ? JABAS_UNROLL_STATS : JABAS_UNROLL_PLAIN;
     constexpr int CT = launch_chunk_tiles(K, DT, OPT, SL);
     constexpr int U0 = UW < CT ? UW : CT;     // never more than a chunk holds
-    constexpr int U = K > 8 ? 1 : U0;      // 9..16 gradient streams: one tile's loads fill the registers
+    // 9..16 gradient streams: one tile's loads fill the registers; so do eight fp32 ones beside the 28 fp64 pair
+    // sums of the Gram level (two tiles in flight: 256 registers and one wave per SIMD, 13 % slower)
+    constexpr int U = (K > 8 || (SL == JABAS_STATS_GRAM && DT == JABAS_F32 && K > 7)) ? 1 : U0;
     static_assert((U & (U - 1)) == 0, "the unroll cascade halves U down to 1");
     const uint32_t nb = sp.bound_count;
     ConstBounds bd = nb ? const_bounds(a.bounds + sp.bound_begin) : nullptr;
