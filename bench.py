@@ -711,12 +711,39 @@ def main():
         print(json.dumps(dict(workload=head_cfg.name, launch_streams=args.bucket_launches, steps=args.steps,
                               buckets=engines[0].plan.n_span, **rate(numel * algorithmic_bytes_per_elem(head_cfg), ms))))
         return
-    results = {}
+    results, failures = {}, {}
+
+    def guarded(label, fn):
+        """A leg beside the headline that raises is named in the line ("failures") instead of taking the line with it."""
+        try:
+            return fn()
+        except Exception as exc:
+            failures[label] = f"{type(exc).__name__}: {exc}"
+            print(f"# {label} failed: {failures[label]}", file=sys.stderr, flush=True)
+            try:
+                torch.cuda.synchronize()
+                torch.cuda.empty_cache()
+            except Exception:
+                pass
+            return None
+
     order = [head_cfg] + ([] if args.no_all else [c for c in W.configs() if c.name != head_cfg.name])
-    for cfg in order:
-        r = results[cfg.name] = time_config(cfg, device, args.steps, args.warmup, torch, extras=not args.no_extras)
+    for cfg in list(order):
+        r = None
+        if not args.no_extras:
+            r = guarded(f"{cfg.name} with its extra legs",
+                        lambda: time_config(cfg, device, args.steps, args.warmup, torch, extras=True))
+        if r is None:                               # the step alone; the headline's own failure is the bench's
+            if cfg is head_cfg:
+                r = time_config(cfg, device, args.steps, args.warmup, torch, extras=False)
+            else:
+                r = guarded(cfg.name, lambda: time_config(cfg, device, args.steps, args.warmup, torch, extras=False))
+        if r is None:
+            order.remove(cfg)
+            continue
+        results[cfg.name] = r
         r["hbm_traffic_bytes_per_launch"] = measured_traffic(cfg.name)
-        if args.no_extras:
+        if args.no_extras or "hook_path_per_bucket_ms" not in r:
             print(f"# {cfg.name}: {r['ms_per_step']:.4f} ms/step, {r['GBps']:.0f} GB/s, {r['pct_hbm_peak']:.1f} % of HBM peak",
                   file=sys.stderr, flush=True)
             continue
@@ -734,20 +761,21 @@ def main():
               f"K hook threads: exposed sync {r['hook_path_threads_2_launch_streams'].get('exposed_sync_ms', float('nan')):.4f} ms",
               file=sys.stderr, flush=True)
     if "faster_rcnn_r50_fpn" in results and not args.no_extras:
-        results["faster_rcnn_r50_fpn"]["launch_modes"] = launch_modes(W.config("faster_rcnn_r50_fpn"), device,
-                                                                      args.steps, torch)
-    ref_metrics = None if args.no_all or args.no_extras else reference_profile_metrics(device, args.steps, torch)
-    copy_gbps = copy_rate(device, args.steps, torch)
-    stat_launches = None if args.no_all or args.no_extras else statistics_launches(device, args.steps, torch)
-    gram = None if args.no_all or args.no_extras else gram_launches(device, args.steps, torch)
+        results["faster_rcnn_r50_fpn"]["launch_modes"] = guarded(
+            "launch_modes", lambda: launch_modes(W.config("faster_rcnn_r50_fpn"), device, args.steps, torch))
+    side = not (args.no_all or args.no_extras)
+    ref_metrics = guarded("reference_profile_metrics", lambda: reference_profile_metrics(device, args.steps, torch)) if side else None
+    copy_gbps = guarded("copy_rate", lambda: copy_rate(device, args.steps, torch))
+    stat_launches = guarded("statistics_launches", lambda: statistics_launches(device, args.steps, torch)) if side else None
+    gram = guarded("gram_launches", lambda: gram_launches(device, args.steps, torch)) if side else None
     head = results[head_cfg.name]
     if not args.no_cpu:
         for cfg in order:
             budget = args.cpu_seconds if cfg.name == head_cfg.name else args.cpu_seconds / 3.0
-            results[cfg.name]["cpu_baseline"] = cpu_baseline(cfg, torch, budget)
-            c = results[cfg.name]["cpu_baseline"]
-            print(f"# cpu {cfg.name}: {c['ms_per_step']:.1f} ms/step on {c['cores']} threads ({c['steps']} steps), "
-                  f"{c['one_thread']['ms_per_step']:.1f} ms on one", file=sys.stderr, flush=True)
+            c = results[cfg.name]["cpu_baseline"] = guarded(f"cpu_baseline {cfg.name}", lambda: cpu_baseline(cfg, torch, budget))
+            if c is not None:
+                print(f"# cpu {cfg.name}: {c['ms_per_step']:.1f} ms/step on {c['cores']} threads ({c['steps']} steps), "
+                      f"{c['one_thread']['ms_per_step']:.1f} ms on one", file=sys.stderr, flush=True)
     bytes_per_launch = head["GB_per_step"] * 1e9
     # one fused-kernel launch per step (plus the statistics' finalize launch, about 1 % of it): the mean
     # launch duration is the HIP-event time of the timed region over its steps
@@ -778,6 +806,7 @@ def main():
                           results.get("vit_b16", {}).get("step_with_per_vsw_norms")},
         "statistics_launches": stat_launches,
         "gram_launches": gram,
+        "failures": failures,
     }
     print(json.dumps(out))
 
