@@ -489,6 +489,28 @@ def copy_rate(device, steps, torch):
     return 2 * (1 << 30) / 1e9 / (ms / 1e3)
 
 
+def device_info(device, torch):
+    """What tells one box from another (boxes of the same model differ by several points on mixed read/write
+    streams): the device's name and clocks as torch reports them, and the clocks and partition modes `rocm-smi`
+    shows at this moment (a child process; absent tool or odd output: left out)."""
+    import subprocess
+    p = torch.cuda.get_device_properties(device)
+    info = dict(name=p.name, compute_units=p.multi_processor_count, memory_GiB=round(p.total_memory / 2 ** 30, 1),
+                gcn_arch=getattr(p, "gcnArchName", None), clock_MHz=getattr(p, "clock_rate", 0) / 1e3 or None,
+                memory_clock_MHz=getattr(p, "memory_clock_rate", 0) / 1e3 or None,
+                l2_MiB=round(getattr(p, "L2_cache_size", 0) / 2 ** 20, 1) or None)
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--showmemorypartition", "--showcomputepartition", "--json"],
+                             capture_output=True, text=True, timeout=20)
+        cards = json.loads(out.stdout)
+        card = cards.get("card0") or next(iter(cards.values()))
+        info["rocm_smi"] = {k: v for k, v in card.items()
+                            if any(w in k.lower() for w in ("mclk", "sclk", "fclk", "socclk", "partition"))}
+    except Exception:
+        pass
+    return info
+
+
 def statistics_launches(device, steps, torch):
     """The similarity hook on a step without weight update (the sequential weight-sync mode): aggregate +
     statistics over a 64 Mi-element bucket set, and the statistics alone, K = 4 and 8, fp32 and bf16."""
@@ -806,6 +828,7 @@ def main():
                           results.get("vit_b16", {}).get("step_with_per_vsw_norms")},
         "statistics_launches": stat_launches,
         "gram_launches": gram,
+        "device": guarded("device_info", lambda: device_info(device, torch)),
         "failures": failures,
     }
     print(json.dumps(out))
